@@ -1,0 +1,552 @@
+/*
+ * x17_oracle.c -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+ *
+ * A plain-C, CPU-only restatement of the arithmetic of the reference's quantized
+ * transformer-block forward path.  Only the test-suite, the smoke check and the
+ * CPU-baseline leg of the benchmark may link or load this file; the shipped HIP
+ * path never calls it.
+ *
+ * Every function cites the reference file:line whose op sequence it follows
+ * (paths relative to the reference checkout).  All arithmetic is IEEE binary32
+ * with explicit fmaf() where the reference uses a fused multiply-add; the file
+ * must be compiled with -ffp-contract=off so that nothing else is fused.
+ *
+ * The reference evaluates ex2 / lg2 / rcp / rsqrt / tanh with NVIDIA's
+ * hardware-defined ".approx" instructions (cuda/utils_core.cuh:259-385), which
+ * cannot be reproduced bit-for-bit off that hardware.  This oracle DEFINES them
+ * as the small deterministic f32 algorithms in the "SFU" section below (each
+ * within a few ulp of the exact function; bounds are checked by the CPU tests
+ * against libm in double precision).  The HIP kernels' "strict" build carries
+ * the same algorithms, which is what makes bit-exact GPU-vs-oracle parity
+ * possible for everything downstream of them.
+ *
+ * How each function is pinned (see tests/test_oracle_*.py):
+ *   conversions      exhaustive/bit-level checks + torch.float8_e4m3fn cross-check
+ *   SFU functions    libm (double) with stated ulp bounds, exact special values
+ *   gemm_i32         numpy int64 matmul
+ *   epilogues        closed-form float64 formulas of the reference's torch oracle
+ *   attention/decode dense float64 softmax restatement, closed-form special cases
+ *   rms_norm         textbook float64 RMS norm + the reference's legacy known-answer
+ * The float32 GEMM (gemm_f32_seq) is pinned against float64 matmul to a stated
+ * tolerance only: its summation order is a definition of this file, the
+ * reference's order being fixed by NVIDIA's MMA hardware.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define X17_EXPORT __attribute__((visibility("default")))
+
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* ------------------------------------------------------------------ conversions */
+
+/* cuda/utils_b8.cuh:629-632  f32_to_fixedi8: clamp to +-127, round to nearest even */
+static inline int8_t fixedi8(float v) {
+	float c = fmaxf(-127.0f, fminf(127.0f, v));
+	return (int8_t)(int32_t)rintf(c);
+}
+
+/* cuda/utils_b8.cuh:636-647  f32_to_e4m3: no subnormals, no NaN, max 448,
+ * round half away from zero, sign dropped when flushing to zero */
+static inline uint8_t e4m3_from_f32(float v) {
+	uint32_t tmp = f2u(v);
+	uint32_t sign = (tmp >> 24) & 0x80u;
+	uint32_t rest = tmp & 0x7FFFFFFFu;
+	uint32_t mn = (120u << 23) + (0xfu << 19);
+	uint32_t mx = (135u << 23) + (0xcu << 19);
+	uint32_t rounded = (rest + ((1u << 19) - (120u << 23))) >> 20;
+	uint32_t clamped = rest > mx ? 0x7eu : rounded;
+	return (uint8_t)(rest < mn ? 0u : (sign | clamped));
+}
+
+/* cuda/utils_b8.cuh:652-657  e4m3_to_bf16 (widened to f32; bf16 holds it exactly) */
+static inline float e4m3_to_f32(uint8_t c) {
+	uint32_t sign = ((uint32_t)c & 0x80u) << 24;
+	uint32_t rest = ((uint32_t)c & 0x7Fu) << 20;
+	if (rest == 0) return 0.0f;
+	return u2f((sign | rest) + (120u << 23));
+}
+
+static inline float bf16_to_f32(uint16_t b) { return u2f((uint32_t)b << 16); }
+
+X17_EXPORT void x17o_f32_to_fixedi8(const float *in, int8_t *out, size_t n) {
+	for (size_t i = 0; i < n; ++i) out[i] = fixedi8(in[i]);
+}
+X17_EXPORT void x17o_f32_to_e4m3(const float *in, uint8_t *out, size_t n) {
+	for (size_t i = 0; i < n; ++i) out[i] = e4m3_from_f32(in[i]);
+}
+X17_EXPORT void x17o_e4m3_to_f32(const uint8_t *in, float *out, size_t n) {
+	for (size_t i = 0; i < n; ++i) out[i] = e4m3_to_f32(in[i]);
+}
+
+/* ------------------------------------------------------------------ SFU definitions
+ * Stand-ins for ex2/lg2/rcp/rsqrt/tanh .approx (cuda/utils_core.cuh:259-385).
+ * Only fmaf, +, -, *, rintf, comparisons and integer bit operations are used, so a
+ * second implementation on any IEEE-754 machine gives identical bits. */
+
+/* 2^x.  Results below 2^-125 are flushed to zero (the reference's ops are .ftz). */
+static inline float sfu_ex2(float x) {
+	if (!(x >= -125.0f)) return 0.0f;
+	x = fminf(x, 126.0f);
+	float n = rintf(x);
+	float f = x - n;                       /* exact, |f| <= 0.5 */
+	float p = 0.00015453163359779865f;
+	p = fmaf(p, f, 0.0013390863314270973f);
+	p = fmaf(p, f, 0.009618083015084267f);
+	p = fmaf(p, f, 0.055503569543361664f);
+	p = fmaf(p, f, 0.24022650718688965f);
+	p = fmaf(p, f, 0.6931471824645996f);
+	p = fmaf(p, f, 1.0f);                  /* 2^f in [0.7071, 1.4143] */
+	int32_t ni = (int32_t)n;
+	return u2f(f2u(p) + ((uint32_t)ni << 23));
+}
+
+/* log2(x) for positive, normal, finite x. */
+static inline float sfu_lg2(float x) {
+	uint32_t b = f2u(x);
+	int32_t e = (int32_t)(b >> 23) - 127;
+	float m = u2f((b & 0x007FFFFFu) | 0x3F800000u);   /* [1,2) */
+	if (m > 1.41421354f) { m = m * 0.5f; e += 1; }     /* [0.7071, 1.4143) */
+	float t = m - 1.0f;                                /* exact */
+	float q = -0.10749789327383041f;
+	q = fmaf(q, t, 0.18476033210754395f);
+	q = fmaf(q, t, -0.19138838350772858f);
+	q = fmaf(q, t, 0.20485764741897583f);
+	q = fmaf(q, t, -0.23960812389850616f);
+	q = fmaf(q, t, 0.28855255246162415f);
+	q = fmaf(q, t, -0.36069655418395996f);
+	q = fmaf(q, t, 0.48089852929115295f);
+	q = fmaf(q, t, -0.7213473320007324f);
+	q = fmaf(q, t, 1.4426950216293335f);
+	return fmaf(t, q, (float)e);
+}
+
+/* 1/x for positive, normal, finite x: bit-trick seed + 4 Newton steps. */
+static inline float sfu_rcp(float x) {
+	float r = u2f(0x7EF311C7u - f2u(x));
+	for (int i = 0; i < 4; ++i) {
+		float e = fmaf(-x, r, 1.0f);
+		r = fmaf(r, e, r);
+	}
+	return r;
+}
+
+/* 1/sqrt(x) for positive, normal, finite x: bit-trick seed + 4 Newton steps. */
+static inline float sfu_rsq(float x) {
+	float y = u2f(0x5F3759DFu - (f2u(x) >> 1));
+	float hx = 0.5f * x;
+	for (int i = 0; i < 4; ++i) {
+		float t = hx * y;
+		t = fmaf(-t, y, 1.5f);
+		y = y * t;
+	}
+	return y;
+}
+
+/* tanh(x) = 1 - 2/(1 + e^{2|x|}), sign restored; |x| capped at 10 (tanh == 1.0f there). */
+static inline float sfu_tanh(float x) {
+	float a = fminf(fabsf(x), 10.0f);
+	float e = sfu_ex2(a * 2.8853900432586670f);        /* 2*log2(e) */
+	float r = sfu_rcp(e + 1.0f);
+	float t = fmaf(-2.0f, r, 1.0f);
+	return copysignf(t, x);
+}
+
+X17_EXPORT void x17o_sfu(int which, const float *in, float *out, size_t n) {
+	for (size_t i = 0; i < n; ++i) {
+		float x = in[i];
+		switch (which) {
+			case 0: out[i] = sfu_ex2(x); break;
+			case 1: out[i] = sfu_lg2(x); break;
+			case 2: out[i] = sfu_rcp(x); break;
+			case 3: out[i] = sfu_rsq(x); break;
+			default: out[i] = sfu_tanh(x); break;
+		}
+	}
+}
+
+/* ------------------------------------------------------------------ compile-time constant math
+ * The reference derives its epilogue constants in double precision with its own
+ * bisection square root (cuda/utils_core.cuh:151-178); a 1-ulp difference in the
+ * double could flip the f32 rounding, so the same routine is restated here. */
+static double constexpr_sqrt(double x) {
+	if (x < 0.0 || x != x) return NAN;
+	if (x == 0.0) return 0.0;
+	if (isinf(x)) return x;
+	double above = x > 1.0 ? x : 1.0;
+	double below = 0.0;
+	int stop = 0;
+	while (!stop) {
+		double v = (0.5 * above) + (0.5 * below);
+		double t = x / v;
+		double new_above = t <= v ? v : above;
+		double new_below = t >= v ? v : below;
+		stop = (new_above == above) && (new_below == below);
+		above = new_above;
+		below = new_below;
+	}
+	double above_err = (above * above) - x;
+	double below_err = x - (below * below);
+	return above_err > below_err ? below : above;
+}
+
+/* cuda/utils_core.cuh:180-210 */
+static double constexpr_inv_sqrt(double x) {
+	if (x < 0.0 || x != x) return NAN;
+	if (x == 0.0) return INFINITY;
+	if (isinf(x)) return 0.0;
+	double above = 2.0 / constexpr_sqrt(x);
+	double below = 0.0;
+	int stop = 0;
+	while (!stop) {
+		double v = (0.5 * above) + (0.5 * below);
+		double t = (x * v) * v;
+		double new_above = t >= 1.0 ? v : above;
+		double new_below = t <= 1.0 ? v : below;
+		stop = (new_above == above) && (new_below == below);
+		above = new_above;
+		below = new_below;
+	}
+	double above_err = ((x * above) * above) - 1.0;
+	double below_err = 1.0 - ((x * below) * below);
+	return above_err > below_err ? below : above;
+}
+
+X17_EXPORT double x17o_constexpr_sqrt(double x) { return constexpr_sqrt(x); }
+X17_EXPORT double x17o_constexpr_inv_sqrt(double x) { return constexpr_inv_sqrt(x); }
+
+#define X17_INV_PI 0.318309886183790671537767526745028724
+#define X17_LN2    0.693147180559945309417232121458176568
+
+/* ------------------------------------------------------------------ GEMM cores */
+
+/* cuda/gemm_b8.cuh:666-754 -- acc[m][n] = sum_k A[m][k]*B[n][k], exact in int32.
+ * A is [M,K] row-major i8, B is [N,K] row-major i8 ("trans" weights). */
+X17_EXPORT void x17o_gemm_i32(const int8_t *A, const int8_t *B, int32_t *acc,
+                              size_t M, size_t N, size_t K) {
+	#pragma omp parallel for schedule(static)
+	for (size_t m = 0; m < M; ++m) {
+		const int8_t *a = A + m * K;
+		for (size_t n = 0; n < N; ++n) {
+			const int8_t *b = B + n * K;
+			int32_t s = 0;
+			for (size_t k = 0; k < K; ++k) s += (int32_t)a[k] * (int32_t)b[k];
+			acc[m * N + n] = s;
+		}
+	}
+}
+
+/* cuda/gemm_b16.cuh:436-567 -- operands that are exactly representable in bf16
+ * (e4m3 or i8 codes), products exact in f32, f32 accumulation.  The order used here
+ * is k ascending, one f32 add per product.  a_kind/b_kind: 0 = i8 codes, 1 = e4m3. */
+X17_EXPORT void x17o_gemm_f32_seq(const uint8_t *A, int a_kind, const uint8_t *B, int b_kind,
+                                  float *acc, size_t M, size_t N, size_t K) {
+	float *Af = (float *)malloc(M * K * sizeof(float));
+	float *Bf = (float *)malloc(N * K * sizeof(float));
+	for (size_t i = 0; i < M * K; ++i) Af[i] = a_kind ? e4m3_to_f32(A[i]) : (float)(int8_t)A[i];
+	for (size_t i = 0; i < N * K; ++i) Bf[i] = b_kind ? e4m3_to_f32(B[i]) : (float)(int8_t)B[i];
+	#pragma omp parallel for schedule(static)
+	for (size_t m = 0; m < M; ++m) {
+		for (size_t n = 0; n < N; ++n) {
+			float s = 0.0f;
+			for (size_t k = 0; k < K; ++k) s = s + Af[m * K + k] * Bf[n * K + k];
+			acc[m * N + n] = s;
+		}
+	}
+	free(Af);
+	free(Bf);
+}
+
+/* ------------------------------------------------------------------ epilogues
+ * `acc` is [M, N_raw] row-major; acc_is_f32 selects int32 or float32 accumulators.
+ * store: 0 = FixedI8 (I8Store, cuda/gemm_b8.cuh:265-276), 1 = E4m3 (E4m3Store, :278-289). */
+
+static inline float acc_at(const void *acc, int is_f32, size_t idx) {
+	return is_f32 ? ((const float *)acc)[idx] : (float)((const int32_t *)acc)[idx];
+}
+static inline uint8_t store_conv(float v, int store) {
+	return store ? e4m3_from_f32(v) : (uint8_t)fixedi8(v);
+}
+
+/* ScaledMatrixWriter, cuda/gemm_b8.cuh:291-339 + b32::cast<SCALE> cuda/utils_b32.cuh:215-222.
+ * SCALE = inp*out in double (templates/basic_gemm/common.cuh:66-74), rounded once to f32. */
+X17_EXPORT void x17o_epilogue_scale(const void *acc, int acc_is_f32, uint8_t *C,
+                                    size_t M, size_t N, double inp_scale, double out_scale,
+                                    int store) {
+	float s = (float)(inp_scale * out_scale);
+	#pragma omp parallel for schedule(static)
+	for (size_t i = 0; i < M * N; ++i) C[i] = store_conv(acc_at(acc, acc_is_f32, i) * s, store);
+}
+
+/* GeGluMatrixWriter cuda/gemm_b8.cuh:341-441 with math::fast::gelu cuda/utils_core.cuh:426-448.
+ * Even raw columns are the gate, odd columns the linear part. */
+X17_EXPORT void x17o_epilogue_geglu(const void *acc, int acc_is_f32, uint8_t *C,
+                                    size_t M, size_t N_raw, double I, double O, int store) {
+	double inp_scale_2 = I * I;
+	double out_scale_2 = O * O;
+	double gelu_inp2 = inp_scale_2;
+	double gelu_out2 = inp_scale_2 * out_scale_2;
+	double k = constexpr_sqrt(gelu_inp2);
+	double k2 = gelu_inp2;
+	double ck = constexpr_sqrt(gelu_inp2 * 2.0 * X17_INV_PI);
+	double ck3 = 0.044715 * ck * k2;
+	double y_scale = 0.5 * constexpr_sqrt(gelu_out2 * 1.0) * k;
+	float fck = (float)ck, fck3 = (float)ck3, fy = (float)y_scale;
+	size_t N = N_raw / 2;
+	#pragma omp parallel for schedule(static)
+	for (size_t m = 0; m < M; ++m) {
+		for (size_t j = 0; j < N; ++j) {
+			float x = acc_at(acc, acc_is_f32, m * N_raw + 2 * j);
+			float lin = acc_at(acc, acc_is_f32, m * N_raw + 2 * j + 1);
+			float x2 = x * x;
+			float s = fmaf(fck3 * x, x2, fck * x);
+			float t = sfu_tanh(s);
+			float gate = fmaf(fy * x, t, fy * x);
+			C[m * N + j] = store_conv(gate * lin, store);
+		}
+	}
+}
+
+/* ResidualMatrixWriter cuda/gemm_b8.cuh:443-622 (residual_gate :484-505),
+ * sigmoid_base4 cuda/utils_core.cuh:397-405, imprecise_softplus_base4 :468-483. */
+X17_EXPORT void x17o_epilogue_residual(const void *acc, int acc_is_f32, const int8_t *R,
+                                       uint8_t *C, size_t M, size_t N_raw,
+                                       double I, double O, int store) {
+	/* sigmoid_base4<-I, 1/8> */
+	float sg_half = (float)(0.5 * (1.0 / 8.0));
+	float sg_in = (float)(X17_LN2 * (-I));
+	/* imprecise_softplus_base4<I, I*O> */
+	double sp_inp = I, sp_out = I * O;
+	float sp_inp_scale = (float)(sp_inp * 2.0);
+	float sp_out_scale = (float)(sp_out / 2.0);
+	float sp_line = (float)(sp_inp * sp_out);
+	size_t N = N_raw / 2;
+	#pragma omp parallel for schedule(static)
+	for (size_t m = 0; m < M; ++m) {
+		for (size_t j = 0; j < N; ++j) {
+			float g = acc_at(acc, acc_is_f32, m * N_raw + 2 * j);
+			float v = acc_at(acc, acc_is_f32, m * N_raw + 2 * j + 1);
+			float old_w = fmaf(sg_half, sfu_tanh(sg_in * g), sg_half);
+			float line = fmaxf(0.0f, g);
+			if (sp_line != 1.0f) line = line * sp_line;
+			float new_w = fmaf(sfu_lg2(1.0f + sfu_ex2(-fabsf(g * sp_inp_scale))), sp_out_scale, line);
+			float old_val = (float)R[m * N + j];
+			float val = fmaf(new_w, v, old_w * old_val);
+			C[m * N + j] = store_conv(val, store);
+		}
+	}
+}
+
+/* L2NormMatrixWriter cuda/gemm_b8.cuh:861-949 with kv_helpers::l2_norm :767-830 and
+ * raw_output :839-858.  Columns are grouped per head as [K (hd) | V (hd)].  The sum of
+ * squares of the K half is kept in four partial sums: partial q owns the columns with
+ * (c % 8) / 2 == q, visited in increasing column order, and the total is
+ * (s0 + s1) + (s2 + s3)  (:789-806).  head_scale = out*sqrt(hd) and sep_scale = inp*out
+ * are formed in double by the caller side (src/device/cuda/gemm.rs:146,152). */
+X17_EXPORT void x17o_epilogue_l2norm(const int32_t *acc, int8_t *C, float *rrms,
+                                     size_t M, size_t N_raw, size_t hd,
+                                     double eps, double head_scale, double sep_scale) {
+	size_t heads = N_raw / (2 * hd);
+	float feps = (float)eps, fhs = (float)head_scale, fss = (float)sep_scale;
+	#pragma omp parallel for schedule(static)
+	for (size_t m = 0; m < M; ++m) {
+		for (size_t h = 0; h < heads; ++h) {
+			const int32_t *a = acc + m * N_raw + h * 2 * hd;
+			int8_t *c = C + m * N_raw + h * 2 * hd;
+			float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+			for (size_t d = 0; d < hd; ++d) {
+				float x = (float)a[d];
+				size_t q = (d % 8) / 2;
+				s[q] = fmaf(x, x, s[q]);
+			}
+			float S = (s[0] + s[1]) + (s[2] + s[3]);
+			float scale = sfu_rsq(S + feps) * fhs;
+			for (size_t d = 0; d < hd; ++d) c[d] = fixedi8((float)a[d] * scale);
+			for (size_t d = 0; d < hd; ++d) c[hd + d] = fixedi8((float)a[hd + d] * fss);
+			rrms[m * heads + h] = scale;
+		}
+	}
+}
+
+/* ------------------------------------------------------------------ attention
+ * AttnForward::run cuda/attn_fwd_i8.cuh:368-619 restated per (head, query):
+ *   window rounded up to a multiple of 16 (:409-412); query i sees keys
+ *   [max(0, i-W'), i-1] plus the sink (masks :79-134, :540-567);
+ *   n = min(W', i) + 4 and temperature = f32(hd^-1/2 / 64) * lg2(n) * head_temp (:444-450, :497);
+ *   running max seeded with the sink score, partial sums seeded with 4 x 63.75,
+ *   O seeded with 255 * sink_v (:489-517);
+ *   per 16-key tile: max update + rescale (:233-256), p = ex2(s - m) * 255 (:265-277),
+ *   four per-lane partial sums over keys 4q..4q+3 of the tile (:279-290),
+ *   P = rne(p) as u8 (cuda/utils.cuh:86-95), O += f32(int32 P.V) (:588-605);
+ *   end: sum = (s0+s1)+(s2+s3), L = lg2(sum) + m, out = fixedi8(O * rcp(sum)) (:293-351).
+ * Tiles that are fully masked for a query leave its state bit-for-bit unchanged, so
+ * only tiles that hold a visible key are visited.
+ *
+ * Layouts: q [T, H*hd], kv [T, H*2*hd] (per head K then V), sinks [H, hd],
+ * out [T, H*hd], L [H, T] (may be NULL).  `pos0` is the absolute position of row 0 of
+ * q relative to row 0 of kv (0 for prefill; used by the decode entry below).
+ * `fast_exp` != 0 replaces sfu_ex2 by exp2f so that the tests can bound how far a
+ * hardware-exponent build may drift from the strict definition. */
+static void attn_rows(size_t n_q, size_t pos0, size_t H, size_t hd,
+                      const int8_t *q, size_t q_stride,
+                      const int8_t *kv, size_t kv_stride,
+                      const int8_t *sink_k, const int8_t *sink_v, const float *head_temp,
+                      int8_t *out, size_t o_stride, float *L, size_t l_stride,
+                      size_t window, int fast_exp) {
+	size_t Wr = window == 0 ? (size_t)-1 : ((window - 1) / 16 + 1) * 16;
+	float base = (float)(constexpr_inv_sqrt((double)hd) / 64.0);
+	#pragma omp parallel for collapse(2) schedule(dynamic, 8)
+	for (size_t h = 0; h < H; ++h) {
+		for (size_t r = 0; r < n_q; ++r) {
+			size_t i = pos0 + r;
+			const int8_t *qi = q + r * q_stride + h * hd;
+			const int8_t *sk = sink_k + h * hd;
+			const int8_t *sv = sink_v + h * hd;
+			size_t visible = i < Wr ? i : Wr;
+			uint32_t n = (uint32_t)visible + 4u;
+			float temp = base * sfu_lg2((float)n);
+			temp = temp * head_temp[h];
+			int32_t sdot = 0;
+			for (size_t d = 0; d < hd; ++d) sdot += (int32_t)qi[d] * (int32_t)sk[d];
+			float m = (float)sdot * temp;
+			float sum[4] = {63.75f, 63.75f, 63.75f, 63.75f};
+			float O[512];
+			for (size_t d = 0; d < hd; ++d) O[d] = (float)((int32_t)sv[d] * 255);
+			size_t j_lo = i - visible;
+			for (size_t t = j_lo / 16; t * 16 < i; ++t) {
+				float s[16];
+				float tmax = -INFINITY;
+				for (size_t k = 0; k < 16; ++k) {
+					size_t j = t * 16 + k;
+					if (j >= i || j < j_lo) { s[k] = -INFINITY; continue; }
+					const int8_t *kj = kv + j * kv_stride + h * 2 * hd;
+					int32_t dot = 0;
+					for (size_t d = 0; d < hd; ++d) dot += (int32_t)qi[d] * (int32_t)kj[d];
+					s[k] = (float)dot * temp;
+					tmax = fmaxf(tmax, s[k]);
+				}
+				float resc = 1.0f;
+				if (tmax > m) {
+					resc = fast_exp ? exp2f(m - tmax) : sfu_ex2(m - tmax);
+					for (size_t d = 0; d < hd; ++d) O[d] = O[d] * resc;
+					m = tmax;
+				}
+				float p[16];
+				int32_t P[16];
+				for (size_t k = 0; k < 16; ++k) {
+					float e = fast_exp ? exp2f(s[k] - m) : sfu_ex2(s[k] - m);
+					p[k] = e * 255.0f;
+					P[k] = (int32_t)rintf(p[k]);
+				}
+				for (size_t qq = 0; qq < 4; ++qq) {
+					float add = (p[4 * qq] + p[4 * qq + 1]) + (p[4 * qq + 2] + p[4 * qq + 3]);
+					sum[qq] = fmaf(sum[qq], resc, add);
+				}
+				int32_t pv[512];
+				memset(pv, 0, hd * sizeof(int32_t));
+				for (size_t k = 0; k < 16; ++k) {
+					if (P[k] == 0) continue;
+					size_t j = t * 16 + k;
+					const int8_t *vj = kv + j * kv_stride + h * 2 * hd + hd;
+					for (size_t d = 0; d < hd; ++d) pv[d] += P[k] * (int32_t)vj[d];
+				}
+				for (size_t d = 0; d < hd; ++d) O[d] = O[d] + (float)pv[d];
+			}
+			float S = (sum[0] + sum[1]) + (sum[2] + sum[3]);
+			if (L) L[h * l_stride + r] = sfu_lg2(S) + m;
+			float inv = sfu_rcp(S);
+			int8_t *o = out + r * o_stride + h * hd;
+			for (size_t d = 0; d < hd; ++d) o[d] = fixedi8(O[d] * inv);
+		}
+	}
+}
+
+X17_EXPORT int x17o_attn_fwd_i8(size_t T, size_t H, size_t hd,
+                                const int8_t *q, const int8_t *kv,
+                                const int8_t *sink_k, const int8_t *sink_v,
+                                const float *head_temp, int8_t *out, float *L,
+                                size_t window, int fast_exp) {
+	if (hd > 512) return -1;
+	attn_rows(T, 0, H, hd, q, H * hd, kv, 2 * H * hd, sink_k, sink_v, head_temp,
+	          out, H * hd, L, T, window, fast_exp);
+	return 0;
+}
+
+/* Single-token decode.  The reference has no int8 decode kernel (TODO.md:10-12 defers
+ * ragged tails to "the incremental kernel"; attn_incremental.cu is its bf16 precedent for
+ * queries appended to a longer KV, :362-367, :440-447).  It is defined here as the prefill
+ * recurrence above for ONE query at absolute position cache_len, against cache rows
+ * [0, cache_len).  cache is [S][cap][H*2*hd], q/out are [S][H*hd], L is [S][H] or NULL. */
+X17_EXPORT int x17o_attn_decode_i8(size_t S, size_t cap, const uint32_t *cache_len,
+                                   size_t H, size_t hd,
+                                   const int8_t *q, const int8_t *cache,
+                                   const int8_t *sink_k, const int8_t *sink_v,
+                                   const float *head_temp, int8_t *out, float *L,
+                                   size_t window, int fast_exp) {
+	if (hd > 512) return -1;
+	for (size_t s = 0; s < S; ++s) {
+		if (cache_len[s] > cap) return -2;
+		attn_rows(1, cache_len[s], H, hd, q + s * H * hd, H * hd,
+		          cache + s * cap * 2 * H * hd, 2 * H * hd,
+		          sink_k, sink_v, head_temp,
+		          out + s * H * hd, H * hd, L ? L + s * H : NULL, 1, window, fast_exp);
+	}
+	return 0;
+}
+
+/* ------------------------------------------------------------------ rms_norm
+ * rms_norm.cu:55-113.  One 32-lane group per row; per 512-column step, lane l runs an fma
+ * chain from zero over its 16 consecutive values and adds the chain to its running sum
+ * (:39-46, :87-93); the lanes are combined with an xor butterfly 16,8,4,2,1 (:32-37);
+ * rrms = rsqrt(sum * f32(1/D) + f32(eps)) (:96); out = fixedi8((x * rrms) * 8) (:51).
+ * in_kind: 1 = e4m3 bytes (the reference's input), 2 = bf16 (same kernel fed bf16). */
+X17_EXPORT int x17o_rms_norm(const void *inp, int in_kind, int8_t *out,
+                             size_t T, size_t D, double eps) {
+	if (D % 512 != 0) return -1;
+	float inv_d = (float)(1.0 / (double)D);
+	float feps = (float)eps;
+	#pragma omp parallel for schedule(static)
+	for (size_t r = 0; r < T; ++r) {
+		float lane[32];
+		for (int l = 0; l < 32; ++l) lane[l] = 0.0f;
+		for (size_t step = 0; step < D / 512; ++step) {
+			for (int l = 0; l < 32; ++l) {
+				float b = 0.0f;
+				for (size_t c = 0; c < 16; ++c) {
+					size_t col = 512 * step + 16 * (size_t)l + c;
+					float x = in_kind == 1 ? e4m3_to_f32(((const uint8_t *)inp)[r * D + col])
+					                       : bf16_to_f32(((const uint16_t *)inp)[r * D + col]);
+					b = fmaf(x, x, b);
+				}
+				lane[l] = lane[l] + b;
+			}
+		}
+		for (int mask = 16; mask > 0; mask >>= 1) {
+			float nxt[32];
+			for (int l = 0; l < 32; ++l) nxt[l] = lane[l] + lane[l ^ mask];
+			memcpy(lane, nxt, sizeof(lane));
+		}
+		float rr = sfu_rsq(lane[0] * inv_d + feps);
+		for (size_t c = 0; c < D; ++c) {
+			float x = in_kind == 1 ? e4m3_to_f32(((const uint8_t *)inp)[r * D + c])
+			                       : bf16_to_f32(((const uint16_t *)inp)[r * D + c]);
+			out[r * D + c] = fixedi8(x * rr * 8.0f);
+		}
+	}
+	return 0;
+}
+
+X17_EXPORT int x17o_num_threads(void) {
+#ifdef _OPENMP
+	return omp_get_max_threads();
+#else
+	return 1;
+#endif
+}
