@@ -1,0 +1,126 @@
+/*
+ * x17ai_host.h -- flat C ABI of the host-side operator layer (libx17ai_host.so).
+ *
+ * The reference's operator layer is Rust (src/device/cuda/{gemm,attn,tensor_check,
+ * kernel_build}.rs, src/tensor.rs, src/device/cuda.rs); its C++ mirror lives in
+ * x17ai_amd/csrc/host/.  This header exposes that mirror to non-C++ callers (the Python
+ * tests and bench drive it through ctypes).  Every function here ends in the C-ABI device
+ * shim of include/x17ai_hip_shim.h; nothing in it computes on the CPU.
+ *
+ * Conventions: functions return 0 on success and non-zero on failure; after a failure
+ * x17h_last_error() returns the message (thread-local, valid until the next call).
+ * Handles are opaque and must be released with the matching *_free.
+ */
+#ifndef X17AI_HOST_H
+#define X17AI_HOST_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct X17hDevice X17hDevice;       /* mirrors CudaDevice, src/device/cuda.rs:25-66 */
+typedef struct X17hTensor X17hTensor;       /* mirrors Tensor, src/tensor.rs:23-256 */
+typedef struct X17hTimer X17hTimer;         /* mirrors CudaTimer, src/device/cuda.rs:79-101 */
+typedef struct X17hGemmKernel X17hGemmKernel;       /* mirrors GemmKernel<E>, src/device/cuda/gemm.rs:350-449 */
+typedef struct X17hAttnKernel X17hAttnKernel;       /* mirrors AttnKernel, src/device/cuda/attn.rs:156-240 */
+typedef struct X17hRmsNormKernel X17hRmsNormKernel; /* rms_norm.cu:55-113 as a kernel object */
+typedef struct X17hDecodeKernel X17hDecodeKernel;   /* single-token decode; no reference counterpart */
+
+/* DType, src/dtype.rs:1-15 */
+enum { X17H_E4M3 = 0, X17H_INT8 = 1, X17H_BF16 = 2, X17H_F32 = 3 };
+/* epilogues, src/device/cuda/gemm.rs:322-349 */
+enum { X17H_EPI_SCALE = 0, X17H_EPI_GEGLU = 1, X17H_EPI_RESIDUAL = 2, X17H_EPI_RMSNORM = 3 };
+
+char const *x17h_last_error(void);
+/* text of the warnings/errors collected by the last *_new call (kernel generation diagnostics) */
+char const *x17h_last_diagnostics(void);
+
+/* CudaDevice::new, src/device/cuda.rs:31-38 */
+int x17h_device_new(size_t device_id, X17hDevice **out);
+void x17h_device_free(X17hDevice *dev);
+int x17h_device_synchronize(X17hDevice *dev);
+char const *x17h_device_name(X17hDevice *dev);
+
+/* Tensor::new_empty + Device::upload_data / download_data, src/tensor.rs:36-112.
+ * dev == NULL places the tensor on the CPU device (host memory), as Tensor::to_cpu does. */
+int x17h_tensor_new_empty(X17hDevice *dev, size_t const *shape, size_t ndim, int dtype, X17hTensor **out);
+void x17h_tensor_free(X17hTensor *t);
+int x17h_tensor_upload(X17hTensor *t, void const *src, size_t bytes);      /* async on the device stream */
+int x17h_tensor_download(X17hTensor *t, void *dst, size_t bytes);          /* async; synchronize before reading */
+void *x17h_tensor_device_ptr(X17hTensor *t);
+size_t x17h_tensor_bytes(X17hTensor *t);
+int x17h_tensor_reshape(X17hTensor *t, size_t const *shape, size_t ndim);  /* Tensor::reshape, in place */
+
+/* CudaTimer, src/device/cuda.rs:79-101 (events on the device's stream) */
+int x17h_timer_new(X17hDevice *dev, X17hTimer **out);
+void x17h_timer_free(X17hTimer *t);
+int x17h_timer_start(X17hTimer *t);
+int x17h_timer_stop(X17hTimer *t);
+int x17h_timer_elapsed_seconds(X17hTimer *t, double *seconds);
+
+/* GemmConfig + epilogue configs, src/device/cuda/gemm.rs:28-76 */
+typedef struct X17hGemmConfig {
+	int a_dtype; size_t a_cols; size_t a_rows; /* 0 = runtime */ int a_trans;
+	int b_dtype; size_t b_cols; size_t b_rows; /* 0 = runtime */ int b_trans;
+	int c_dtype;
+	int epilogue;            /* X17H_EPI_* */
+	double inp_scale;
+	double out_scale;
+	double eps;              /* RMSNorm only */
+	size_t head_dim;         /* RMSNorm only */
+	size_t sep_dim;          /* RMSNorm only */
+	int strict_math;         /* 1: deterministic transcendentals (parity build), 0: hardware ones */
+} X17hGemmConfig;
+
+/* GemmKernel::<E>::new, gemm.rs:368-437.  dev == NULL: generate and compile only. */
+int x17h_gemm_kernel_new(X17hDevice *dev, char const *kernel_name, X17hGemmConfig const *config, X17hGemmKernel **out);
+void x17h_gemm_kernel_free(X17hGemmKernel *k);
+/* GemmKernel::launch, gemm.rs:439-443; extra = rrms (RMSNorm) / residual (Residual) / NULL */
+int x17h_gemm_kernel_launch(X17hGemmKernel *k, X17hTensor *a, X17hTensor *b, X17hTensor *c, X17hTensor *extra);
+/* GemmKernel::n_ops, gemm.rs:445-449 */
+double x17h_gemm_kernel_n_ops(X17hGemmKernel *k, X17hTensor *a, X17hTensor *b);
+/* launch geometry read back from meta.json: THREADS_PER_BLOCK, SMEM_BYTES, M_PER_BLOCK, N_PER_BLOCK */
+int x17h_gemm_kernel_metadata(X17hGemmKernel *k, size_t out[4]);
+/* resources of the loaded kernel: x17ai_hip_read_kernel_attrs (9 x int32) */
+int x17h_gemm_kernel_attrs(X17hGemmKernel *k, int32_t out[9]);
+
+/* AttnKernelConfig, attn.rs:45-152 */
+typedef struct X17hAttnConfig {
+	int dtype; size_t n_heads; size_t head_dim; size_t q_stride; size_t kv_stride; size_t o_stride;
+	int strict_math;
+} X17hAttnConfig;
+/* AttnKernel::new, attn.rs:170-232 */
+int x17h_attn_kernel_new(X17hDevice *dev, char const *kernel_name, X17hAttnConfig const *config, X17hAttnKernel **out);
+void x17h_attn_kernel_free(X17hAttnKernel *k);
+/* AttnKernel::launch, attn.rs:234-236 / 353-447.  l may be NULL.  batch > 1 is an extension:
+ * the rows of q/kv/out are `batch` independent sequences of equal length. */
+int x17h_attn_kernel_launch(X17hAttnKernel *k, X17hTensor *q, X17hTensor *kv, X17hTensor *sink_k,
+                            X17hTensor *sink_v, X17hTensor *attn_temperature, X17hTensor *out,
+                            X17hTensor *l, size_t window_size, size_t batch);
+/* AttnKernelConfig::n_ops, attn.rs:72-84 */
+double x17h_attn_kernel_n_ops(X17hAttnKernel *k, size_t seq_len, size_t window_size);
+int x17h_attn_kernel_metadata(X17hAttnKernel *k, size_t out[3]);
+int x17h_attn_kernel_attrs(X17hAttnKernel *k, int32_t out[9]);
+
+/* rms_norm.cu:55-113: out[T, D] int8 = fixedi8(x * rsqrt(mean(x^2) + eps) * 8); in_dtype e4m3 or bf16 */
+int x17h_rms_norm_kernel_new(X17hDevice *dev, char const *kernel_name, int in_dtype, size_t model_dim,
+                             double eps, X17hRmsNormKernel **out);
+void x17h_rms_norm_kernel_free(X17hRmsNormKernel *k);
+int x17h_rms_norm_kernel_launch(X17hRmsNormKernel *k, X17hTensor *inp, X17hTensor *out);
+
+/* Single-token decode against an int8 KV cache [S, capacity, 2*H*hd]: the attention recurrence
+ * of attn_fwd_i8 for one query per sequence at position cache_len[s]. */
+int x17h_decode_kernel_new(X17hDevice *dev, char const *kernel_name, size_t n_heads, size_t head_dim,
+                           size_t cache_capacity, int strict_math, X17hDecodeKernel **out);
+void x17h_decode_kernel_free(X17hDecodeKernel *k);
+int x17h_decode_kernel_launch(X17hDecodeKernel *k, X17hTensor *q, X17hTensor *cache, X17hTensor *cache_len,
+                              X17hTensor *sink_k, X17hTensor *sink_v, X17hTensor *attn_temperature,
+                              X17hTensor *out, X17hTensor *l, size_t window_size);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* X17AI_HOST_H */

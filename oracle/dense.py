@@ -108,33 +108,39 @@ def ssmax_n(seq_len: int, window: int) -> np.ndarray:
 
 
 def attn_one_head(q, k, v, sink_k, sink_v, temperature_scale: float, window: int,
-                  prob_steps: float = 8.0):
+                  prob_steps: float = 8.0, row_block: int = 2048):
 	"""new_block.py:183-232.  q, k, v are real values on the FixedI8 grid, [T, hd].
 	prob_steps = 8 reproduces the reference oracle (probabilities rounded to 1/8 steps,
 	:225); prob_steps = 255 models the CUDA kernel's u8 probabilities instead.
+	The dense [T, T+1] matrices are formed `row_block` query rows at a time (and only up to
+	the last causally visible column), which changes nothing in the arithmetic of a row.
 	Returns (o [T, hd], l [T]) with l in the kernel's convention log2(sum * 255) + max*log2e."""
 	t, hd = q.shape
 	k = np.concatenate((sink_k[None, :], k), axis=0)
 	v = np.concatenate((sink_v[None, :], v), axis=0)
-	s = q @ k.T
 	temperature = math.sqrt(1.0 / hd) * np.log(ssmax_n(t, window)) * temperature_scale
-	rows = np.arange(t)[:, None]
-	cols = np.arange(t)[None, :]
-	real_mask = cols >= rows
-	if window > 0:
-		real_mask |= cols < rows - window
-	mask = np.zeros((t, t + 1), dtype=bool)
-	mask[:, 1:] = real_mask
-	s = np.where(mask, -np.inf, s)
-	s = s * temperature
-	mx = s.max(axis=1, keepdims=True)
-	p = np.exp(s - mx)
-	total = p.sum(axis=1, keepdims=True)
 	log2e = 1.0 / math.log(2.0)
-	l = (np.log(total) + mx)[:, 0] * log2e + math.log2(255.0)
-	pq = np.rint(p[:, 1:] * prob_steps) / prob_steps      # p <= 1, so quantize()'s clamp is idle
-	p = np.concatenate((p[:, :1], pq), axis=1)
-	o = (p @ v) / total
+	o = np.empty((t, hd), dtype=np.float64)
+	l = np.empty((t,), dtype=np.float64)
+	for r0 in range(0, t, row_block):
+		r1 = min(t, r0 + row_block)
+		ncol = r1 + 1                                   # sink + keys 0 .. r1-1
+		s = q[r0:r1] @ k[:ncol].T
+		rows = np.arange(r0, r1)[:, None]
+		cols = np.arange(ncol - 1)[None, :]
+		real_mask = cols >= rows
+		if window > 0:
+			real_mask |= cols < rows - window
+		mask = np.zeros((r1 - r0, ncol), dtype=bool)
+		mask[:, 1:] = real_mask
+		s = np.where(mask, -np.inf, s)
+		s = s * temperature[r0:r1]
+		mx = s.max(axis=1, keepdims=True)
+		p = np.exp(s - mx)
+		total = p.sum(axis=1, keepdims=True)
+		l[r0:r1] = (np.log(total) + mx)[:, 0] * log2e + math.log2(255.0)
+		p[:, 1:] = np.rint(p[:, 1:] * prob_steps) / prob_steps   # p <= 1: quantize()'s clamp is idle
+		o[r0:r1] = (p @ v[:ncol]) / total
 	return o, l
 
 

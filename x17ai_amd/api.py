@@ -1,0 +1,367 @@
+"""Python mirror of the reference's operator API for the quantized block-forward path.
+
+Names and argument meaning follow the Rust side: GemmKernel / GemmConfig / ScaleConfig /
+RMSNormConfig / ResidualConfig / GeGluConfig (src/device/cuda/gemm.rs:28-449), AttnKernel /
+AttnKernelConfig (src/device/cuda/attn.rs:45-240), Tensor (src/tensor.rs), CudaDevice and
+CudaTimer (src/device/cuda.rs) -- here Device and Timer.  Each object owns a handle of the
+C++ operator layer; numpy arrays only cross at Tensor.upload / Tensor.download.
+"""
+from __future__ import annotations
+
+import ctypes
+import dataclasses
+from typing import Optional, Sequence, Union
+
+import numpy as np
+
+from . import _ffi
+from ._ffi import X17Error, check
+
+# DType, src/dtype.rs:1-15
+E4M3, INT8, BF16, F32 = 0, 1, 2, 3
+_DTYPE_BYTES = {E4M3: 1, INT8: 1, BF16: 2, F32: 4}
+_DTYPE_NAME = {E4M3: "e4m3", INT8: "i8", BF16: "bf16", F32: "f32"}
+
+
+class Device:
+	"""CudaDevice::new(device_id), src/device/cuda.rs:31-38 -- one HIP device with one stream."""
+
+	def __init__(self, device_id: int = 0):
+		self._h = ctypes.c_void_p()
+		check(_ffi.host().x17h_device_new(device_id, ctypes.byref(self._h)))
+
+	def synchronize(self) -> None:
+		check(_ffi.host().x17h_device_synchronize(self._h))
+
+	@property
+	def name(self) -> str:
+		return _ffi.host().x17h_device_name(self._h).decode()
+
+	def close(self) -> None:
+		if self._h:
+			_ffi.host().x17h_device_free(self._h)
+			self._h = ctypes.c_void_p()
+
+	def __del__(self):
+		try:
+			self.close()
+		except Exception:
+			pass
+
+
+class Tensor:
+	"""Contiguous tensor = (dtype, shape, device buffer), src/tensor.rs:23-112."""
+
+	def __init__(self, device: Optional[Device], shape: Sequence[int], dtype: int):
+		self.device = device
+		self.shape = tuple(int(s) for s in shape)
+		self.dtype = dtype
+		self._h = ctypes.c_void_p()
+		arr = (ctypes.c_size_t * len(self.shape))(*self.shape)
+		check(_ffi.host().x17h_tensor_new_empty(device._h if device is not None else None, arr, len(self.shape), dtype,
+		                                        ctypes.byref(self._h)))
+
+	@classmethod
+	def new_empty(cls, shape: Sequence[int], dtype: int, device: Optional[Device]) -> "Tensor":
+		return cls(device, shape, dtype)
+
+	@classmethod
+	def from_numpy(cls, device: Optional[Device], array: np.ndarray, dtype: int) -> "Tensor":
+		t = cls(device, array.shape, dtype)
+		t.upload(array)
+		return t
+
+	@property
+	def nbytes(self) -> int:
+		return int(_ffi.host().x17h_tensor_bytes(self._h))
+
+	def upload(self, array: np.ndarray) -> None:
+		array = np.ascontiguousarray(array)
+		if array.nbytes != self.nbytes:
+			raise X17Error(f"upload of {array.nbytes} bytes into a tensor of {self.nbytes} bytes")
+		# the copy is asynchronous on the device stream; the source must outlive it
+		self._staging = array
+		check(_ffi.host().x17h_tensor_upload(self._h, array.ctypes.data_as(ctypes.c_void_p), array.nbytes))
+
+	def download(self, np_dtype=None) -> np.ndarray:
+		"""Tensor::to_cpu + synchronize (src/tensor.rs:98-112, src/main.rs:265)."""
+		if np_dtype is None:
+			np_dtype = {E4M3: np.uint8, INT8: np.int8, BF16: np.uint16, F32: np.float32}[self.dtype]
+		out = np.empty(self.shape, dtype=np_dtype)
+		if out.nbytes != self.nbytes:
+			raise X17Error(f"download of {self.nbytes} bytes into an array of {out.nbytes} bytes")
+		check(_ffi.host().x17h_tensor_download(self._h, out.ctypes.data_as(ctypes.c_void_p), out.nbytes))
+		if self.device is not None:
+			self.device.synchronize()
+		return out
+
+	def reshape(self, shape: Sequence[int]) -> "Tensor":
+		shape = tuple(int(s) for s in shape)
+		arr = (ctypes.c_size_t * len(shape))(*shape)
+		check(_ffi.host().x17h_tensor_reshape(self._h, arr, len(shape)))
+		self.shape = shape
+		return self
+
+	def device_ptr(self) -> int:
+		return int(_ffi.host().x17h_tensor_device_ptr(self._h) or 0)
+
+	def close(self) -> None:
+		if self._h:
+			_ffi.host().x17h_tensor_free(self._h)
+			self._h = ctypes.c_void_p()
+
+	def __del__(self):
+		try:
+			self.close()
+		except Exception:
+			pass
+
+
+class Timer:
+	"""CudaTimer, src/device/cuda.rs:79-101: a pair of events on the device's stream."""
+
+	def __init__(self, device: Device):
+		self.device = device
+		self._h = ctypes.c_void_p()
+		check(_ffi.host().x17h_timer_new(device._h, ctypes.byref(self._h)))
+
+	def start(self) -> None:
+		check(_ffi.host().x17h_timer_start(self._h))
+
+	def stop(self) -> None:
+		check(_ffi.host().x17h_timer_stop(self._h))
+
+	def elapsed_seconds(self) -> float:
+		s = ctypes.c_double()
+		check(_ffi.host().x17h_timer_elapsed_seconds(self._h, ctypes.byref(s)))
+		return float(s.value)
+
+	def __del__(self):
+		try:
+			if self._h:
+				_ffi.host().x17h_timer_free(self._h)
+				self._h = ctypes.c_void_p()
+		except Exception:
+			pass
+
+
+# ---------------------------------------------------------------- GEMM
+
+@dataclasses.dataclass
+class GemmInputConfig:          # gemm.rs:59-64
+	dtype: int
+	cols: int
+	rows: Optional[int]
+	trans: bool
+
+
+@dataclasses.dataclass
+class GemmConfig:               # gemm.rs:66-70
+	a: GemmInputConfig
+	b: GemmInputConfig
+	c_dtype: int
+
+
+@dataclasses.dataclass
+class ScaleConfig:              # gemm.rs:33-36
+	inp_scale: float
+	out_scale: float
+	kind = 0
+
+
+@dataclasses.dataclass
+class GeGluConfig:              # gemm.rs:52-55
+	inp_scale: float
+	out_scale: float
+	kind = 1
+
+
+@dataclasses.dataclass
+class ResidualConfig:           # gemm.rs:47-50
+	inp_scale: float
+	out_scale: float
+	kind = 2
+
+
+@dataclasses.dataclass
+class RMSNormConfig:            # gemm.rs:38-45
+	eps: float
+	head_dim: int
+	sep_dim: int
+	inp_scale: float
+	out_scale: float
+	kind = 3
+
+
+EpilogueConfig = Union[ScaleConfig, GeGluConfig, ResidualConfig, RMSNormConfig]
+
+
+def _attrs_dict(raw) -> dict:
+	names = ["max_threads_per_block", "static_shared_size_bytes", "const_size_bytes", "local_size_bytes", "num_regs",
+	         "ptx_version", "binary_version", "max_dynamic_shared_size_bytes", "preferred_shared_memory_carveout"]
+	return {n: int(raw[i]) for i, n in enumerate(names)}
+
+
+class GemmKernel:
+	"""GemmKernel::<Epilogue>::new / launch / n_ops, src/device/cuda/gemm.rs:350-449.
+
+	`device=None` generates and compiles the code object without loading it (what a build
+	step on a machine without a GPU does).  `strict_math` picks the deterministic
+	transcendental build (bit-exact against the CPU checker) over the hardware one."""
+
+	def __init__(self, device: Optional[Device], kernel_name: str, gemm_config: GemmConfig,
+	             epilogue_config: EpilogueConfig, strict_math: bool = True):
+		c = _ffi.GemmConfigC()
+		c.a_dtype, c.a_cols, c.a_rows, c.a_trans = gemm_config.a.dtype, gemm_config.a.cols, gemm_config.a.rows or 0, int(gemm_config.a.trans)
+		c.b_dtype, c.b_cols, c.b_rows, c.b_trans = gemm_config.b.dtype, gemm_config.b.cols, gemm_config.b.rows or 0, int(gemm_config.b.trans)
+		c.c_dtype = gemm_config.c_dtype
+		c.epilogue = epilogue_config.kind
+		c.inp_scale = epilogue_config.inp_scale
+		c.out_scale = epilogue_config.out_scale
+		c.eps = getattr(epilogue_config, "eps", 0.0)
+		c.head_dim = getattr(epilogue_config, "head_dim", 0)
+		c.sep_dim = getattr(epilogue_config, "sep_dim", 0)
+		c.strict_math = int(strict_math)
+		self.device = device
+		self.name = kernel_name
+		self.epilogue_kind = epilogue_config.kind
+		self._h = ctypes.c_void_p()
+		check(_ffi.host().x17h_gemm_kernel_new(device._h if device is not None else None, kernel_name.encode(),
+		                                       ctypes.byref(c), ctypes.byref(self._h)))
+		self.diagnostics = _ffi.last_diagnostics()
+
+	def launch(self, a: Tensor, b: Tensor, c: Tensor, extra: Optional[Tensor] = None) -> None:
+		check(_ffi.host().x17h_gemm_kernel_launch(self._h, a._h, b._h, c._h, extra._h if extra is not None else None))
+
+	def n_ops(self, a: Tensor, b: Tensor) -> float:
+		return float(_ffi.host().x17h_gemm_kernel_n_ops(self._h, a._h, b._h))
+
+	@property
+	def metadata(self) -> dict:
+		out = (ctypes.c_size_t * 4)()
+		check(_ffi.host().x17h_gemm_kernel_metadata(self._h, out))
+		return dict(zip(["THREADS_PER_BLOCK", "SMEM_BYTES", "M_PER_BLOCK", "N_PER_BLOCK"], [int(v) for v in out]))
+
+	@property
+	def attrs(self) -> dict:
+		out = (ctypes.c_int32 * 9)()
+		check(_ffi.host().x17h_gemm_kernel_attrs(self._h, out))
+		return _attrs_dict(out)
+
+	def __del__(self):
+		try:
+			if self._h:
+				_ffi.host().x17h_gemm_kernel_free(self._h)
+				self._h = ctypes.c_void_p()
+		except Exception:
+			pass
+
+
+# ---------------------------------------------------------------- attention
+
+@dataclasses.dataclass
+class AttnKernelConfig:         # attn.rs:45-84
+	dtype: int
+	n_heads: int
+	head_dim: int
+	q_stride: int
+	kv_stride: int
+	o_stride: int
+
+	def heads_per_kernel(self) -> int:
+		return 1 if self.head_dim == 0 else max(128 // self.head_dim, 1)
+
+	def head_group_cnt(self) -> int:
+		return self.n_heads // self.heads_per_kernel()
+
+
+class AttnKernel:
+	"""AttnKernel::new / launch, src/device/cuda/attn.rs:156-240."""
+
+	def __init__(self, device: Optional[Device], kernel_name: str, config: AttnKernelConfig, strict_math: bool = True):
+		c = _ffi.AttnConfigC(config.dtype, config.n_heads, config.head_dim, config.q_stride, config.kv_stride,
+		                     config.o_stride, int(strict_math))
+		self.device = device
+		self.name = kernel_name
+		self.config = config
+		self._h = ctypes.c_void_p()
+		check(_ffi.host().x17h_attn_kernel_new(device._h if device is not None else None, kernel_name.encode(),
+		                                       ctypes.byref(c), ctypes.byref(self._h)))
+		self.diagnostics = _ffi.last_diagnostics()
+
+	def launch(self, q: Tensor, kv: Tensor, sink_k: Tensor, sink_v: Tensor, attn_temperature: Tensor, out: Tensor,
+	           l: Optional[Tensor], window_size: int, batch: int = 1) -> None:
+		check(_ffi.host().x17h_attn_kernel_launch(self._h, q._h, kv._h, sink_k._h, sink_v._h, attn_temperature._h, out._h,
+		                                          l._h if l is not None else None, window_size, batch))
+
+	def n_ops(self, seq_len: int, window_size: int) -> float:
+		return float(_ffi.host().x17h_attn_kernel_n_ops(self._h, seq_len, window_size))
+
+	@property
+	def metadata(self) -> dict:
+		out = (ctypes.c_size_t * 3)()
+		check(_ffi.host().x17h_attn_kernel_metadata(self._h, out))
+		return dict(zip(["THREADS_PER_BLOCK", "SMEM_BYTES", "Q_PER_BLOCK"], [int(v) for v in out]))
+
+	@property
+	def attrs(self) -> dict:
+		out = (ctypes.c_int32 * 9)()
+		check(_ffi.host().x17h_attn_kernel_attrs(self._h, out))
+		return _attrs_dict(out)
+
+	def __del__(self):
+		try:
+			if self._h:
+				_ffi.host().x17h_attn_kernel_free(self._h)
+				self._h = ctypes.c_void_p()
+		except Exception:
+			pass
+
+
+class RmsNormKernel:
+	"""The reference's stand-alone rms_norm kernel (rms_norm.cu:55-113) as a kernel object."""
+
+	def __init__(self, device: Optional[Device], kernel_name: str, in_dtype: int, model_dim: int, eps: float):
+		self.device = device
+		self.name = kernel_name
+		self._h = ctypes.c_void_p()
+		check(_ffi.host().x17h_rms_norm_kernel_new(device._h if device is not None else None, kernel_name.encode(),
+		                                           in_dtype, model_dim, eps, ctypes.byref(self._h)))
+		self.diagnostics = _ffi.last_diagnostics()
+
+	def launch(self, inp: Tensor, out: Tensor) -> None:
+		check(_ffi.host().x17h_rms_norm_kernel_launch(self._h, inp._h, out._h))
+
+	def __del__(self):
+		try:
+			if self._h:
+				_ffi.host().x17h_rms_norm_kernel_free(self._h)
+				self._h = ctypes.c_void_p()
+		except Exception:
+			pass
+
+
+class AttnDecodeKernel:
+	"""Single-token decode against an int8 KV cache (no counterpart in the reference)."""
+
+	def __init__(self, device: Optional[Device], kernel_name: str, n_heads: int, head_dim: int, cache_capacity: int,
+	             strict_math: bool = True):
+		self.device = device
+		self.name = kernel_name
+		self._h = ctypes.c_void_p()
+		check(_ffi.host().x17h_decode_kernel_new(device._h if device is not None else None, kernel_name.encode(),
+		                                         n_heads, head_dim, cache_capacity, int(strict_math), ctypes.byref(self._h)))
+		self.diagnostics = _ffi.last_diagnostics()
+
+	def launch(self, q: Tensor, cache: Tensor, cache_len: Tensor, sink_k: Tensor, sink_v: Tensor,
+	           attn_temperature: Tensor, out: Tensor, l: Optional[Tensor], window_size: int) -> None:
+		check(_ffi.host().x17h_decode_kernel_launch(self._h, q._h, cache._h, cache_len._h, sink_k._h, sink_v._h,
+		                                            attn_temperature._h, out._h, l._h if l is not None else None, window_size))
+
+	def __del__(self):
+		try:
+			if self._h:
+				_ffi.host().x17h_decode_kernel_free(self._h)
+				self._h = ctypes.c_void_p()
+		except Exception:
+			pass
