@@ -1,0 +1,174 @@
+"""GPU parity of the int8 sliding-window attention (prefill), the single-token decode and rms_norm.
+
+Checker: the CPU oracle's restatement of the reference's op sequence (oracle/x17_oracle.c), which
+itself reproduces the CUDA side of the reference's golden report (tests/test_oracle_golden.py).
+Bars: strict_math builds are bit-exact (int8 output codes and the f32 log-sum-exp bits);
+hardware-exponent builds stay within one output code in a stated small fraction of elements.
+"""
+import numpy as np
+import pytest
+
+import x17ai_amd as X
+from x17ai_amd import recipes
+from oracle import strict as S
+from tests.gpu_common import e4m3_bytes, i8_codes, rng_for
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+	d = X.Device(0)
+	yield d
+	d.synchronize()
+
+
+def _attn_inputs(rng, rows, h, hd):
+	q = i8_codes(rng, (rows, h * hd))
+	k = rng.standard_normal((rows, h, hd))
+	k /= np.sqrt((k * k).mean(-1, keepdims=True))                  # K is RMS-normed upstream
+	v = rng.standard_normal((rows, h, hd)) * 1.3
+	kv = S.f32_to_fixedi8((np.concatenate((k, v), axis=2).reshape(rows, 2 * h * hd) * 8).astype(np.float32))
+	sk = rng.standard_normal((h, hd))
+	sk /= np.sqrt((sk * sk).mean(-1, keepdims=True))
+	sink_k = S.f32_to_fixedi8((sk * 8).astype(np.float32))
+	sink_v = i8_codes(rng, (h, hd), 1.3)
+	temp = (0.5 + rng.random(h)).astype(np.float32)
+	return q, kv, sink_k, sink_v, temp
+
+
+def _run_attn(dev, kern, q, kv, sink_k, sink_v, temp, window, batch=1, want_l=True):
+	h = sink_k.shape[0]
+	out = X.Tensor(dev, q.shape, X.INT8)
+	l = X.Tensor(dev, (h, q.shape[0]), X.F32) if want_l else None
+	kern.launch(X.Tensor.from_numpy(dev, q, X.INT8), X.Tensor.from_numpy(dev, kv, X.INT8),
+	            X.Tensor.from_numpy(dev, sink_k, X.INT8), X.Tensor.from_numpy(dev, sink_v, X.INT8),
+	            X.Tensor.from_numpy(dev, temp, X.F32), out, l, window, batch)
+	return out.download(), (l.download() if want_l else None)
+
+
+# (T, H, hd, window)
+CASES = [
+	(256, 4, 32, 0), (256, 4, 32, 64), (384, 2, 64, 0), (512, 2, 64, 128), (512, 2, 64, 16),
+	(384, 2, 128, 0), (640, 2, 128, 256), (1024, 8, 64, 256),          # the last one is BASELINE config 1
+]
+
+
+@pytest.mark.parametrize("t,h,hd,w", CASES)
+def test_attn_strict_bit_exact(dev, t, h, hd, w):
+	rng = rng_for("attn", t, h, hd, w)
+	q, kv, sk, sv, temp = _attn_inputs(rng, t, h, hd)
+	kern = recipes.attn_kernel(dev, h, hd, True)
+	got, got_l = _run_attn(dev, kern, q, kv, sk, sv, temp, w)
+	want, want_l = S.attn_fwd_i8(q, kv, sk, sv, temp, h, hd, w)
+	assert np.array_equal(got, want)
+	assert np.array_equal(got_l.view(np.uint32), want_l.view(np.uint32))
+
+
+@pytest.mark.parametrize("t,h,hd,w", [(512, 2, 64, 128), (640, 2, 128, 256), (1024, 8, 64, 256)])
+def test_attn_fast_within_one_code(dev, t, h, hd, w):
+	rng = rng_for("attn", t, h, hd, w)
+	q, kv, sk, sv, temp = _attn_inputs(rng, t, h, hd)
+	kern = recipes.attn_kernel(dev, h, hd, False)
+	got, got_l = _run_attn(dev, kern, q, kv, sk, sv, temp, w)
+	want, want_l = S.attn_fwd_i8(q, kv, sk, sv, temp, h, hd, w)
+	d = np.abs(got.astype(np.int32) - want.astype(np.int32))
+	assert d.max() <= 1 and np.mean(d > 0) < 0.02, (d.max(), np.mean(d > 0))
+	assert np.max(np.abs(got_l - want_l)) < 1e-4
+
+
+def test_attn_batched_sequences_and_no_l(dev):
+	"""gridDim.z extension: stacked sequences are independent; L may be omitted (attn.rs:396)."""
+	t, h, hd, w, b = 256, 2, 64, 64, 3
+	rng = rng_for("attn-batch")
+	q, kv, sk, sv, temp = _attn_inputs(rng, b * t, h, hd)
+	kern = recipes.attn_kernel(dev, h, hd, True)
+	got, got_l = _run_attn(dev, kern, q, kv, sk, sv, temp, w, batch=b)
+	got2, _ = _run_attn(dev, kern, q, kv, sk, sv, temp, w, batch=b, want_l=False)
+	for i in range(b):
+		want, want_l = S.attn_fwd_i8(q[i * t:(i + 1) * t], kv[i * t:(i + 1) * t], sk, sv, temp, h, hd, w)
+		assert np.array_equal(got[i * t:(i + 1) * t], want)
+		assert np.array_equal(got_l[:, i * t:(i + 1) * t].view(np.uint32), want_l.view(np.uint32))
+	assert np.array_equal(got, got2)
+
+
+def test_attn_special_cases(dev):
+	"""Closed-form cases: query 0 sees only the sink; constant V gives V back; a window that covers
+	the whole sequence equals no window."""
+	t, h, hd = 256, 2, 64
+	rng = rng_for("attn-special")
+	q, kv, sk, sv, temp = _attn_inputs(rng, t, h, hd)
+	kern = recipes.attn_kernel(dev, h, hd, True)
+	got, _ = _run_attn(dev, kern, q, kv, sk, sv, temp, 0)
+	assert np.array_equal(got[0].reshape(h, hd), sv)
+	got_w, _ = _run_attn(dev, kern, q, kv, sk, sv, temp, 256)
+	assert np.array_equal(got, got_w)
+	kv2 = kv.reshape(t, h, 2, hd).copy()
+	kv2[:, :, 1, :] = 40
+	sv2 = np.full_like(sv, 40)
+	got_c, _ = _run_attn(dev, kern, q, kv2.reshape(t, -1), sk, sv2, temp, 64)
+	assert np.all(got_c == 40)
+
+
+def test_attn_launch_rejects_bad_arguments(dev):
+	h, hd = 2, 64
+	kern = recipes.attn_kernel(dev, h, hd, True)
+	rng = rng_for("attn-bad")
+	q, kv, sk, sv, temp = _attn_inputs(rng, 256, h, hd)
+	with pytest.raises(X.X17Error, match="window_size must be zero or divisible by 16"):
+		_run_attn(dev, kern, q, kv, sk, sv, temp, 24)
+	with pytest.raises(X.X17Error, match="seq_len must be divisible by 128"):
+		_run_attn(dev, kern, q[:64], kv[:64], sk, sv, temp, 0)
+	with pytest.raises(X.X17Error, match="kv has 128 rows, but should have 256"):
+		_run_attn(dev, kern, q, kv[:128], sk, sv, temp, 0)
+
+
+# ---------------------------------------------------------------- decode
+
+@pytest.mark.parametrize("h,hd,cap,w", [(4, 32, 256, 0), (4, 64, 256, 64), (2, 128, 512, 128), (2, 128, 512, 0)])
+def test_decode_bit_exact_and_equals_prefill_row(dev, h, hd, cap, w):
+	s = 6
+	rng = rng_for("decode", h, hd, cap, w)
+	q, kv, sk, sv, temp = _attn_inputs(rng, s * cap, h, hd)
+	cache = kv.reshape(s, cap, 2 * h * hd)
+	qd = q[:s]
+	lens = np.array([0, 1, 17, cap // 2 + 5, cap - 1, cap], dtype=np.uint32)
+	kern = recipes.attn_decode_kernel(dev, h, hd, cap, True)
+	out = X.Tensor(dev, (s, h * hd), X.INT8)
+	l = X.Tensor(dev, (s, h), X.F32)
+	kern.launch(X.Tensor.from_numpy(dev, qd, X.INT8), X.Tensor.from_numpy(dev, cache, X.INT8),
+	            X.Tensor.from_numpy(dev, lens.view(np.float32), X.F32), X.Tensor.from_numpy(dev, sk, X.INT8),
+	            X.Tensor.from_numpy(dev, sv, X.INT8), X.Tensor.from_numpy(dev, temp, X.F32), out, l, w)
+	got, got_l = out.download(), l.download()
+	want, want_l = S.attn_decode_i8(qd, cache, lens, sk, sv, temp, h, hd, w)
+	assert np.array_equal(got, want)
+	assert np.array_equal(got_l.view(np.uint32), want_l.view(np.uint32))
+	# the definition: decoding at position p equals row p of a prefill over the first p+1 rows
+	seq = 3
+	p = int(lens[seq])
+	rows = ((p + 1 + 127) // 128) * 128
+	qq = np.zeros((rows, h * hd), np.int8)
+	qq[p] = qd[seq]
+	kk = np.zeros((rows, 2 * h * hd), np.int8)
+	kk[:p] = cache[seq, :p]
+	pre, pre_l = S.attn_fwd_i8(qq, kk, sk, sv, temp, h, hd, w)
+	assert np.array_equal(pre[p], got[seq])
+	assert np.array_equal(pre_l[:, p].view(np.uint32), got_l[seq].view(np.uint32))
+
+
+# ---------------------------------------------------------------- rms_norm
+
+@pytest.mark.parametrize("rows,d", [(8, 512), (64, 2048), (256, 4096)])
+def test_rms_norm_bit_exact(dev, rows, d):
+	rng = rng_for("rms", rows, d)
+	x = e4m3_bytes(rng, (rows, d), 1.5)
+	kern = recipes.rms_norm_kernel(dev, d, X.E4M3)
+	out = X.Tensor(dev, (rows, d), X.INT8)
+	kern.launch(X.Tensor.from_numpy(dev, x, X.E4M3), out)
+	assert np.array_equal(out.download(), S.rms_norm(x, recipes.L2_NORM_EPS, "e4m3"))
+	xb = (rng.standard_normal((rows, d)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+	kern_b = recipes.rms_norm_kernel(dev, d, X.BF16)
+	kern_b.launch(X.Tensor.from_numpy(dev, xb, X.BF16), out)
+	assert np.array_equal(out.download(), S.rms_norm(xb, recipes.L2_NORM_EPS, "bf16"))
+	with pytest.raises(X.X17Error, match="rows must be divisible by 8"):
+		kern.launch(X.Tensor(dev, (4, d), X.E4M3), X.Tensor(dev, (4, d), X.INT8))

@@ -1,0 +1,189 @@
+"""GPU parity of the 8-bit GEMM family (gemm_b8 / gemm_f8 and their four fused epilogues).
+
+Every call goes Python -> flat C ABI of the operator layer -> C-ABI device shim -> HIP kernel.
+The checker is the CPU oracle (oracle/x17_oracle.c).  Bars:
+  * int32 accumulators, Scale and L2-norm outputs, and everything built with strict_math:
+    bit-exact;
+  * hardware-transcendental builds (strict_math=False): at most one output code apart, in a
+    stated small fraction of elements;
+  * f32-accumulated GEMMs (any e4m3 operand): the summation order inside the matrix cores is
+    not the oracle's, so outputs may differ by one output code in a stated small fraction.
+"""
+import math
+
+import numpy as np
+import pytest
+
+import x17ai_amd as X
+from x17ai_amd import recipes
+from oracle import strict as S
+from tests.gpu_common import e4m3_bytes, e4m3_compare, i8_codes, rng_for
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+	d = X.Device(0)
+	yield d
+	d.synchronize()
+
+
+def _up(dev, arr, dtype):
+	return X.Tensor.from_numpy(dev, arr, dtype)
+
+
+SHAPES = [(256, 128, 256), (512, 1024, 512), (256, 2048, 1024)]     # (M, K, N_raw)
+
+
+@pytest.mark.parametrize("m,k,n", SHAPES)
+def test_scale_epilogue_bit_exact(dev, m, k, n):
+	rng = rng_for("scale", m, k, n)
+	a, b = i8_codes(rng, (m, k)), i8_codes(rng, (n, k))
+	kern = recipes.attn_q_kernel(dev, k, n)
+	c = X.Tensor(dev, (m, n), X.INT8)
+	kern.launch(_up(dev, a, X.INT8), _up(dev, b, X.INT8), c)
+	got = c.download()
+	want = S.epilogue_scale(S.gemm_i32(a, b), 1.0 / math.sqrt(k) / 64.0, 8.0)
+	assert np.array_equal(got, want)
+	assert kern.n_ops(_up(dev, a, X.INT8), _up(dev, b, X.INT8)) == 2.0 * m * k * n
+
+
+def test_int32_accumulators_bit_exact(dev):
+	"""Reads raw accumulators out through a Scale epilogue with scale 1: sparse +-1/0 operands keep
+	every |acc| <= 127, so the int8 output IS the accumulator."""
+	m, k, n = 256, 1024, 256
+	rng = rng_for("acc")
+	a = (rng.integers(-1, 2, (m, k)) * (rng.random((m, k)) < 0.05)).astype(np.int8)
+	b = (rng.integers(-1, 2, (n, k)) * (rng.random((n, k)) < 0.5)).astype(np.int8)
+	cfg = X.GemmConfig(X.GemmInputConfig(X.INT8, k, None, False), X.GemmInputConfig(X.INT8, k, n, True), X.INT8)
+	kern = X.GemmKernel(dev, f"acc_probe-k{k}-n{n}", cfg, X.ScaleConfig(1.0, 1.0))
+	c = X.Tensor(dev, (m, n), X.INT8)
+	kern.launch(_up(dev, a, X.INT8), _up(dev, b, X.INT8), c)
+	acc = a.astype(np.int64) @ b.astype(np.int64).T
+	assert np.abs(acc).max() <= 127 and np.abs(acc).max() >= 8
+	assert np.array_equal(c.download().astype(np.int64), acc)
+	# and the other extreme: saturated operands, |acc| up to K * 127 * 127, read through a small scale
+	a2 = np.where(rng.random((m, k)) < 0.5, 127, -127).astype(np.int8)
+	b2 = np.where(rng.random((n, k)) < 0.5, 127, -127).astype(np.int8)
+	a2[:8] = 127
+	b2[:8] = 127
+	kern2 = X.GemmKernel(dev, f"acc_probe2-k{k}-n{n}", cfg, X.ScaleConfig(1.0 / (k * 127.0), 1.0))
+	kern2.launch(_up(dev, a2, X.INT8), _up(dev, b2, X.INT8), c)
+	want = S.epilogue_scale(S.gemm_i32(a2, b2), 1.0 / (k * 127.0), 1.0)
+	assert want.max() == 127
+	assert np.array_equal(c.download(), want)
+
+
+@pytest.mark.parametrize("hd", [32, 64, 128])
+@pytest.mark.parametrize("m,k", [(256, 512), (512, 2048)])
+def test_l2norm_epilogue_bit_exact(dev, hd, m, k):
+	n = 512
+	rng = rng_for("l2", hd, m, k)
+	a, b = i8_codes(rng, (m, k)), i8_codes(rng, (n, k))
+	kern = recipes.attn_kv_kernel(dev, k, n, hd)
+	c = X.Tensor(dev, (m, n), X.INT8)
+	rrms = X.Tensor(dev, (m, n // (2 * hd)), X.F32)
+	kern.launch(_up(dev, a, X.INT8), _up(dev, b, X.INT8), c, rrms)
+	want_c, want_r = S.epilogue_l2norm(S.gemm_i32(a, b), hd, recipes.L2_NORM_EPS, 1.0 / math.sqrt(k) / 64.0, 8.0)
+	assert np.array_equal(c.download(), want_c)
+	assert np.array_equal(rrms.download().view(np.uint32), want_r.view(np.uint32))
+
+
+@pytest.mark.parametrize("store", [X.E4M3, X.INT8])
+@pytest.mark.parametrize("m,k,n", SHAPES)
+def test_geglu_epilogue(dev, m, k, n, store):
+	rng = rng_for("geglu", m, k, n, store)
+	a, b = i8_codes(rng, (m, k)), i8_codes(rng, (n, k))
+	acc = S.gemm_i32(a, b)
+	inp = 1.0 / math.sqrt(k) / 64.0
+	out_scale = 1.0 if store == X.E4M3 else 8.0
+	want = S.epilogue_geglu(acc, inp, out_scale, S.STORE_E4M3 if store == X.E4M3 else S.STORE_I8)
+	for strict in (True, False):
+		kern = recipes.ffn_f_kernel(dev, k, n, strict, store)
+		c = X.Tensor(dev, (m, n // 2), store)
+		kern.launch(_up(dev, a, X.INT8), _up(dev, b, X.INT8), c)
+		got = c.download()
+		if strict:
+			assert np.array_equal(got, want)
+		elif store == X.E4M3:
+			neq, beyond = e4m3_compare(got, want)
+			assert neq < 2e-3 and beyond == 0.0, (neq, beyond)
+		else:
+			d = np.abs(got.astype(np.int32) - want.astype(np.int32))
+			assert d.max() <= 1 and np.mean(d > 0) < 2e-3
+
+
+@pytest.mark.parametrize("store", [X.E4M3, X.INT8])
+@pytest.mark.parametrize("m,k,n", SHAPES)
+def test_residual_epilogue(dev, m, k, n, store):
+	rng = rng_for("residual", m, k, n, store)
+	a, b = i8_codes(rng, (m, k)), i8_codes(rng, (n, k))
+	r = i8_codes(rng, (m, n // 2))
+	acc = S.gemm_i32(a, b)
+	inp = 1.0 / math.sqrt(k) / 64.0
+	want = S.epilogue_residual(acc, r, inp, 1.0, S.STORE_E4M3 if store == X.E4M3 else S.STORE_I8)
+	for strict in (True, False):
+		kern = recipes.attn_y_kernel(dev, n // 2, k, strict, store)
+		c = X.Tensor(dev, (m, n // 2), store)
+		kern.launch(_up(dev, a, X.INT8), _up(dev, b, X.INT8), c, _up(dev, r, X.INT8))
+		got = c.download()
+		if strict:
+			assert np.array_equal(got, want)
+		elif store == X.E4M3:
+			neq, beyond = e4m3_compare(got, want)
+			assert neq < 2e-3 and beyond == 0.0, (neq, beyond)
+		else:
+			d = np.abs(got.astype(np.int32) - want.astype(np.int32))
+			assert d.max() <= 1 and np.mean(d > 0) < 2e-3
+
+
+@pytest.mark.parametrize("m,k,n", [(256, 512, 256), (512, 2048, 512)])
+def test_mixed_e4m3_i8_residual(dev, m, k, n):
+	"""ffn_y_fwd_f8: e4m3 activations x int8 weights on the bf16 matrix cores, f32 accumulate."""
+	rng = rng_for("mixed", m, k, n)
+	a = e4m3_bytes(rng, (m, k), 0.6)
+	b = i8_codes(rng, (n, k))
+	r = i8_codes(rng, (m, n // 2))
+	inp = math.sqrt(recipes.GELU_VAR_FIX_2 / k) / 8.0
+	want = S.epilogue_residual(S.gemm_f32_seq(a, True, b, False), r, inp, 1.0, S.STORE_E4M3)
+	kern = recipes.ffn_y_kernel(dev, n // 2, k, True)
+	c = X.Tensor(dev, (m, n // 2), X.E4M3)
+	kern.launch(_up(dev, a, X.E4M3), _up(dev, b, X.INT8), c, _up(dev, r, X.INT8))
+	neq, beyond = e4m3_compare(c.download(), want)
+	assert neq < 5e-3 and beyond == 0.0, (neq, beyond)
+
+
+@pytest.mark.parametrize("m,k,n", [(256, 512, 256), (512, 4096, 512)])
+def test_fp8_geglu(dev, m, k, n):
+	"""All-fp8 ffn_f: e4m3 x e4m3 on the fp8 matrix cores, f32 accumulate, GeGLU -> e4m3."""
+	rng = rng_for("fp8", m, k, n)
+	a = e4m3_bytes(rng, (m, k))
+	b = e4m3_bytes(rng, (n, k))
+	want = S.epilogue_geglu(S.gemm_f32_seq(a, True, b, True), 1.0 / math.sqrt(k), 1.0, S.STORE_E4M3)
+	kern = recipes.ffn_f_f8_kernel(dev, k, n, True)
+	c = X.Tensor(dev, (m, n // 2), X.E4M3)
+	kern.launch(_up(dev, a, X.E4M3), _up(dev, b, X.E4M3), c)
+	neq, beyond = e4m3_compare(c.download(), want)
+	assert neq < 5e-3 and beyond == 0.0, (neq, beyond)
+
+
+def test_launch_rejects_bad_arguments(dev):
+	"""Shape / dtype / device checks of the launcher (src/device/cuda/tensor_check.rs, gemm.rs:591-616)."""
+	k, n = 128, 256
+	kern = recipes.attn_q_kernel(dev, k, n)
+	a = X.Tensor(dev, (256, k), X.INT8)
+	b = X.Tensor(dev, (n, k), X.INT8)
+	c = X.Tensor(dev, (256, n), X.INT8)
+	with pytest.raises(X.X17Error, match="has dtype e4m3, but should have i8"):
+		kern.launch(X.Tensor(dev, (256, k), X.E4M3), b, c)
+	with pytest.raises(X.X17Error, match="columns, but should have 128"):
+		kern.launch(X.Tensor(dev, (256, 2 * k), X.INT8), b, c)
+	with pytest.raises(X.X17Error, match="must be 2D"):
+		kern.launch(X.Tensor(dev, (256, k, 1), X.INT8), b, c)
+	with pytest.raises(X.X17Error, match="must be divisible by tile shape"):
+		kern.launch(X.Tensor(dev, (64, k), X.INT8), b, X.Tensor(dev, (64, n), X.INT8))
+	with pytest.raises(X.X17Error, match="is not on device"):
+		kern.launch(X.Tensor(None, (256, k), X.INT8), b, c)
+	kern.launch(a, b, c)
+	dev.synchronize()

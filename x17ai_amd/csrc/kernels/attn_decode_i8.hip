@@ -1,0 +1,222 @@
+// attn_decode_i8.hip -- single-token attention against an int8 KV cache, for gfx950.
+//
+// The reference has no int8 decode kernel (its TODO.md:10-12 defers ragged tails to "the
+// incremental kernel"; attn_incremental.cu is the bf16 precedent for queries appended to a
+// longer KV).  This kernel is DEFINED as the prefill recurrence of cuda/attn_fwd_i8.cuh:368-619
+// for ONE query per sequence, at position cache_len[s], against cache rows [0, cache_len[s]):
+// same window rounding, same n = min(W', p) + 4, same 16-key tiles aligned at absolute
+// positions, same per-tile max / rescale / u8 probabilities / four partial sums / one f32 add
+// of the int32 P.V per tile.  So appending a token and decoding it gives bit for bit what a
+// prefill over the longer sequence gives for that row.
+//
+// The work is bandwidth: every cached K byte and V byte is read exactly once.  One workgroup
+// per (sequence, head); the recurrence is cut into phases so that only two cheap scans remain
+// sequential:
+//   1  scores: HD/16 lanes per key row (16-byte coalesced loads), v_dot4 + lane reduction
+//   2  per-tile max, prefix max over tiles (exact), rescale factors, probabilities, quad sums
+//   3  four partial-sum chains (4 lanes)
+//   4  P.V partials per tile in int32 (every lane, 16 dims x 16 keys), then one lane per output
+//      dim runs the O = O * rescale + f32(partial) chain over the tiles
+//
+// common.h provides X17_N_HEADS, X17_HEAD_DIM, X17_CACHE_CAPACITY, X17_STRICT_MATH.
+// Layouts: q, out [S, H*hd]; cache [S, CAPACITY, H*2*hd] (per head K then V, as kv of the
+// prefill kernel); cache_len u32 [S]; L [S, H] or null.
+
+#include "common.h"
+#include "x17_device.h"
+#include "decode_tile.h"
+
+using namespace x17;
+namespace dt = x17::decode_tile;
+
+namespace {
+constexpr u32 HD = X17_HEAD_DIM;
+constexpr u32 N_HEADS = X17_N_HEADS;
+constexpr u32 CAP = X17_CACHE_CAPACITY;
+constexpr u32 CPR = HD / 16;                         // lanes per key row
+constexpr u32 ROW = 2 * N_HEADS * HD;                // bytes per cache row
+constexpr u32 KEYS_PER_PASS = dt::THREADS_PER_BLOCK / CPR;
+constexpr f32 BASE_TEMPERATURE = f32(constexpr_inv_sqrt(f64(HD)) / 64.0);
+static_assert(HD == 32 || HD == 64 || HD == 128, "head_dim must be 32, 64 or 128");
+static_assert(CAP % 16 == 0, "cache capacity must be a multiple of 16");
+static_assert(dt::CHUNK_TILES * CPR == dt::THREADS_PER_BLOCK || dt::CHUNK_TILES * CPR < dt::THREADS_PER_BLOCK,
+              "one thread per (tile, 16-dim group) of a chunk");
+}
+
+extern "C" __global__ __launch_bounds__(dt::THREADS_PER_BLOCK)
+void kernel(
+	i8 const *q, i8 const *cache, u32 const *cache_len,
+	i8 const *sink_k, i8 const *sink_v, f32 const *attn_temperature,
+	i8 *out, f32 *l_out, u32 window_size
+) {
+	extern __shared__ __attribute__((aligned(16))) u8 smem[];
+	f32 *s_score = reinterpret_cast<f32 *>(smem);                               // [CAP]
+	u8 *s_prob = smem + CAP * 4;                                                 // [CAP]
+	f32 *s_quad = reinterpret_cast<f32 *>(smem + CAP * 5);                       // [CAP / 4]
+	f32 *s_tmax = reinterpret_cast<f32 *>(smem + CAP * 6);                       // [MAX_TILES]
+	f32 *s_resc = s_tmax + dt::MAX_TILES;                                        // [MAX_TILES]
+	f32 *s_mrun = s_resc + dt::MAX_TILES;                                        // [MAX_TILES]
+	f32 *s_bmax = s_mrun + dt::MAX_TILES;                                        // [256]
+	i32 *s_pv = reinterpret_cast<i32 *>(s_bmax + 256);                           // [CHUNK_TILES][HD]
+	f32 *s_sum = reinterpret_cast<f32 *>(s_pv + dt::CHUNK_TILES * HD);           // [4]
+
+	u32 const tid = threadIdx.x;
+	u32 const head = blockIdx.x;
+	u32 const seq = blockIdx.y;
+	u32 const pos_raw = cache_len[seq];                  // the query's position; keys are rows < pos
+	u32 const pos = pos_raw < CAP ? pos_raw : CAP;       // never read past the cache
+	u32 const wr = window_size == 0 ? 0xFFFFFFFFu : ((window_size - 1) / 16 + 1) * 16;
+	u32 const visible = pos < wr ? pos : wr;
+	u32 const j_lo = pos - visible;
+	u32 const t0 = j_lo / 16;
+	u32 const n_tiles = visible == 0 ? 0 : (pos - 1) / 16 - t0 + 1;
+
+	i8 const *kv_head = cache + (size_t)seq * CAP * ROW + (size_t)head * 2 * HD;
+	i8 const *q_head = q + (size_t)seq * N_HEADS * HD + (size_t)head * HD;
+
+	f32 temperature = BASE_TEMPERATURE * strict::lg2(f32(visible + 4u));
+	temperature = temperature * attn_temperature[head];
+
+	// this lane's 16 bytes of the query (chunk tid % CPR)
+	u32 const c = tid % CPR;
+	v4i const qc = *reinterpret_cast<v4i const *>(q_head + 16 * c);
+
+	// sink score (every group of CPR lanes computes it)
+	i32 sink_dot = 0;
+	{
+		v4i sk = *reinterpret_cast<v4i const *>(sink_k + (size_t)head * HD + 16 * c);
+		X17_UNROLL for (int w = 0; w < 4; ++w) sink_dot = __builtin_amdgcn_sdot4(qc[w], sk[w], sink_dot, false);
+		X17_UNROLL for (u32 mask = 1; mask < CPR; mask <<= 1) sink_dot += __shfl_xor(sink_dot, (int)mask, 64);
+	}
+	f32 const m0 = f32(sink_dot) * temperature;
+
+	// ---- phase 1: scores of all keys of the walked tiles
+	u32 const n_keys = n_tiles * 16;
+	for (u32 base = 0; base < n_keys; base += KEYS_PER_PASS) {
+		u32 kidx = base + tid / CPR;
+		u32 j = t0 * 16 + kidx;
+		bool in_range = kidx < n_keys;
+		bool vis = in_range && j >= j_lo && j < pos;
+		i32 dot = 0;
+		if (vis) {
+			v4i kc = *reinterpret_cast<v4i const *>(kv_head + (size_t)j * ROW + 16 * c);
+			X17_UNROLL for (int w = 0; w < 4; ++w) dot = __builtin_amdgcn_sdot4(qc[w], kc[w], dot, false);
+		}
+		X17_UNROLL for (u32 mask = 1; mask < CPR; mask <<= 1) dot += __shfl_xor(dot, (int)mask, 64);
+		if (in_range && c == 0) {
+			s_score[kidx] = vis ? f32(dot) * temperature : -__builtin_inff();
+		}
+	}
+	__syncthreads();
+
+	// ---- phase 2a: per-tile max; each thread owns TPT consecutive tiles
+	constexpr u32 TPT = (dt::MAX_TILES + dt::THREADS_PER_BLOCK - 1) / dt::THREADS_PER_BLOCK;
+	f32 block_max = -__builtin_inff();
+	X17_UNROLL for (u32 i = 0; i < TPT; ++i) {
+		u32 t = tid * TPT + i;
+		if (t < n_tiles) {
+			f32 mx = -__builtin_inff();
+			X17_UNROLL for (int k = 0; k < 16; k += 4) {
+				v4f v = *reinterpret_cast<v4f const *>(s_score + t * 16 + k);
+				mx = __builtin_fmaxf(mx, __builtin_fmaxf(__builtin_fmaxf(v[0], v[1]), __builtin_fmaxf(v[2], v[3])));
+			}
+			s_tmax[t] = mx;
+			block_max = __builtin_fmaxf(block_max, mx);
+		}
+	}
+	s_bmax[tid] = block_max;
+	__syncthreads();
+
+	// ---- phase 2b: running max before each thread's tiles (max is exact, so any grouping works),
+	// then running max and rescale factor of every tile (cuda/attn_fwd_i8.cuh:233-256)
+	{
+		f32 m_prev = m0;
+		for (u32 t = 0; t < tid; ++t) m_prev = __builtin_fmaxf(m_prev, s_bmax[t]);
+		X17_UNROLL for (u32 i = 0; i < TPT; ++i) {
+			u32 t = tid * TPT + i;
+			if (t < n_tiles) {
+				f32 tm = s_tmax[t];
+				f32 resc = 1.0f;
+				if (tm > m_prev) {
+					resc = sfu::ex2(m_prev - tm);
+					m_prev = tm;
+				}
+				s_mrun[t] = m_prev;
+				s_resc[t] = resc;
+			}
+		}
+	}
+	__syncthreads();
+
+	// ---- phase 2c: probabilities and quad sums (:265-290); one key quad per thread per pass
+	for (u32 quad = tid; quad < n_tiles * 4; quad += dt::THREADS_PER_BLOCK) {
+		f32 m = s_mrun[quad / 4];
+		v4f s = *reinterpret_cast<v4f const *>(s_score + quad * 4);
+		f32 p0 = sfu::ex2(s[0] - m) * 255.0f;
+		f32 p1 = sfu::ex2(s[1] - m) * 255.0f;
+		f32 p2 = sfu::ex2(s[2] - m) * 255.0f;
+		f32 p3 = sfu::ex2(s[3] - m) * 255.0f;
+		s_quad[quad] = (p0 + p1) + (p2 + p3);
+		u32 packed = (u32)(i32)__builtin_rintf(p0) | ((u32)(i32)__builtin_rintf(p1) << 8)
+			| ((u32)(i32)__builtin_rintf(p2) << 16) | ((u32)(i32)__builtin_rintf(p3) << 24);
+		*reinterpret_cast<u32 *>(s_prob + quad * 4) = packed;
+	}
+	__syncthreads();
+
+	// ---- phase 3: the four partial-sum chains
+	if (tid < 4) {
+		f32 sum = 63.75f;
+		for (u32 t = 0; t < n_tiles; ++t) sum = fmaf32(sum, s_resc[t], s_quad[t * 4 + tid]);
+		s_sum[tid] = sum;
+	}
+
+	// ---- phase 4: O chains.  Lane d < HD owns output dim d.
+	f32 o = 0.0f;
+	if (tid < HD) {
+		o = f32((i32)sink_v[(size_t)head * HD + tid] * 255);
+	}
+	for (u32 chunk = 0; chunk < n_tiles; chunk += dt::CHUNK_TILES) {
+		u32 const tiles_here = n_tiles - chunk < dt::CHUNK_TILES ? n_tiles - chunk : dt::CHUNK_TILES;
+		// 4a: int32 P.V of one tile x 16 dims per thread
+		u32 const tl = tid / CPR;
+		if (tl < tiles_here) {
+			u32 const t = chunk + tl;
+			i32 acc[16];
+			X17_UNROLL for (int i = 0; i < 16; ++i) acc[i] = 0;
+			v4u probs = *reinterpret_cast<v4u const *>(s_prob + t * 16);
+			X17_UNROLL for (int k = 0; k < 16; ++k) {
+				i32 p = (i32)((probs[k / 4] >> (8 * (k % 4))) & 0xFFu);
+				u32 j = (t0 + t) * 16 + k;
+				if (p != 0) {     // masked keys have p == 0 (and may lie outside the cache)
+					v4i vv = *reinterpret_cast<v4i const *>(kv_head + (size_t)j * ROW + HD + 16 * c);
+					X17_UNROLL for (int i = 0; i < 16; ++i) {
+						acc[i] += p * (i32)(i8)(((u32)vv[i / 4] >> (8 * (i % 4))) & 0xFFu);
+					}
+				}
+			}
+			X17_UNROLL for (int i = 0; i < 16; i += 4) {
+				*reinterpret_cast<v4i *>(s_pv + tl * HD + 16 * c + i) = v4i{acc[i], acc[i + 1], acc[i + 2], acc[i + 3]};
+			}
+		}
+		__syncthreads();
+		// 4b: one f32 multiply (rescale) and one f32 add per tile (:247-252, :588-605)
+		if (tid < HD) {
+			for (u32 tl2 = 0; tl2 < tiles_here; ++tl2) {
+				o = o * s_resc[chunk + tl2];
+				o = o + f32(s_pv[tl2 * HD + tid]);
+			}
+		}
+		__syncthreads();
+	}
+
+	// ---- finish (:293-351)
+	__syncthreads();
+	f32 const total = (s_sum[0] + s_sum[1]) + (s_sum[2] + s_sum[3]);
+	f32 const m_final = n_tiles == 0 ? m0 : s_mrun[n_tiles - 1];
+	if (tid == 0 && l_out != nullptr) {
+		l_out[(size_t)seq * N_HEADS + head] = strict::lg2(total) + m_final;
+	}
+	if (tid < HD) {
+		out[(size_t)seq * N_HEADS * HD + (size_t)head * HD + tid] = (i8)f32_to_fixedi8(o * strict::rcp(total));
+	}
+}

@@ -1,0 +1,332 @@
+// attn_fwd_i8.hip -- int8 causal sliding-window flash-attention forward with a sink token and
+// scalable-softmax temperature, for gfx950.
+//
+// Replaces the reference's AttnForward (cuda/attn_fwd_i8.cuh:30-620); the kernel entry and its
+// parameters follow templates/attn/kernel.cu:9-33.  The arithmetic it reproduces, per head and
+// query i (0-based position inside its sequence):
+//   keys j in [max(0, i - W'), i - 1] plus one sink key/value; W' = window rounded up to 16
+//   (0 = no window);  n = min(W', i) + 4;  temperature = f32(hd^-1/2 / 64) * lg2(n) * head_temp[h];
+//   s_j = f32(q_i . k_j) * temperature (int32 dot);  running max starts at the sink score, the
+//   partial sums at 4 x 63.75, O at 255 * sink_v;  per 16-key tile (ascending): rescale when the
+//   max grows, p_j = ex2(s_j - max) * 255, four partial sums over key quads of the tile,
+//   P_j = rne(p_j), O += f32(sum_j P_j v_j);  at the end sum = (s0+s1)+(s2+s3),
+//   L = lg2(sum) + max, out = fixedi8(O / sum).
+//
+// Design, MI355X-first:
+//   * One workgroup = 4 wavefronts = 128 queries of one head; a wavefront owns 32 queries.
+//     Keys/values are staged 32 keys per step (two 16-key tiles), double-buffered in LDS.
+//   * S^T = K . Q^T on v_mfma_i32_32x32x32_i8 with the KEYS as the MFMA "A" operand: a lane then
+//     owns one query (lane % 32) and 8 keys of each 16-key tile; the other 8 keys sit in lane+32.
+//     Row max needs one cross-lane exchange per tile; the four per-quad partial sums of the
+//     reference fall two-and-two into the lane pair, so they need none until the very end.
+//   * P stays in registers: packed to bf16 it already IS the "B" operand of O^T = V^T . P^T.
+//     PV runs on v_mfma_f32_32x32x16_bf16: K = 16 is exactly one 16-key tile, P (0..255) and
+//     int8 V are exact in bf16 and every tile sum is below 2^24, so the f32 result equals the
+//     reference's f32(int32 dot) bit for bit.  (CDNA4 has no unsigned x signed int8 MFMA; an
+//     int8 PV would need two MFMAs per tile for the 8-bit probabilities.)
+//   * V is widened to bf16 once per workgroup on its way into LDS and fetched transposed with
+//     ds_read_b64_tr_b16, so no register transposes; K goes global -> LDS directly.
+//   * X17_STRICT_MATH = 1: deterministic ex2 and one explicit f32 add per tile (parity build).
+//     X17_STRICT_MATH = 0: v_exp_f32 and accumulation inside the PV MFMA (speed build).
+//
+// common.h (generated per kernel) provides X17_N_HEADS, X17_HEAD_DIM, X17_Q_STRIDE,
+// X17_KV_STRIDE, X17_O_STRIDE, X17_STRICT_MATH.
+//
+// Extension over the reference ABI: gridDim.z = number of independent sequences stacked along
+// the rows of q / kv / out (each `seq_len` rows, own causal origin); L is [H, gridDim.z * seq_len].
+
+#include "common.h"
+#include "x17_device.h"
+#include "attn_tile.h"
+
+using namespace x17;
+namespace at = x17::attn_tile;
+
+namespace {
+
+constexpr u32 HD = X17_HEAD_DIM;
+constexpr u32 N_HEADS = X17_N_HEADS;
+constexpr u32 Q_STRIDE = X17_Q_STRIDE;
+constexpr u32 KV_STRIDE = X17_KV_STRIDE;
+constexpr u32 O_STRIDE = X17_O_STRIDE;
+constexpr u32 HPK = at::HEADS_PER_KERNEL;
+constexpr u32 K_SLICES = HD / 32;      // 32 bytes of head_dim per QK MFMA
+constexpr u32 D_BLOCKS = HD / 32;      // 32 output dims per PV MFMA
+constexpr u32 CPR = HD / 16;           // 16-byte chunks per key row
+constexpr bool STRICT = X17_STRICT_MATH != 0;
+
+static_assert(HD == 32 || HD == 64 || HD == 128, "head_dim must be 32, 64 or 128");
+static_assert(N_HEADS % HPK == 0, "n_heads must be divisible by heads_per_kernel");
+
+constexpr f32 PROB_SCALE = 255.0f;                                  // cuda/attn_fwd_i8.cuh:206
+constexpr f32 BASE_TEMPERATURE = f32(constexpr_inv_sqrt(f64(HD)) / 64.0);   // :47, :447-449
+
+typedef short v4s __attribute__((ext_vector_type(4)));
+
+// value of lane ^ 32
+X17_DEV f32 partner_f32(f32 x, u32 half) {
+	u32 u = f2u(x);
+	auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+	return u2f(half == 0 ? r[1] : r[0]);
+}
+X17_DEV i32 partner_i32(i32 x, u32 half) {
+	auto r = __builtin_amdgcn_permlane32_swap((u32)x, (u32)x, false, false);
+	return (i32)(half == 0 ? r[1] : r[0]);
+}
+
+// K tile: linear 16-byte chunk n = key * CPR + c lives in 128-byte line n / 8 at position
+// (n % 8) ^ (line & 7), which keeps ds_read_b128 of 8 consecutive keys conflict-free for every
+// supported head_dim.
+X17_DEV u32 k_chunk_offset(u32 key, u32 c) {
+	u32 n = key * CPR + c;
+	u32 line = n >> 3;
+	return (line << 7) | (((n & 7) ^ (line & 7)) << 4);
+}
+
+// V tile (bf16): linear 32-byte granule n = key * CPR + c (16 dims) lives in 256-byte line n / 8
+// at position (n % 8) ^ (line & 7).
+X17_DEV u32 v_granule_offset(u32 key, u32 c) {
+	u32 n = key * CPR + c;
+	u32 line = n >> 3;
+	return (line << 8) | (((n & 7) ^ (line & 7)) << 5);
+}
+
+X17_DEV u32 pack_bf16(f32 lo, f32 hi) {
+	// both values are exactly representable in bf16: keep the upper halves
+	return __builtin_amdgcn_perm(f2u(hi), f2u(lo), 0x07060302u);
+}
+
+} // namespace
+
+extern "C" __global__ __launch_bounds__(at::THREADS_PER_BLOCK)
+void kernel(
+	u32 seq_len,
+	i8 const *q,
+	i8 const *kv,
+	i8 const *sink_k,
+	i8 const *sink_v,
+	f32 const *attn_temperature,
+	i8 *out,
+	f32 *l_out,
+	u32 window_size
+) {
+	extern __shared__ __attribute__((aligned(1024))) u8 smem[];
+
+	u32 const tid = threadIdx.x;
+	u32 const lane = tid % 64;
+	u32 const wave = __builtin_amdgcn_readfirstlane(tid / 64);
+	u32 const half = lane / 32;
+	u32 const qlane = lane % 32;
+
+	u32 const seq = blockIdx.z;
+	size_t const row_base = (size_t)seq * seq_len;          // first row of this sequence
+	u32 const q_block0 = blockIdx.x * at::Q_PER_BLOCK;      // position of the block's first query
+	u32 const q_wave0 = q_block0 + wave * at::Q_PER_WAVE;
+	u32 const qi = q_wave0 + qlane;                         // this lane's query position
+
+	// cuda/attn_fwd_i8.cuh:408-412 -- window 0 means "no window"; otherwise rounded up to 16
+	u32 const wr = window_size == 0 ? 0xFFFFFFFFu : ((window_size - 1) / 16 + 1) * 16;
+
+	// key blocks (32 keys) the workgroup walks, and the sub-range this wave needs
+	u32 const kb_begin = (q_block0 - (q_block0 < wr ? q_block0 : wr)) / at::KV_PER_STEP;
+	u32 const kb_end = q_block0 / at::KV_PER_STEP + at::Q_WAVES;             // exclusive
+	u32 const wave_kb_first = (q_wave0 - (q_wave0 < wr ? q_wave0 : wr)) / at::KV_PER_STEP;
+	u32 const wave_kb_last = q_wave0 / at::KV_PER_STEP;                      // inclusive
+
+	for (u32 hh = 0; hh < HPK; ++hh) {
+		u32 const head = blockIdx.y * HPK + hh;
+		i8 const *q_head = q + row_base * Q_STRIDE + (size_t)head * HD;
+		i8 const *kv_head = kv + row_base * KV_STRIDE + (size_t)head * 2 * HD;
+
+		// ---- staging helpers for one 32-key block
+		auto issue_k_load = [&](u32 kb, u32 stage) {
+			if (tid < 32 * CPR) {
+				// lane `tid` fills stored chunk `tid` of the K tile; find which logical chunk lives there
+				u32 line = tid >> 3;
+				u32 n = (line << 3) | ((tid & 7) ^ (line & 7));
+				u32 key = n / CPR, c = n % CPR;
+				i8 const *src = kv_head + (size_t)(kb * at::KV_PER_STEP + key) * KV_STRIDE + c * 16;
+				u8 *dst = smem + stage * at::STAGE_BYTES + (tid / 64) * 1024;
+				__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(src), X17_LDS_PTR(dst), 16, 0, 0);
+			}
+		};
+		auto load_v = [&](u32 kb) -> v4i {
+			v4i v = {0, 0, 0, 0};
+			if (tid < 32 * CPR) {
+				u32 key = tid / CPR, c = tid % CPR;
+				v = *reinterpret_cast<v4i const *>(kv_head + (size_t)(kb * at::KV_PER_STEP + key) * KV_STRIDE + HD + c * 16);
+			}
+			return v;
+		};
+		auto store_v = [&](v4i raw, u32 stage) {
+			if (tid < 32 * CPR) {
+				u32 key = tid / CPR, c = tid % CPR;
+				u32 w[8];
+				X17_UNROLL for (int i = 0; i < 8; ++i) {
+					u32 word = (u32)raw[i / 2];
+					u32 b0 = (word >> (16 * (i % 2))) & 0xFFu;
+					u32 b1 = (word >> (16 * (i % 2) + 8)) & 0xFFu;
+					w[i] = (f2u(f32((i32)(i8)b0)) >> 16) | (f2u(f32((i32)(i8)b1)) & 0xFFFF0000u);
+				}
+				u8 *dst = smem + stage * at::STAGE_BYTES + at::K_TILE_BYTES + v_granule_offset(key, c);
+				*reinterpret_cast<v4u *>(dst) = v4u{w[0], w[1], w[2], w[3]};
+				*reinterpret_cast<v4u *>(dst + 16) = v4u{w[4], w[5], w[6], w[7]};
+			}
+		};
+
+		// ---- per-query setup (cuda/attn_fwd_i8.cuh:444-517)
+		v4i qf[K_SLICES];
+		X17_UNROLL for (u32 s = 0; s < K_SLICES; ++s) {
+			qf[s] = *reinterpret_cast<v4i const *>(q_head + (size_t)qi * Q_STRIDE + 32 * s + 16 * half);
+		}
+		u32 const visible = qi < wr ? qi : wr;
+		f32 temperature = BASE_TEMPERATURE * strict::lg2(f32(visible + 4u));
+		temperature = temperature * attn_temperature[head];
+
+		i32 sink_dot = 0;
+		X17_UNROLL for (u32 s = 0; s < K_SLICES; ++s) {
+			v4i sk = *reinterpret_cast<v4i const *>(sink_k + (size_t)head * HD + 32 * s + 16 * half);
+			X17_UNROLL for (int w = 0; w < 4; ++w) sink_dot = __builtin_amdgcn_sdot4(qf[s][w], sk[w], sink_dot, false);
+		}
+		sink_dot += partner_i32(sink_dot, half);
+
+		f32 m = f32(sink_dot) * temperature;
+		f32 sum_lo = 0.25f * PROB_SCALE;     // partial sum of key quad `half` of every tile
+		f32 sum_hi = 0.25f * PROB_SCALE;     // partial sum of key quad `2 + half`
+		// (the lane pair holds the reference's four partial sums two-and-two; each starts at 63.75)
+		v16f o_acc[D_BLOCKS];                // O^T: lane = query, register r = dim 32*db + 8*(r/4) + 4*half + r%4
+		X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
+			X17_UNROLL for (int r4 = 0; r4 < 4; ++r4) {
+				u32 word = *reinterpret_cast<u32 const *>(sink_v + (size_t)head * HD + 32 * db + 8 * r4 + 4 * half);
+				X17_UNROLL for (int b = 0; b < 4; ++b) {
+					o_acc[db][4 * r4 + b] = f32((i32)(i8)((word >> (8 * b)) & 0xFFu) * 255);
+				}
+			}
+		}
+
+		// ---- pipeline prologue
+		__syncthreads();                      // previous head's tiles are no longer read
+		issue_k_load(kb_begin, 0);
+		store_v(load_v(kb_begin), 0);
+
+		for (u32 kb = kb_begin; kb < kb_end; ++kb) {
+			u32 const stage = (kb - kb_begin) % at::STAGES;
+			__builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): this block's K tile has landed
+			__syncthreads();
+			v4i v_next = {0, 0, 0, 0};
+			bool const has_next = kb + 1 < kb_end;
+			if (has_next) {
+				issue_k_load(kb + 1, stage ^ 1);
+				v_next = load_v(kb + 1);
+			}
+
+			if (kb >= wave_kb_first && kb <= wave_kb_last) {
+				u8 const *k_tile = smem + stage * at::STAGE_BYTES;
+				u8 const *v_tile = k_tile + at::K_TILE_BYTES;
+
+				// S^T block: rows = 32 keys, columns = this wave's 32 queries
+				v16i s_acc = {0};
+				X17_UNROLL for (u32 s = 0; s < K_SLICES; ++s) {
+					v4i kf = *reinterpret_cast<v4i const *>(k_tile + k_chunk_offset(qlane, 2 * s + half));
+					s_acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[s], s_acc, 0, 0, 0);
+				}
+
+				u32 const key0 = kb * at::KV_PER_STEP;
+				// fully visible for all 32 queries of the wave?  (cuda/attn_fwd_i8.cuh:540-567)
+				bool const need_mask = !(key0 + 31 < q_wave0 && (q_wave0 + 31 - key0) <= wr);
+
+				X17_UNROLL for (u32 tile = 0; tile < 2; ++tile) {
+					f32 s[8];
+					X17_UNROLL for (u32 r = 0; r < 8; ++r) s[r] = f32(s_acc[8 * tile + r]) * temperature;
+					if (need_mask) {
+						X17_UNROLL for (u32 r = 0; r < 8; ++r) {
+							u32 j = key0 + 16 * tile + 8 * (r / 4) + 4 * half + (r % 4);
+							bool vis = j < qi && (qi - j) <= wr;
+							s[r] = vis ? s[r] : -__builtin_inff();
+						}
+					}
+					f32 lmax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fmaxf(s[0], s[1]), __builtin_fmaxf(s[2], s[3])),
+					                           __builtin_fmaxf(__builtin_fmaxf(s[4], s[5]), __builtin_fmaxf(s[6], s[7])));
+					f32 tmax = __builtin_fmaxf(lmax, partner_f32(lmax, half));
+
+					// cuda/attn_fwd_i8.cuh:233-256 -- rescale only when some row's max grew
+					f32 resc = 1.0f;
+					if (__any(tmax > m)) {
+						f32 new_m = __builtin_fmaxf(tmax, m);
+						resc = sfu::ex2(m - new_m);      // exactly 1 for rows whose max did not move
+						m = new_m;
+						X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
+							X17_UNROLL for (int r = 0; r < 16; ++r) o_acc[db][r] = o_acc[db][r] * resc;
+						}
+					}
+
+					// :265-290 -- p = ex2(s - max) * 255; partial sums over key quads; P = rne(p)
+					f32 p[8];
+					X17_UNROLL for (u32 r = 0; r < 8; ++r) p[r] = sfu::ex2(s[r] - m) * PROB_SCALE;
+					f32 add_lo = (p[0] + p[1]) + (p[2] + p[3]);
+					f32 add_hi = (p[4] + p[5]) + (p[6] + p[7]);
+					sum_lo = fmaf32(sum_lo, resc, add_lo);
+					sum_hi = fmaf32(sum_hi, resc, add_hi);
+
+					v4u pp;
+					X17_UNROLL for (int w = 0; w < 4; ++w) {
+						pp[w] = pack_bf16(__builtin_rintf(p[2 * w]), __builtin_rintf(p[2 * w + 1]));
+					}
+					v8bf const pfrag = __builtin_bit_cast(v8bf, pp);
+
+					// :588-605 -- O += f32(P . V) for this 16-key tile
+					X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
+						// V^T operand: lane = dim 32*db + lane%32, slots = keys 16*tile + {4*half..+3, 8+4*half..+3}
+						u32 t = lane % 16;
+						u32 dh = (lane / 16) % 2;
+						v4s lo4, hi4;
+						{
+							u32 key = 16 * tile + 4 * half + (t >> 2);
+							u8 const *p0 = v_tile + v_granule_offset(key, 2 * db + dh) + 8 * (t & 3);
+							u8 const *p1 = v_tile + v_granule_offset(key + 8, 2 * db + dh) + 8 * (t & 3);
+							lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3))) *)p0);
+							hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3))) *)p1);
+						}
+						typedef short v8s __attribute__((ext_vector_type(8)));
+						v8s both = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+						v8bf const vfrag = __builtin_bit_cast(v8bf, both);
+						if constexpr (STRICT) {
+							v16f zero = {0};
+							v16f pv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfrag, pfrag, zero, 0, 0, 0);
+							X17_UNROLL for (int r = 0; r < 16; ++r) o_acc[db][r] = o_acc[db][r] + pv[r];
+						} else {
+							o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfrag, pfrag, o_acc[db], 0, 0, 0);
+						}
+					}
+				}
+			}
+
+			if (has_next) {
+				store_v(v_next, stage ^ 1);
+			}
+		}
+
+		// ---- finish (cuda/attn_fwd_i8.cuh:293-351): the lane pair holds partial sums (s0, s2) and (s1, s3)
+		f32 other_lo = partner_f32(sum_lo, half);
+		f32 other_hi = partner_f32(sum_hi, half);
+		f32 s0 = half == 0 ? sum_lo : other_lo;
+		f32 s1 = half == 0 ? other_lo : sum_lo;
+		f32 s2 = half == 0 ? sum_hi : other_hi;
+		f32 s3 = half == 0 ? other_hi : sum_hi;
+		f32 total = (s0 + s1) + (s2 + s3);
+		if (l_out != nullptr && half == 0) {
+			l_out[(size_t)head * ((size_t)gridDim.z * seq_len) + row_base + qi] = strict::lg2(total) + m;
+		}
+		f32 inv = strict::rcp(total);
+		i8 *o_row = out + (row_base + qi) * O_STRIDE + (size_t)head * HD;
+		X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
+			X17_UNROLL for (int r4 = 0; r4 < 4; ++r4) {
+				u32 word = 0;
+				X17_UNROLL for (int b = 0; b < 4; ++b) {
+					word |= ((u32)f32_to_fixedi8(o_acc[db][4 * r4 + b] * inv) & 0xFFu) << (8 * b);
+				}
+				*reinterpret_cast<u32 *>(o_row + 32 * db + 8 * r4 + 4 * half) = word;
+			}
+		}
+	}
+}

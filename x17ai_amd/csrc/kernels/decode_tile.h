@@ -1,0 +1,20 @@
+// decode_tile.h -- launch geometry of the single-token decode kernel (shared with its meta program).
+// Needs X17_HEAD_DIM and X17_CACHE_CAPACITY from common.h.
+#pragma once
+
+namespace x17 { namespace decode_tile {
+
+constexpr unsigned HEAD_DIM = X17_HEAD_DIM;
+constexpr unsigned CAPACITY = X17_CACHE_CAPACITY;       // cache rows per sequence, multiple of 16
+constexpr unsigned THREADS_PER_BLOCK = 256;
+constexpr unsigned HEADS_PER_BLOCK = 1;
+constexpr unsigned MAX_TILES = CAPACITY / 16;           // 16-key tiles
+constexpr unsigned CHUNK_TILES = 32;                    // tiles whose P.V partials are staged at once
+
+// LDS: scores f32[CAPACITY] | probabilities u8[CAPACITY] | quad sums f32[CAPACITY/4]
+//      | per tile: max, running max, rescale f32[3 * MAX_TILES] | block maxima f32[256]
+//      | P.V partials i32[CHUNK_TILES * HEAD_DIM] | final partial sums f32[4]
+constexpr unsigned SMEM_BYTES =
+	CAPACITY * 4 + CAPACITY + CAPACITY + 3 * MAX_TILES * 4 + 256 * 4 + CHUNK_TILES * HEAD_DIM * 4 + 16;
+
+}} // namespace x17::decode_tile

@@ -305,15 +305,30 @@ void kernel(
 		u8 const *w_tile = smem + (ks % gt::STAGES) * STAGE_BYTES + X_TILE_BYTES + wn * 128 * ROW_BYTES + lo.frag_row;
 
 		if constexpr (MMA == 0) {
-			X17_UNROLL for (u32 s = 0; s < 4; ++s) {            // 32 bytes of K per MFMA
-				v4i wf[4], xf[4];
-				u32 kc = 2 * s + lo.half;
-				X17_UNROLL for (int bn = 0; bn < 4; ++bn) wf[bn] = lds_chunk(w_tile, bn * 32 * ROW_BYTES, kc, lo.swz);
-				X17_UNROLL for (int bm = 0; bm < 4; ++bm) xf[bm] = lds_chunk(x_tile, bm * 32 * ROW_BYTES, kc, lo.swz);
+			// 32 bytes of K per MFMA; operand fragments of slice s+1 are fetched before the
+			// MFMAs of slice s are issued, so LDS latency hides under matrix-core time
+			v4i wf[2][4], xf[2][4];
+			X17_UNROLL for (int bn = 0; bn < 4; ++bn) wf[0][bn] = lds_chunk(w_tile, bn * 32 * ROW_BYTES, lo.half, lo.swz);
+			X17_UNROLL for (int bm = 0; bm < 4; ++bm) xf[0][bm] = lds_chunk(x_tile, bm * 32 * ROW_BYTES, lo.half, lo.swz);
+			X17_UNROLL for (u32 s = 0; s < 4; ++s) {
+				if (s + 1 < 4) {
+					u32 kc = 2 * (s + 1) + lo.half;
+					X17_UNROLL for (int bn = 0; bn < 4; ++bn) wf[(s + 1) & 1][bn] = lds_chunk(w_tile, bn * 32 * ROW_BYTES, kc, lo.swz);
+					X17_UNROLL for (int bm = 0; bm < 4; ++bm) xf[(s + 1) & 1][bm] = lds_chunk(x_tile, bm * 32 * ROW_BYTES, kc, lo.swz);
+				}
 				X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
 					X17_UNROLL for (int bm = 0; bm < 4; ++bm) {
-						acc[bn][bm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[bn], xf[bm], acc[bn][bm], 0, 0, 0);
+						acc[bn][bm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[s & 1][bn], xf[s & 1][bm], acc[bn][bm], 0, 0, 0);
 					}
+				}
+				// pin the issue order: two MFMAs, then one of the eight LDS reads of the next slice
+				if (s + 1 < 4) {
+					X17_UNROLL for (int i = 0; i < 8; ++i) {
+						__builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+						__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+					}
+				} else {
+					__builtin_amdgcn_sched_group_barrier(0x008, 16, 0);
 				}
 			}
 		} else if constexpr (MMA == 1) {
@@ -369,9 +384,11 @@ void kernel(
 		u32 row = row0 + 32 * bm;
 		f32 x[64];
 		X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
+			// (bit-casting a single vector element in place reads element 0; cast the whole vector first)
+			v16f const as_f32 = __builtin_bit_cast(v16f, acc[bn][bm]);
 			X17_UNROLL for (int r = 0; r < 16; ++r) {
 				if constexpr (ACC_F32) {
-					x[16 * bn + r] = __builtin_bit_cast(f32, acc[bn][bm][r]);
+					x[16 * bn + r] = as_f32[r];
 				} else {
 					x[16 * bn + r] = f32(acc[bn][bm][r]);
 				}

@@ -1,0 +1,97 @@
+"""Compiles, without a GPU, every code object the tests, the smoke check and the benchmark ask for.
+
+The operator layer builds kernels on demand (one code object per configuration, cached by
+content hash); a machine that runs the tests should find all of them already built.
+"""
+from __future__ import annotations
+
+import concurrent.futures
+import os
+import subprocess
+
+from . import recipes
+from .api import E4M3, INT8, BF16, GemmConfig, GemmInputConfig, GemmKernel, ScaleConfig
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+TEST_SHAPES = [(256, 128, 256), (512, 1024, 512), (256, 2048, 1024)]
+
+
+def _specs():
+	s = []
+	add = s.append
+	# ---- tests/test_gpu_gemm.py
+	for _, k, n in TEST_SHAPES:
+		add(("attn_q", k, n))
+		for store in (E4M3, INT8):
+			for strict in (True, False):
+				add(("ffn_f", k, n, strict, store))
+				add(("attn_y", n // 2, k, strict, store))
+	add(("acc_probe",))
+	for hd in (32, 64, 128):
+		for k in (512, 2048):
+			add(("attn_kv", k, 512, hd))
+	for k, n in ((512, 256), (2048, 512)):
+		add(("ffn_y", n // 2, k, True, E4M3, INT8))
+	for k, n in ((512, 256), (4096, 512)):
+		add(("ffn_f_f8", k, n, True))
+	# ---- tests/test_gpu_attn.py
+	for h, hd in ((4, 32), (2, 64), (2, 128), (8, 64)):
+		add(("attn", h, hd, True))
+	for h, hd in ((2, 64), (2, 128), (8, 64)):
+		add(("attn", h, hd, False))
+	for h, hd, cap in ((4, 32, 256), (4, 64, 256), (2, 128, 512)):
+		add(("decode", h, hd, cap, True))
+	for d in (512, 2048, 4096):
+		add(("rms_norm", d, E4M3))
+		add(("rms_norm", d, BF16))
+	return s
+
+
+def _build_one(spec) -> str:
+	kind = spec[0]
+	if kind == "attn_q":
+		return recipes.attn_q_kernel(None, spec[1], spec[2]).name
+	if kind == "ffn_f":
+		return recipes.ffn_f_kernel(None, spec[1], spec[2], spec[3], spec[4]).name
+	if kind == "attn_y":
+		return recipes.attn_y_kernel(None, spec[1], spec[2], spec[3], spec[4]).name
+	if kind == "attn_kv":
+		return recipes.attn_kv_kernel(None, spec[1], spec[2], spec[3]).name
+	if kind == "ffn_y":
+		return recipes.ffn_y_kernel(None, spec[1], spec[2], spec[3], spec[4], spec[5]).name
+	if kind == "ffn_f_f8":
+		return recipes.ffn_f_f8_kernel(None, spec[1], spec[2], spec[3]).name
+	if kind == "attn":
+		return recipes.attn_kernel(None, spec[1], spec[2], spec[3]).name
+	if kind == "decode":
+		return recipes.attn_decode_kernel(None, spec[1], spec[2], spec[3], spec[4]).name
+	if kind == "rms_norm":
+		return recipes.rms_norm_kernel(None, spec[1], spec[2]).name
+	if kind == "acc_probe":
+		k, n = 1024, 256
+		cfg = GemmConfig(GemmInputConfig(INT8, k, None, False), GemmInputConfig(INT8, k, n, True), INT8)
+		GemmKernel(None, f"acc_probe-k{k}-n{n}", cfg, ScaleConfig(1.0, 1.0))
+		return GemmKernel(None, f"acc_probe2-k{k}-n{n}", cfg, ScaleConfig(1.0 / (k * 127.0), 1.0)).name
+	raise ValueError(spec)
+
+
+def build_host_libraries() -> None:
+	subprocess.run(["make", "-C", os.path.join(_HERE, "csrc"), "-j4"], check=True, stdout=subprocess.DEVNULL)
+
+
+def build_all(workers: int = 8) -> list:
+	build_host_libraries()
+	specs = _specs()
+	names = []
+	with concurrent.futures.ThreadPoolExecutor(max_workers=workers) as pool:
+		for name in pool.map(_build_one, specs):
+			names.append(name)
+	return names
+
+
+if __name__ == "__main__":
+	import time
+	t0 = time.time()
+	built = build_all()
+	print(f"built {len(built)} kernels in {time.time() - t0:.1f}s")

@@ -1,0 +1,108 @@
+"""The block's kernels with the reference's scale recipes (src/main.rs:387-675).
+
+Each function mirrors one create_*_kernel of the reference's block driver: same operand
+dtypes, same epilogue, same scale expressions.  Kernel names carry the shape so that
+several configurations can live side by side in the kernel cache.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+from .api import (
+	E4M3, INT8,
+	AttnDecodeKernel, AttnKernel, AttnKernelConfig, Device, GeGluConfig, GemmConfig, GemmInputConfig, GemmKernel,
+	ResidualConfig, RMSNormConfig, RmsNormKernel, ScaleConfig,
+)
+
+FIXED_I8_SCALE = 8.0                     # src/main.rs:33
+L2_NORM_EPS = 1.0 / 2.0 ** 70            # src/main.rs:35
+# src/main.rs:650 == cuda/utils_core.cuh:414-418
+GELU_VAR_FIX_2 = 1.0 / ((1.0 / 3.0) + (0.5 / math.pi) * (1.0 / math.sqrt(3.0)))
+
+
+def _inv_sqrt(x: float) -> float:       # src/util.rs:20-24
+	return 1.0 / math.sqrt(x)
+
+
+def _mode(strict: bool) -> str:
+	return "strict" if strict else "fast"
+
+
+def _gemm(a_dtype, b_dtype, c_dtype, k, n_raw):
+	return GemmConfig(GemmInputConfig(a_dtype, k, None, False), GemmInputConfig(b_dtype, k, n_raw, True), c_dtype)
+
+
+def attn_q_kernel(device: Optional[Device], model_dim: int, q_proj_outputs: int, strict: bool = True) -> GemmKernel:
+	"""src/main.rs:387-438 -- x[i8] . Wq[i8]^T with the Scale epilogue -> q[i8]."""
+	cfg = ScaleConfig(_inv_sqrt(model_dim) / (FIXED_I8_SCALE * FIXED_I8_SCALE), FIXED_I8_SCALE)
+	return GemmKernel(device, f"attn_q_fwd-k{model_dim}-n{q_proj_outputs}-{_mode(strict)}",
+	                  _gemm(INT8, INT8, INT8, model_dim, q_proj_outputs), cfg, strict)
+
+
+def attn_kv_kernel(device: Optional[Device], model_dim: int, kv_proj_outputs: int, head_dim: int,
+                   strict: bool = True) -> GemmKernel:
+	"""src/main.rs:440-493 -- x . Wkv^T with the L2-norm (RMSNorm) epilogue -> kv[i8], rrms[f32]."""
+	cfg = RMSNormConfig(L2_NORM_EPS, head_dim, head_dim,
+	                    _inv_sqrt(model_dim) / (FIXED_I8_SCALE * FIXED_I8_SCALE), FIXED_I8_SCALE)
+	return GemmKernel(device, f"attn_kv_fwd-k{model_dim}-n{kv_proj_outputs}-hd{head_dim}-{_mode(strict)}",
+	                  _gemm(INT8, INT8, INT8, model_dim, kv_proj_outputs), cfg, strict)
+
+
+def attn_kernel(device: Optional[Device], n_heads: int, head_dim: int, strict: bool = True) -> AttnKernel:
+	"""src/main.rs:495-523 -- int8 sliding-window attention; strides are the dense widths."""
+	width = n_heads * head_dim
+	cfg = AttnKernelConfig(INT8, n_heads, head_dim, width, 2 * width, width)
+	return AttnKernel(device, f"attn_fwd_i8-h{n_heads}-hd{head_dim}-{_mode(strict)}", cfg, strict)
+
+
+def attn_y_kernel(device: Optional[Device], model_dim: int, attn_width: int, strict: bool = True,
+                  c_dtype: int = E4M3) -> GemmKernel:
+	"""src/main.rs:525-576 -- attn_out[i8] . Wy[i8]^T with the gated-residual epilogue -> e4m3."""
+	cfg = ResidualConfig(_inv_sqrt(attn_width) / (FIXED_I8_SCALE * FIXED_I8_SCALE), 1.0)
+	return GemmKernel(device, f"attn_y_fwd-k{attn_width}-n{2 * model_dim}-c{c_dtype}-{_mode(strict)}",
+	                  _gemm(INT8, INT8, c_dtype, attn_width, 2 * model_dim), cfg, strict)
+
+
+def ffn_f_kernel(device: Optional[Device], model_dim: int, ffn_f_proj_outputs: int, strict: bool = True,
+                 c_dtype: int = E4M3) -> GemmKernel:
+	"""src/main.rs:578-627 -- x[i8] . Wf[i8]^T with the GeGLU epilogue -> f[e4m3].
+	c_dtype=INT8 emits f as FixedI8 instead (out_scale 8), the operand of an int8 ffn_y."""
+	out_scale = 1.0 if c_dtype == E4M3 else FIXED_I8_SCALE
+	cfg = GeGluConfig(_inv_sqrt(model_dim) / (FIXED_I8_SCALE * FIXED_I8_SCALE), out_scale)
+	return GemmKernel(device, f"ffn_f_fwd-k{model_dim}-n{ffn_f_proj_outputs}-c{c_dtype}-{_mode(strict)}",
+	                  _gemm(INT8, INT8, c_dtype, model_dim, ffn_f_proj_outputs), cfg, strict)
+
+
+def ffn_y_kernel(device: Optional[Device], model_dim: int, f_width: int, strict: bool = True,
+                 a_dtype: int = E4M3, b_dtype: int = INT8) -> GemmKernel:
+	"""src/main.rs:629-678 -- f . Wy^T with the gated-residual epilogue -> e4m3.
+	a_dtype=E4M3, b_dtype=INT8 is the reference's ffn_y_fwd_f8; INT8 x INT8 is the int8 variant
+	(f in FixedI8 carries one more factor 8); E4M3 x E4M3 is the all-fp8 variant."""
+	inp = math.sqrt(GELU_VAR_FIX_2 / f_width)
+	if a_dtype == INT8:
+		inp /= FIXED_I8_SCALE
+	if b_dtype == INT8:
+		inp /= FIXED_I8_SCALE
+	cfg = ResidualConfig(inp, 1.0)
+	return GemmKernel(device, f"ffn_y_fwd-a{a_dtype}b{b_dtype}-k{f_width}-n{2 * model_dim}-{_mode(strict)}",
+	                  _gemm(a_dtype, b_dtype, E4M3, f_width, 2 * model_dim), cfg, strict)
+
+
+def ffn_f_f8_kernel(device: Optional[Device], model_dim: int, ffn_f_proj_outputs: int, strict: bool = True) -> GemmKernel:
+	"""All-fp8 ffn_f: x[e4m3] . Wf[e4m3]^T, f32 accumulate, GeGLU -> e4m3.  Operands are real values
+	(no FixedI8 factor), so only the 1/sqrt(K) variance fix remains in inp_scale."""
+	cfg = GeGluConfig(_inv_sqrt(model_dim), 1.0)
+	return GemmKernel(device, f"ffn_f_fwd_f8-k{model_dim}-n{ffn_f_proj_outputs}-{_mode(strict)}",
+	                  _gemm(E4M3, E4M3, E4M3, model_dim, ffn_f_proj_outputs), cfg, strict)
+
+
+def rms_norm_kernel(device: Optional[Device], model_dim: int, in_dtype: int = E4M3, eps: float = L2_NORM_EPS) -> RmsNormKernel:
+	"""rms_norm.cu:55-113."""
+	return RmsNormKernel(device, f"rms_norm-d{model_dim}-in{in_dtype}", in_dtype, model_dim, eps)
+
+
+def attn_decode_kernel(device: Optional[Device], n_heads: int, head_dim: int, cache_capacity: int,
+                       strict: bool = True) -> AttnDecodeKernel:
+	return AttnDecodeKernel(device, f"attn_decode_i8-h{n_heads}-hd{head_dim}-cap{cache_capacity}-{_mode(strict)}",
+	                        n_heads, head_dim, cache_capacity, strict)
