@@ -1,0 +1,152 @@
+"""Host-side checks that need no GPU: the two shared libraries load and export exactly what
+include/*.h declares, errors travel as diagnostics (never exceptions or aborts), kernel
+configurations are validated as the reference validates them, and the kernel cache works."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+import x17ai_amd as X
+from x17ai_amd import _ffi, recipes
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared(header):
+	text = open(os.path.join(ROOT, "include", header)).read()
+	text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+	return sorted(set(re.findall(r"\b(x17(?:ai|h)_[a-z0-9_]+)\s*\(", text)))
+
+
+def _exported(lib):
+	out = subprocess.run(["nm", "-D", "--defined-only", lib], check=True, capture_output=True, text=True).stdout
+	return sorted(set(l.split()[-1] for l in out.splitlines() if " T " in l))
+
+
+def test_shim_exports_exactly_the_declared_entry_points():
+	declared = _declared("x17ai_hip_shim.h")
+	assert len(declared) == 21              # the reference's FFI surface, src/device/cuda/cuda_shim.rs:76-158
+	exported = [s for s in _exported(_ffi.lib_paths()["shim"]) if s.startswith("x17ai_")]
+	assert exported == declared
+
+
+def test_host_library_exports_every_declared_entry_point():
+	declared = _declared("x17ai_host.h")
+	exported = set(_exported(_ffi.lib_paths()["host"]))
+	assert declared and not [s for s in declared if s not in exported]
+
+
+def test_struct_layouts_match_the_reference_ffi():
+	# CudaKernelAttrs: nine int32 (cuda_shim.rs:51-63); PtrResult: two pointers (cuda_shim.rs:70-74)
+	src = open(os.path.join(ROOT, "include", "x17ai_hip_shim.h")).read()
+	body = src[src.index("typedef struct X17HipKernelAttrs {"):src.index("} X17HipKernelAttrs;")]
+	assert len(re.findall(r"int32_t\s+\w+;", body)) == 9
+	prog = r'''
+	#include "x17ai_hip_shim.h"
+	#include <stdio.h>
+	int main(void) { printf("%zu %zu %zu %zu\n", sizeof(X17HipKernelAttrs), sizeof(X17StreamResult), sizeof(X17FfiBuffer), sizeof(X17FfiSpan)); return 0; }
+	'''
+	exe = os.path.join(ROOT, "_work", "layout_probe")
+	os.makedirs(os.path.dirname(exe), exist_ok=True)
+	subprocess.run(["gcc", "-x", "c", "-", "-I", os.path.join(ROOT, "include"), "-o", exe], input=prog, text=True, check=True)
+	assert subprocess.run([exe], capture_output=True, text=True, check=True).stdout.split() == ["36", "16", "16", "16"]
+
+
+def test_errors_are_diagnostics_not_crashes():
+	"""Without a GPU (or with a bad ordinal) opening a device fails with the shim's message, moved
+	through x17ai_move_diagnostic into the caller's buffer (cpp/ffi.hpp:84-175)."""
+	with pytest.raises(X.X17Error, match=r"x17ai_hip_open_context\(\)"):
+		X.Device(10 ** 6)
+	# a NULL diagnostic is a no-op; handing one to move_diagnostic must not crash
+	shim = ctypes.CDLL(_ffi.lib_paths()["shim"])
+
+	class Buf(ctypes.Structure):
+		_fields_ = [("instance", ctypes.c_void_p), ("vmt", ctypes.c_void_p)]
+	shim.x17ai_move_diagnostic.argtypes = [ctypes.c_void_p, Buf]
+	shim.x17ai_move_diagnostic.restype = None
+	shim.x17ai_move_diagnostic(None, Buf(None, None))
+
+
+def _gemm(a, b, c, k=256, n=256, trans_a=False, trans_b=True, rows=True):
+	return X.GemmConfig(X.GemmInputConfig(a, k, None, trans_a), X.GemmInputConfig(b, k, n if rows else None, trans_b), c)
+
+
+@pytest.mark.parametrize("cfg,epi,msg", [
+	(_gemm(X.INT8, X.INT8, X.INT8, trans_a=True), X.ScaleConfig(1.0, 1.0), "transposed GEMM input A"),
+	(_gemm(X.INT8, X.INT8, X.INT8, trans_b=False), X.ScaleConfig(1.0, 1.0), "non-transposed GEMM input B"),
+	(_gemm(X.INT8, X.INT8, X.INT8, rows=False), X.ScaleConfig(1.0, 1.0), "runtime column count"),
+	(_gemm(X.INT8, X.INT8, X.E4M3), X.ScaleConfig(1.0, 1.0), "Scale epilogue requires an i8 output"),
+	(_gemm(X.BF16, X.INT8, X.INT8), X.ScaleConfig(1.0, 1.0), "unsupported GEMM input dtype bf16"),
+	(_gemm(X.INT8, X.INT8, X.F32), X.GeGluConfig(1.0, 1.0), "GeGLU epilogue requires"),
+	(_gemm(X.INT8, X.INT8, X.E4M3), X.GeGluConfig(-1.0, 1.0), "invalid GeGLU scale values"),
+	(_gemm(X.INT8, X.INT8, X.E4M3), X.ResidualConfig(1.0, float("nan")), "invalid residual GEMM scale values"),
+	(_gemm(X.INT8, X.INT8, X.INT8), X.RMSNormConfig(1e-9, 48, 48, 1.0, 1.0), "multiples of 32"),
+	(_gemm(X.INT8, X.INT8, X.INT8), X.RMSNormConfig(1e-9, 32, 64, 1.0, 1.0), "head_dim == sep_dim"),
+	(_gemm(X.INT8, X.INT8, X.INT8, k=200), X.ScaleConfig(1.0, 1.0), "multiple of 128"),
+	(_gemm(X.INT8, X.INT8, X.INT8, n=192), X.ScaleConfig(1.0, 1.0), "raw output columns must be a multiple of 256"),
+])
+def test_gemm_kernel_config_validation(cfg, epi, msg):
+	with pytest.raises(X.X17Error, match=msg):
+		X.GemmKernel(None, "cpu-validation-probe", cfg, epi)
+
+
+def test_kernel_names_are_path_safe():
+	for bad in ("", ".", "..", "a/b", "a\\b"):
+		with pytest.raises(X.X17Error, match="invalid kernel name"):
+			X.GemmKernel(None, bad, _gemm(X.INT8, X.INT8, X.INT8), X.ScaleConfig(1.0, 1.0))
+
+
+def test_attention_kernel_config_validation():
+	bad = [
+		(X.AttnKernelConfig(X.E4M3, 4, 64, 256, 512, 256), "requires dtype i8"),
+		(X.AttnKernelConfig(X.INT8, 0, 64, 256, 512, 256), "n_heads > 0"),
+		(X.AttnKernelConfig(X.INT8, 4, 48, 256, 512, 256), "multiple of 32"),
+		(X.AttnKernelConfig(X.INT8, 3, 64, 192, 384, 192), "divisible by heads_per_kernel"),
+		(X.AttnKernelConfig(X.INT8, 4, 64, 128, 512, 256), "q_stride >= n_heads"),
+		(X.AttnKernelConfig(X.INT8, 4, 64, 256, 256, 256), "kv_stride >= 2"),
+	]
+	for cfg, msg in bad:
+		with pytest.raises(X.X17Error, match=msg):
+			X.AttnKernel(None, "cpu-validation-probe", cfg)
+	with pytest.raises(X.X17Error, match="multiple of 512"):
+		X.RmsNormKernel(None, "cpu-validation-probe", X.E4M3, 1000, 1e-9)
+	with pytest.raises(X.X17Error, match="multiple of 16"):
+		X.AttnDecodeKernel(None, "cpu-validation-probe", 4, 64, 100)
+
+
+def test_kernel_build_metadata_and_cache(tmp_path, monkeypatch):
+	"""The code object and meta.json are generated per configuration and reused when nothing changed
+	(the reference recompiles on every run, src/device/cuda/gemm.rs:408-416)."""
+	monkeypatch.setenv("X17AI_KERNEL_CACHE", str(tmp_path))
+	k = recipes.attn_q_kernel(None, 256, 256)
+	assert k.metadata == {"THREADS_PER_BLOCK": 256, "SMEM_BYTES": 131072, "M_PER_BLOCK": 256, "N_PER_BLOCK": 256}
+	d = tmp_path / k.name
+	assert (d / "kernel.hsaco").stat().st_size > 1000
+	text = (d / "common.h").read_text()
+	assert "#define X17_A_COLS 256" in text and "#define X17_EPILOGUE 0" in text
+	# inv_sqrt(256) / 64 printed with 17 significant digits, as gemm.rs:257-259 does
+	assert "#define X17_INP_SCALE 9.76562500000000000e-04" in text
+	stamp = (d / "kernel.hsaco").stat().st_mtime_ns
+	recipes.attn_q_kernel(None, 256, 256)
+	assert (d / "kernel.hsaco").stat().st_mtime_ns == stamp
+	with pytest.raises(X.X17Error, match="built without a device"):
+		k.launch(X.Tensor(None, (256, 256), X.INT8), X.Tensor(None, (256, 256), X.INT8), X.Tensor(None, (256, 256), X.INT8))
+	a = k  # n_ops is pure host arithmetic (gemm.rs:445-449)
+	assert a.n_ops(X.Tensor(None, (512, 256), X.INT8), X.Tensor(None, (256, 256), X.INT8)) == 2.0 * 512 * 256 * 256
+
+
+def test_cpu_tensors_round_trip():
+	import numpy as np
+	t = X.Tensor.from_numpy(None, np.arange(24, dtype=np.int8).reshape(4, 6), X.INT8)
+	assert t.download().tolist() == np.arange(24).reshape(4, 6).tolist()
+	assert t.reshape((6, 4)).shape == (6, 4)
+	with pytest.raises(X.X17Error):
+		t.reshape((5, 5))
+
+
+def test_bench_refuses_more_than_one_gpu():
+	r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+	assert r.returncode != 0 and "one GPU" in r.stderr

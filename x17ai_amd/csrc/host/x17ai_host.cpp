@@ -424,7 +424,8 @@ namespace kernel_build {
 		std::snprintf(keybuf, sizeof keybuf, "%016llx", (unsigned long long)h);
 
 		std::string have;
-		if (read_file(key_path, have) && have == keybuf && file_exists(out.code_object_path) && file_exists(out.meta_json_path)) {
+		bool const force = std::getenv("X17AI_FORCE_REBUILD") != nullptr;
+		if (!force && read_file(key_path, have) && have == keybuf && file_exists(out.code_object_path) && file_exists(out.meta_json_path)) {
 			out.cache_hit = true;
 			return out;
 		}

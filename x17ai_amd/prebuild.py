@@ -45,6 +45,24 @@ def _specs():
 	for d in (512, 2048, 4096):
 		add(("rms_norm", d, E4M3))
 		add(("rms_norm", d, BF16))
+	# ---- __graft_entry__.smoke()
+	add(("ffn_f", 512, 512, True, INT8))
+	add(("ffn_y", 512, 256, True, INT8, INT8))
+	# ---- bench.py
+	for strict in (False, True):
+		add(("ffn_f", 2048, 16384, strict, INT8))
+		add(("ffn_y", 2048, 8192, strict, INT8, INT8))
+		add(("attn", 32, 128, strict))
+		add(("decode", 32, 128, 4096, strict))
+	add(("ffn_f_f8", 4096, 32768, False))
+	add(("ffn_y", 4096, 16384, False, E4M3, E4M3))
+	add(("attn_q", 2048, 2048))
+	add(("attn_kv", 2048, 4096, 128))
+	add(("attn", 16, 128, False))
+	add(("attn_y", 2048, 2048, False, E4M3))
+	add(("ffn_f", 2048, 16384, False, E4M3))
+	add(("ffn_y", 2048, 8192, False, E4M3, INT8))
+	add(("attn", 8, 64, False))
 	return s
 
 
