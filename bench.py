@@ -37,7 +37,7 @@ PEAK_BF16_TFLOPS = 2500.0    # dense bf16
 PEAK_HBM_GBS = 8000.0        # HBM3E
 
 # HBM bytes per ffn_f launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), or None
-FFN_F_TRAFFIC_BYTES = None
+FFN_F_TRAFFIC_BYTES = int((196803 * 2.0 + 65536 * 1.0) * 1024)
 
 
 def _rand_i8(rng, shape):
@@ -276,6 +276,8 @@ def main():
 	ap.add_argument("--warmup", type=int, default=10)
 	ap.add_argument("--no-extras", action="store_true")
 	ap.add_argument("--no-cpu", action="store_true")
+	ap.add_argument("--copy-probe", action="store_true",
+	                help="only run a 1 GiB device-to-device copy kernel (calibrates the HBM traffic counters)")
 	args = ap.parse_args()
 	if args.gpus != 1:
 		print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -285,6 +287,17 @@ def main():
 	from x17ai_amd import recipes
 
 	dev = X.Device(0)
+	if args.copy_probe:
+		from x17ai_amd.api import CopyProbe
+		n = 1 << 30
+		src = X.Tensor.from_numpy(dev, np.zeros(n, np.int8), X.INT8)
+		dst = X.Tensor(dev, (n,), X.INT8)
+		probe = CopyProbe(dev)
+		for _ in range(5):
+			probe.launch(src, dst)
+		dev.synchronize()
+		print(json.dumps({"copy_probe_bytes_read": n, "copy_probe_bytes_written": n, "launches": 5}))
+		return
 	h = headline(dev, X, recipes, args.steps, args.warmup)
 	value = h["ops_per_step"] * args.steps / h["wall_s"] / 1e12
 	achieved = h["k1_ops"] / h["k1_mean_s"] / 1e12

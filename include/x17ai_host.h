@@ -120,6 +120,13 @@ int x17h_decode_kernel_launch(X17hDecodeKernel *k, X17hTensor *q, X17hTensor *ca
                               X17hTensor *sink_k, X17hTensor *sink_v, X17hTensor *attn_temperature,
                               X17hTensor *out, X17hTensor *l, size_t window_size);
 
+/* Measurement aid with no reference counterpart: a plain device-to-device copy kernel of known
+ * size, against which HBM-traffic counters are calibrated (src and dst: equal sizes, multiple of 16). */
+typedef struct X17hCopyProbe X17hCopyProbe;
+int x17h_copy_probe_new(X17hDevice *dev, X17hCopyProbe **out);
+void x17h_copy_probe_free(X17hCopyProbe *p);
+int x17h_copy_probe_launch(X17hCopyProbe *p, X17hTensor *src, X17hTensor *dst);
+
 #ifdef __cplusplus
 }
 #endif

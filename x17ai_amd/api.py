@@ -365,3 +365,23 @@ class AttnDecodeKernel:
 				self._h = ctypes.c_void_p()
 		except Exception:
 			pass
+
+
+class CopyProbe:
+	"""A plain device-to-device copy kernel of known size (measurement aid for counter calibration)."""
+
+	def __init__(self, device: Optional[Device]):
+		self.device = device
+		self._h = ctypes.c_void_p()
+		check(_ffi.host().x17h_copy_probe_new(device._h if device is not None else None, ctypes.byref(self._h)))
+
+	def launch(self, src: Tensor, dst: Tensor) -> None:
+		check(_ffi.host().x17h_copy_probe_launch(self._h, src._h, dst._h))
+
+	def __del__(self):
+		try:
+			if self._h:
+				_ffi.host().x17h_copy_probe_free(self._h)
+				self._h = ctypes.c_void_p()
+		except Exception:
+			pass

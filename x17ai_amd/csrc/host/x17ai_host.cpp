@@ -1176,4 +1176,36 @@ int x17h_decode_kernel_launch(X17hDecodeKernel *k, X17hTensor *q, X17hTensor *ca
 	return from_status(k->k->launch(a));
 }
 
+// ---- measurement aid: a plain copy kernel of known size (see kernels/copy_probe.hip)
+struct X17hCopyProbe { std::shared_ptr<HipDevice> dev; std::unique_ptr<HipKernel> k; size_t blocks; };
+
+int x17h_copy_probe_new(X17hDevice *dev, X17hCopyProbe **out) {
+	try {
+		Diagnostics diag;
+		auto built = kernel_build::build("copy_probe", "// copy probe\n", "copy_probe.hip", "copy_probe_meta.cpp", diag);
+		if (!built) return fail_diag("copy probe", diag);
+		auto meta = kernel_build::read_metadata_json(built->meta_json_path, diag);
+		if (!meta) return fail_diag("copy probe", diag);
+		auto p = std::make_unique<X17hCopyProbe>();
+		p->blocks = *kernel_build::meta_get(*meta, "BLOCKS");
+		if (dev != nullptr) {
+			p->k = kernel_build::load_kernel(*dev->dev->stream, built->code_object_path, "kernel", 0, diag);
+			if (!p->k) return fail_diag("copy probe", diag);
+			p->dev = dev->dev;
+		}
+		*out = p.release();
+		return 0;
+	} catch (std::exception const &e) { return fail(e.what()); }
+}
+void x17h_copy_probe_free(X17hCopyProbe *p) { delete p; }
+int x17h_copy_probe_launch(X17hCopyProbe *p, X17hTensor *src, X17hTensor *dst) {
+	if (!p->k) return fail("copy probe was built without a device");
+	if (src->t->bytes != dst->t->bytes || src->t->bytes % 16 != 0 || src->t->bytes / 16 > 0xFFFFFFFFull) return fail("copy probe needs equal sizes, multiple of 16 bytes");
+	void *s = src->t->ptr, *d = dst->t->ptr;
+	size_t n = src->t->bytes / 16;
+	void *args[3] = {&s, &n, &d};
+	size_t grid[3] = {p->blocks, 1, 1}, block[3] = {256, 1, 1};
+	return from_status(p->k->launch(*p->dev->stream, grid, block, 0, args));
+}
+
 } // extern "C"

@@ -63,6 +63,7 @@ def _specs():
 	add(("ffn_f", 2048, 16384, False, E4M3))
 	add(("ffn_y", 2048, 8192, False, E4M3, INT8))
 	add(("attn", 8, 64, False))
+	add(("copy_probe",))
 	return s
 
 
@@ -86,6 +87,10 @@ def _build_one(spec) -> str:
 		return recipes.attn_decode_kernel(None, spec[1], spec[2], spec[3], spec[4]).name
 	if kind == "rms_norm":
 		return recipes.rms_norm_kernel(None, spec[1], spec[2]).name
+	if kind == "copy_probe":
+		from .api import CopyProbe
+		CopyProbe(None)
+		return "copy_probe"
 	if kind == "acc_probe":
 		k, n = 1024, 256
 		cfg = GemmConfig(GemmInputConfig(INT8, k, None, False), GemmInputConfig(INT8, k, n, True), INT8)
