@@ -93,8 +93,10 @@ def test_attn_batched_sequences_and_no_l(dev):
 
 
 def test_attn_special_cases(dev):
-	"""Closed-form cases: query 0 sees only the sink; constant V gives V back; a window that covers
-	the whole sequence equals no window."""
+	"""Closed-form cases: query 0 sees only the sink; a window that covers the whole sequence equals
+	no window; constant V comes back exactly when all scores are equal (q = 0: every probability is
+	exactly 255) and within one code otherwise (the numerator sums rounded probabilities, the
+	denominator unrounded ones)."""
 	t, h, hd = 256, 2, 64
 	rng = rng_for("attn-special")
 	q, kv, sk, sv, temp = _attn_inputs(rng, t, h, hd)
@@ -106,8 +108,12 @@ def test_attn_special_cases(dev):
 	kv2 = kv.reshape(t, h, 2, hd).copy()
 	kv2[:, :, 1, :] = 40
 	sv2 = np.full_like(sv, 40)
-	got_c, _ = _run_attn(dev, kern, q, kv2.reshape(t, -1), sk, sv2, temp, 64)
+	got_c, _ = _run_attn(dev, kern, np.zeros_like(q), kv2.reshape(t, -1), sk, sv2, temp, 64)
 	assert np.all(got_c == 40)
+	got_r, _ = _run_attn(dev, kern, q, kv2.reshape(t, -1), sk, sv2, temp, 64)
+	assert np.all(np.abs(got_r.astype(np.int32) - 40) <= 1)
+	want_r, _ = S.attn_fwd_i8(q, kv2.reshape(t, -1), sk, sv2, temp, h, hd, 64)
+	assert np.array_equal(got_r, want_r)
 
 
 def test_attn_launch_rejects_bad_arguments(dev):

@@ -75,20 +75,22 @@ X17_DEV i32 partner_i32(i32 x, u32 half) {
 }
 
 // K tile: linear 16-byte chunk n = key * CPR + c lives in 128-byte line n / 8 at position
-// (n % 8) ^ (line & 7), which keeps ds_read_b128 of 8 consecutive keys conflict-free for every
-// supported head_dim.
+// (n % 8) ^ ((line >> 1) & 7).  The LDS serves a ds_read_b128 sixteen lanes at a time out of 64
+// four-byte banks; with this mapping the sixteen keys of such a group land in sixteen different
+// 16-byte slots for every supported head_dim.
 X17_DEV u32 k_chunk_offset(u32 key, u32 c) {
 	u32 n = key * CPR + c;
 	u32 line = n >> 3;
-	return (line << 7) | (((n & 7) ^ (line & 7)) << 4);
+	return (line << 7) | (((n & 7) ^ ((line >> 1) & 7)) << 4);
 }
 
 // V tile (bf16): linear 32-byte granule n = key * CPR + c (16 dims) lives in 256-byte line n / 8
-// at position (n % 8) ^ (line & 7).
+// at position (n % 8) ^ ((line & 3) << 1): the 4 keys x 2 granules that 32 lanes of a transposed
+// read touch then cover all 64 banks exactly once (checked exhaustively for head_dim 32/64/128).
 X17_DEV u32 v_granule_offset(u32 key, u32 c) {
 	u32 n = key * CPR + c;
 	u32 line = n >> 3;
-	return (line << 8) | (((n & 7) ^ (line & 7)) << 5);
+	return (line << 8) | (((n & 7) ^ ((line & 3) << 1)) << 5);
 }
 
 X17_DEV u32 pack_bf16(f32 lo, f32 hi) {
@@ -143,7 +145,7 @@ void kernel(
 			if (tid < 32 * CPR) {
 				// lane `tid` fills stored chunk `tid` of the K tile; find which logical chunk lives there
 				u32 line = tid >> 3;
-				u32 n = (line << 3) | ((tid & 7) ^ (line & 7));
+				u32 n = (line << 3) | ((tid & 7) ^ ((line >> 1) & 7));
 				u32 key = n / CPR, c = n % CPR;
 				i8 const *src = kv_head + (size_t)(kb * at::KV_PER_STEP + key) * KV_STRIDE + c * 16;
 				u8 *dst = smem + stage * at::STAGE_BYTES + (tid / 64) * 1024;

@@ -6,7 +6,8 @@
 // entry and its parameters follow templates/basic_gemm/kernel.cu:9-32.
 //
 // Design, MI355X-first (nothing here is derived from the SM80 kernel):
-//   * One workgroup = 4 wavefronts = a 256 (tokens) x 256 (raw columns) output tile; each
+//   * One workgroup = a 256 (tokens) x 256 (raw columns) output tile, by default 8 wavefronts of
+//     64 x 128 (two per SIMD; gemm_tile.h can also build 4 wavefronts of 128 x 128); in the 4-wave form each
 //     wavefront owns 128 x 128 as a 4 x 4 grid of 32x32 MFMA blocks (256 accumulator
 //     registers per lane, one wavefront per SIMD).
 //   * The WEIGHTS are the MFMA "A" operand and the TOKENS the "B" operand, i.e. the matrix
@@ -17,7 +18,7 @@
 //     code needs a 4x4 shuffle transpose per 32x32 tile, cuda/gemm_b8.cuh:411, 570, 592).
 //   * Global -> LDS goes through the gfx950 16-byte direct-to-LDS load (no register staging),
 //     K_STEP = 128 bytes per step, two stages, one barrier per step.  Rows are 128 bytes;
-//     16-byte chunks are XOR-swizzled with the row index so ds_read_b128 is conflict-free.
+//     16-byte chunks are XOR-swizzled with the row-pair index so ds_read_b128 is conflict-free.
 //   * int8: v_mfma_i32_32x32x32_i8.  e4m3 x e4m3: v_mfma_f32_32x32x64_f8f6f4.  Mixed
 //     e4m3 x int8: both widened exactly to bf16 in registers, v_mfma_f32_32x32x16_bf16
 //     (int8 codes need 7 significand bits, e4m3 has 4).
@@ -57,6 +58,11 @@ constexpr u32 X_TILE_BYTES = gt::M_PER_BLOCK * ROW_BYTES;   // tokens
 constexpr u32 W_TILE_BYTES = gt::N_PER_BLOCK * ROW_BYTES;   // weights
 constexpr u32 STAGE_BYTES = X_TILE_BYTES + W_TILE_BYTES;
 constexpr u32 K_STEPS = K_TOTAL / gt::K_STEP;
+
+constexpr int BM = gt::WAVE_M / 32;                         // 32-token MFMA blocks per wave
+constexpr u32 WAVES = gt::WAVES_M * gt::WAVES_N;
+constexpr u32 ROWS_PER_WAVE = 256 / WAVES;                  // rows of each tile a wave copies per stage
+constexpr u32 UNITS = ROWS_PER_WAVE / 8;                    // 8-row direct-to-LDS loads per wave and tile
 
 using Acc = __attribute__((ext_vector_type(16))) int;       // raw 16 registers; reinterpreted as f32 when ACC_F32
 
@@ -171,33 +177,37 @@ static_assert(HEAD_DIM == 32 || HEAD_DIM == 64 || HEAD_DIM == 128, "head_dim mus
 
 // ------------------------------------------------------------------ tile loads
 
+// LDS rows are 128 bytes = 8 chunks of 16; logical chunk c of row r is stored at position
+// c ^ ((r >> 1) & 7).  The LDS has 64 four-byte banks and serves a ds_read_b128 sixteen lanes at a
+// time, so sixteen consecutive rows (two per 256-byte bank line) must land in sixteen different
+// 16-byte slots: the row PAIR index is what has to be mixed in.
 struct LaneOffsets {
-	u32 x_src;      // per-lane byte offset into A for a direct-to-LDS load
-	u32 w_src;      // per-lane byte offset into B
+	u32 x_src[2];   // per-lane byte offset into A for a direct-to-LDS load (even / odd 8-row unit)
+	u32 w_src[2];   // per-lane byte offset into B
 	u32 frag_row;   // (lane % 32) * ROW_BYTES
 	u32 half;       // lane / 32
-	u32 swz;        // lane & 7
+	u32 swz;        // (lane >> 1) & 7
 };
 
 X17_DEV void issue_stage_loads(
 	u8 const *a_tile, u8 const *b_tile, u8 *stage, u32 k0, u32 wave, LaneOffsets const &lo
 ) {
-	// Wave w copies token rows [64w, 64w+64) and LDS weight rows [64w, 64w+64), 8 rows per load.
-	u8 *x_lds = stage + wave * 64 * ROW_BYTES;
-	u8 *w_lds = stage + X_TILE_BYTES + wave * 64 * ROW_BYTES;
-	u8 const *x_src = a_tile + (size_t)(wave * 64) * K_TOTAL + k0;
-	X17_UNROLL for (u32 u = 0; u < 8; ++u) {
+	// Wave w copies token rows and LDS weight rows [ROWS_PER_WAVE * w, +ROWS_PER_WAVE), 8 rows per load.
+	u8 *x_lds = stage + wave * ROWS_PER_WAVE * ROW_BYTES;
+	u8 *w_lds = stage + X_TILE_BYTES + wave * ROWS_PER_WAVE * ROW_BYTES;
+	u8 const *x_src = a_tile + (size_t)(wave * ROWS_PER_WAVE) * K_TOTAL + k0;
+	X17_UNROLL for (u32 u = 0; u < UNITS; ++u) {
 		__builtin_amdgcn_global_load_lds(
-			X17_GLOBAL_PTR(x_src + (size_t)(u * 8) * K_TOTAL + lo.x_src),
+			X17_GLOBAL_PTR(x_src + (size_t)(u * 8) * K_TOTAL + lo.x_src[u & 1]),
 			X17_LDS_PTR(x_lds + u * 8 * ROW_BYTES), 16, 0, 0);
 	}
 	// LDS weight row R = 128*wn + 32*bn + i holds weight row 128*wn + 64*((i/4)%2) + 16*bn + 4*(i/8) + i%4
 	// (see the header comment); for the 8 rows of one load the lane-dependent part is constant.
-	X17_UNROLL for (u32 u = 0; u < 8; ++u) {
-		u32 r0 = wave * 64 + u * 8;
+	X17_UNROLL for (u32 u = 0; u < UNITS; ++u) {
+		u32 r0 = wave * ROWS_PER_WAVE + u * 8;
 		u32 n_uniform = 128 * (r0 / 128) + 16 * ((r0 % 128) / 32) + 4 * ((r0 % 32) / 8);
 		__builtin_amdgcn_global_load_lds(
-			X17_GLOBAL_PTR(b_tile + (size_t)n_uniform * K_TOTAL + k0 + lo.w_src),
+			X17_GLOBAL_PTR(b_tile + (size_t)n_uniform * K_TOTAL + k0 + lo.w_src[u & 1]),
 			X17_LDS_PTR(w_lds + u * 8 * ROW_BYTES), 16, 0, 0);
 	}
 }
@@ -274,20 +284,23 @@ void kernel(
 	LaneOffsets lo;
 	{
 		u32 r = lane >> 3, p = lane & 7;
-		u32 chunk = p ^ r;
-		lo.x_src = r * K_TOTAL + 16 * chunk;
-		lo.w_src = (64 * ((lane >> 5) & 1) + ((lane >> 3) & 3)) * K_TOTAL + 16 * chunk;
+		X17_UNROLL for (u32 odd = 0; odd < 2; ++odd) {
+			// the 8 rows of a load unit start at a multiple of 8: row pair index & 7 = 4 * (unit & 1) + r / 2
+			u32 chunk = p ^ (4 * odd + (r >> 1));
+			lo.x_src[odd] = r * K_TOTAL + 16 * chunk;
+			lo.w_src[odd] = (64 * ((lane >> 5) & 1) + ((lane >> 3) & 3)) * K_TOTAL + 16 * chunk;
+		}
 		lo.frag_row = (lane % 32) * ROW_BYTES;
 		lo.half = lane / 32;
-		lo.swz = lane & 7;
+		lo.swz = (lane >> 1) & 7;
 	}
 
 	u8 const *a_tile = a + (size_t)(tile_m * gt::M_PER_BLOCK) * K_TOTAL;
 	u8 const *b_tile = b + (size_t)(tile_n * gt::N_PER_BLOCK) * K_TOTAL;
 
-	Acc acc[4][4];   // [bn][bm]
+	Acc acc[4][BM];   // [bn][bm]
 	X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
-		X17_UNROLL for (int bm = 0; bm < 4; ++bm) {
+		X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
 			X17_UNROLL for (int r = 0; r < 16; ++r) acc[bn][bm][r] = 0;
 		}
 	}
@@ -301,52 +314,52 @@ void kernel(
 			issue_stage_loads(a_tile, b_tile, smem + ((ks + 1) % gt::STAGES) * STAGE_BYTES,
 			                  (ks + 1) * gt::K_STEP, wave, lo);
 		}
-		u8 const *x_tile = smem + (ks % gt::STAGES) * STAGE_BYTES + wm * 128 * ROW_BYTES + lo.frag_row;
+		u8 const *x_tile = smem + (ks % gt::STAGES) * STAGE_BYTES + wm * gt::WAVE_M * ROW_BYTES + lo.frag_row;
 		u8 const *w_tile = smem + (ks % gt::STAGES) * STAGE_BYTES + X_TILE_BYTES + wn * 128 * ROW_BYTES + lo.frag_row;
 
 		if constexpr (MMA == 0) {
 			// 32 bytes of K per MFMA; operand fragments of slice s+1 are fetched before the
 			// MFMAs of slice s are issued, so LDS latency hides under matrix-core time
-			v4i wf[2][4], xf[2][4];
+			v4i wf[2][4], xf[2][BM];
 			X17_UNROLL for (int bn = 0; bn < 4; ++bn) wf[0][bn] = lds_chunk(w_tile, bn * 32 * ROW_BYTES, lo.half, lo.swz);
-			X17_UNROLL for (int bm = 0; bm < 4; ++bm) xf[0][bm] = lds_chunk(x_tile, bm * 32 * ROW_BYTES, lo.half, lo.swz);
+			X17_UNROLL for (int bm = 0; bm < BM; ++bm) xf[0][bm] = lds_chunk(x_tile, bm * 32 * ROW_BYTES, lo.half, lo.swz);
 			X17_UNROLL for (u32 s = 0; s < 4; ++s) {
 				if (s + 1 < 4) {
 					u32 kc = 2 * (s + 1) + lo.half;
 					X17_UNROLL for (int bn = 0; bn < 4; ++bn) wf[(s + 1) & 1][bn] = lds_chunk(w_tile, bn * 32 * ROW_BYTES, kc, lo.swz);
-					X17_UNROLL for (int bm = 0; bm < 4; ++bm) xf[(s + 1) & 1][bm] = lds_chunk(x_tile, bm * 32 * ROW_BYTES, kc, lo.swz);
+					X17_UNROLL for (int bm = 0; bm < BM; ++bm) xf[(s + 1) & 1][bm] = lds_chunk(x_tile, bm * 32 * ROW_BYTES, kc, lo.swz);
 				}
 				X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
-					X17_UNROLL for (int bm = 0; bm < 4; ++bm) {
+					X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
 						acc[bn][bm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[s & 1][bn], xf[s & 1][bm], acc[bn][bm], 0, 0, 0);
 					}
 				}
 				// pin the issue order: two MFMAs, then one of the eight LDS reads of the next slice
 				if (s + 1 < 4) {
-					X17_UNROLL for (int i = 0; i < 8; ++i) {
-						__builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+					X17_UNROLL for (int i = 0; i < 4 + BM; ++i) {
+						__builtin_amdgcn_sched_group_barrier(0x008, (4 * BM) / (4 + BM), 0);
 						__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
 					}
 				} else {
-					__builtin_amdgcn_sched_group_barrier(0x008, 16, 0);
+					__builtin_amdgcn_sched_group_barrier(0x008, 4 * BM, 0);
 				}
 			}
 		} else if constexpr (MMA == 1) {
 			X17_UNROLL for (u32 s = 0; s < 2; ++s) {            // 64 bytes of K per MFMA
-				v8i wf[4], xf[4];
+				v8i wf[4], xf[BM];
 				u32 kc = 4 * s + 2 * lo.half;
 				X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
 					v4i lo4 = lds_chunk(w_tile, bn * 32 * ROW_BYTES, kc, lo.swz);
 					v4i hi4 = lds_chunk(w_tile, bn * 32 * ROW_BYTES, kc + 1, lo.swz);
 					wf[bn] = v8i{lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
 				}
-				X17_UNROLL for (int bm = 0; bm < 4; ++bm) {
+				X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
 					v4i lo4 = lds_chunk(x_tile, bm * 32 * ROW_BYTES, kc, lo.swz);
 					v4i hi4 = lds_chunk(x_tile, bm * 32 * ROW_BYTES, kc + 1, lo.swz);
 					xf[bm] = v8i{lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
 				}
 				X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
-					X17_UNROLL for (int bm = 0; bm < 4; ++bm) {
+					X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
 						v16f r = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
 							wf[bn], xf[bm], __builtin_bit_cast(v16f, acc[bn][bm]), 0, 0, 0, 0, 0, 0);
 						acc[bn][bm] = __builtin_bit_cast(Acc, r);
@@ -356,15 +369,15 @@ void kernel(
 		} else {
 			X17_UNROLL for (u32 s = 0; s < 4; ++s) {            // 32 bytes of K = two bf16 MFMAs of 16
 				u32 kc = 2 * s + lo.half;
-				v4i wraw[4], xraw[4];
+				v4i wraw[4], xraw[BM];
 				X17_UNROLL for (int bn = 0; bn < 4; ++bn) wraw[bn] = lds_chunk(w_tile, bn * 32 * ROW_BYTES, kc, lo.swz);
-				X17_UNROLL for (int bm = 0; bm < 4; ++bm) xraw[bm] = lds_chunk(x_tile, bm * 32 * ROW_BYTES, kc, lo.swz);
+				X17_UNROLL for (int bm = 0; bm < BM; ++bm) xraw[bm] = lds_chunk(x_tile, bm * 32 * ROW_BYTES, kc, lo.swz);
 				X17_UNROLL for (int h = 0; h < 2; ++h) {
-					v8bf wf[4], xf[4];
+					v8bf wf[4], xf[BM];
 					X17_UNROLL for (int bn = 0; bn < 4; ++bn) wf[bn] = widen8(wraw[bn][2 * h], wraw[bn][2 * h + 1], B_KIND);
-					X17_UNROLL for (int bm = 0; bm < 4; ++bm) xf[bm] = widen8(xraw[bm][2 * h], xraw[bm][2 * h + 1], A_KIND);
+					X17_UNROLL for (int bm = 0; bm < BM; ++bm) xf[bm] = widen8(xraw[bm][2 * h], xraw[bm][2 * h + 1], A_KIND);
 					X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
-						X17_UNROLL for (int bm = 0; bm < 4; ++bm) {
+						X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
 							v16f r = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
 								wf[bn], xf[bm], __builtin_bit_cast(v16f, acc[bn][bm]), 0, 0, 0);
 							acc[bn][bm] = __builtin_bit_cast(Acc, r);
@@ -377,10 +390,10 @@ void kernel(
 
 	// ---- epilogue.  Lane owns token (32*bm + lane%32) of its wave and raw columns
 	// 64*(lane/32) + 16*bn + r of its wave, r = accumulator register index.
-	u32 const row0 = tile_m * gt::M_PER_BLOCK + wm * 128 + lane % 32;
+	u32 const row0 = tile_m * gt::M_PER_BLOCK + wm * gt::WAVE_M + lane % 32;
 	u32 const n0 = tile_n * gt::N_PER_BLOCK + wn * 128 + 64 * lo.half;
 
-	X17_UNROLL for (int bm = 0; bm < 4; ++bm) {
+	X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
 		u32 row = row0 + 32 * bm;
 		f32 x[64];
 		X17_UNROLL for (int bn = 0; bn < 4; ++bn) {

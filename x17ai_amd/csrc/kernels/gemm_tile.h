@@ -9,11 +9,16 @@
 namespace x17 { namespace gemm_tile {
 
 constexpr unsigned WAVE = 64;
-constexpr unsigned WAVES_M = 2;                 // waves along the token (M) dimension
+#ifndef X17_GEMM_WAVES_M
+#define X17_GEMM_WAVES_M 4
+#endif
+// 4 x 2 waves (two per SIMD, 64 x 128 each: the second wave fills the first one's MFMA issue gaps)
+// or 2 x 2 waves (one per SIMD, 128 x 128 each: fewest LDS reads per MFMA)
+constexpr unsigned WAVES_M = X17_GEMM_WAVES_M;  // waves along the token (M) dimension
 constexpr unsigned WAVES_N = 2;                 // waves along the output-column (N) dimension
 constexpr unsigned THREADS_PER_BLOCK = WAVE * WAVES_M * WAVES_N;
 
-constexpr unsigned WAVE_M = 128;                // tokens per wave
+constexpr unsigned WAVE_M = 256 / WAVES_M;      // tokens per wave
 constexpr unsigned WAVE_N = 128;                // raw output columns per wave
 constexpr unsigned M_PER_BLOCK = WAVE_M * WAVES_M;
 constexpr unsigned N_PER_BLOCK = WAVE_N * WAVES_N;
