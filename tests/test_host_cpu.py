@@ -122,7 +122,7 @@ def test_kernel_build_metadata_and_cache(tmp_path, monkeypatch):
 	(the reference recompiles on every run, src/device/cuda/gemm.rs:408-416)."""
 	monkeypatch.setenv("X17AI_KERNEL_CACHE", str(tmp_path))
 	k = recipes.attn_q_kernel(None, 256, 256)
-	assert k.metadata == {"THREADS_PER_BLOCK": 256, "SMEM_BYTES": 131072, "M_PER_BLOCK": 256, "N_PER_BLOCK": 256}
+	assert k.metadata == {"THREADS_PER_BLOCK": 512, "SMEM_BYTES": 131072, "M_PER_BLOCK": 256, "N_PER_BLOCK": 256}
 	d = tmp_path / k.name
 	assert (d / "kernel.hsaco").stat().st_size > 1000
 	text = (d / "common.h").read_text()

@@ -624,7 +624,7 @@ std::unique_ptr<GemmKernel> GemmKernel::create(std::shared_ptr<HipDevice> device
 	if (!meta) return nullptr;
 	auto out = std::make_unique<GemmKernel>();
 	auto get = [&](char const *k) { auto v = kernel_build::meta_get(*meta, k); return v ? *v : size_t(0); };
-	out->metadata = GemmLauncherMetadata{get("THREADS_PER_BLOCK"), get("SMEM_BYTES"), get("M_PER_BLOCK"), get("N_PER_BLOCK")};
+	out->metadata = GemmLauncherMetadata{get("THREADS_PER_BLOCK"), get("SMEM_BYTES"), get("M_PER_BLOCK"), get("N_PER_BLOCK"), get("MAX_BLOCKS")};
 	// gemm.rs:561-570
 	if (out->metadata.THREADS_PER_BLOCK == 0 || !is_pow2(out->metadata.M_PER_BLOCK) || !is_pow2(out->metadata.N_PER_BLOCK)) {
 		diag.add_error("Invalid JSON metadata in " + built->meta_json_path);
@@ -705,6 +705,11 @@ Status GemmKernel::launch(GemmArgs const &args) {
 	void *extra_ptr = args.extra != nullptr ? args.extra->ptr : nullptr;
 	void *raw_args[6] = {&a_ptr, &a_rows_arg, &b_ptr, &b_rows_arg, &c_ptr, &extra_ptr};
 	size_t grid[3] = {grid_x, grid_y, 1};
+	if (metadata.MAX_BLOCKS != 0 && grid_x * grid_y > metadata.MAX_BLOCKS) {
+		// persistent kernel: the workgroups share the tiles out among themselves
+		grid[0] = metadata.MAX_BLOCKS;
+		grid[1] = 1;
+	}
 	size_t block[3] = {metadata.THREADS_PER_BLOCK, 1, 1};
 	return kernel->launch(*device->stream, grid, block, metadata.SMEM_BYTES, raw_args);
 }

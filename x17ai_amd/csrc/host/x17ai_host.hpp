@@ -192,7 +192,8 @@ using EpilogueConfig = std::variant<ScaleConfig, GeGluConfig, ResidualConfig, RM
 struct GemmInputConfig { DType dtype; size_t cols; std::optional<size_t> rows; bool trans; };
 struct GemmConfig { GemmInputConfig a, b; DType c_dtype; };
 
-struct GemmLauncherMetadata { size_t THREADS_PER_BLOCK, SMEM_BYTES, M_PER_BLOCK, N_PER_BLOCK; };
+// MAX_BLOCKS (0 = one workgroup per tile, as in the reference) caps the grid of the persistent kernel
+struct GemmLauncherMetadata { size_t THREADS_PER_BLOCK, SMEM_BYTES, M_PER_BLOCK, N_PER_BLOCK, MAX_BLOCKS; };
 
 struct GemmArgs {
 	Tensor const *a; Tensor const *b; Tensor const *c;

@@ -16,9 +16,9 @@
 //     columns across the four blocks.  Gate/value pairs, whole K|V heads and 16-byte output
 //     vectors all live inside one lane: the epilogues need no cross-lane shuffles (the SM80
 //     code needs a 4x4 shuffle transpose per 32x32 tile, cuda/gemm_b8.cuh:411, 570, 592).
-//   * Global -> LDS goes through the gfx950 16-byte direct-to-LDS load (no register staging),
-//     K_STEP = 128 bytes per step, two stages, one barrier per step.  Rows are 128 bytes;
-//     16-byte chunks are XOR-swizzled with the row-pair index so ds_read_b128 is conflict-free.
+//   * Global -> LDS goes through the gfx950 16-byte direct-to-LDS load (no register staging) into
+//     a ring of LDS stages (gemm_tile.h: K_STEP bytes of K per step), one barrier per step;
+//     16-byte chunks are XOR-swizzled so that ds_read_b128 is conflict-free.
 //   * int8: v_mfma_i32_32x32x32_i8.  e4m3 x e4m3: v_mfma_f32_32x32x64_f8f6f4.  Mixed
 //     e4m3 x int8: both widened exactly to bf16 in registers, v_mfma_f32_32x32x16_bf16
 //     (int8 codes need 7 significand bits, e4m3 has 4).
@@ -53,7 +53,7 @@ constexpr bool ACC_F32 = MMA != 0;
 static_assert(K_TOTAL % gt::K_STEP == 0, "K must be a multiple of 128");
 static_assert(N_RAW % gt::N_PER_BLOCK == 0, "raw output columns must be a multiple of 256");
 
-constexpr u32 ROW_BYTES = gt::K_STEP;                       // one LDS row = 128 bytes of K
+constexpr u32 ROW_BYTES = gt::K_STEP;                       // one LDS row = one step of K
 constexpr u32 X_TILE_BYTES = gt::M_PER_BLOCK * ROW_BYTES;   // tokens
 constexpr u32 W_TILE_BYTES = gt::N_PER_BLOCK * ROW_BYTES;   // weights
 constexpr u32 STAGE_BYTES = X_TILE_BYTES + W_TILE_BYTES;
@@ -177,42 +177,80 @@ static_assert(HEAD_DIM == 32 || HEAD_DIM == 64 || HEAD_DIM == 128, "head_dim mus
 
 // ------------------------------------------------------------------ tile loads
 
-// LDS rows are 128 bytes = 8 chunks of 16; logical chunk c of row r is stored at position
-// c ^ ((r >> 1) & 7).  The LDS has 64 four-byte banks and serves a ds_read_b128 sixteen lanes at a
-// time, so sixteen consecutive rows (two per 256-byte bank line) must land in sixteen different
-// 16-byte slots: the row PAIR index is what has to be mixed in.
+// LDS rows hold K_STEP bytes = CHUNKS chunks of 16; logical chunk c of row r is stored at position
+// c ^ ((r >> SWZ_SHIFT) & (CHUNKS - 1)).  The LDS has 64 four-byte banks (256 bytes per bank line)
+// and serves a ds_read_b128 sixteen lanes at a time, so sixteen consecutive rows must land in sixteen
+// different 16-byte slots of the bank line: with 128-byte rows two rows share a bank line and the row
+// PAIR index has to be mixed in, with 64-byte rows the row QUAD index.
+constexpr u32 CHUNKS = gt::K_STEP / 16;
+constexpr u32 SWZ_SHIFT = gt::K_STEP == 128 ? 1 : 2;
+constexpr u32 UNIT_ROWS = 64 / CHUNKS;                      // rows one 64-lane x 16-byte direct-to-LDS load fills
+constexpr u32 X_UNITS = gt::M_PER_BLOCK / UNIT_ROWS / WAVES; // such loads per wave, stage and tile
+constexpr u32 W_UNITS = gt::N_PER_BLOCK / UNIT_ROWS / WAVES;
+constexpr u32 LOADS_PER_STAGE = X_UNITS + W_UNITS;
+static_assert((X_UNITS * UNIT_ROWS) % 16 == 0 && (W_UNITS * UNIT_ROWS) % 16 == 0, "a wave's share must keep the swizzle phase");
+
 struct LaneOffsets {
-	u32 x_src[2];   // per-lane byte offset into A for a direct-to-LDS load (even / odd 8-row unit)
+	u32 x_src[2];   // per-lane byte offset into A for a direct-to-LDS load (even / odd load unit)
 	u32 w_src[2];   // per-lane byte offset into B
 	u32 frag_row;   // (lane % 32) * ROW_BYTES
 	u32 half;       // lane / 32
-	u32 swz;        // (lane >> 1) & 7
+	u32 swz;        // swizzle key of the fragment row this lane reads
 };
 
-X17_DEV void issue_stage_loads(
+// Direct-to-LDS load `i` (0 .. LOADS_PER_STAGE-1) of this wave's share of one stage: first the token
+// units, then the weight units.  Wave w copies token rows [X_UNITS * UNIT_ROWS * w, +X_UNITS * UNIT_ROWS)
+// and as many LDS weight rows.
+// LDS weight row R = 128*wn + 32*bn + i holds weight row 128*wn + 64*((i/4)%2) + 16*bn + 4*(i/8) + i%4:
+// the MFMA hands output row i = 8*(r/4) + 4*(lane/32) + r%4 to register r, so a lane collects columns
+// 64*(lane/32) + 16*bn + r.  For the rows of one load unit the lane-dependent part is constant.
+template <u32 I>
+X17_DEV void issue_stage_load(
 	u8 const *a_tile, u8 const *b_tile, u8 *stage, u32 k0, u32 wave, LaneOffsets const &lo
 ) {
-	// Wave w copies token rows and LDS weight rows [ROWS_PER_WAVE * w, +ROWS_PER_WAVE), 8 rows per load.
-	u8 *x_lds = stage + wave * ROWS_PER_WAVE * ROW_BYTES;
-	u8 *w_lds = stage + X_TILE_BYTES + wave * ROWS_PER_WAVE * ROW_BYTES;
-	u8 const *x_src = a_tile + (size_t)(wave * ROWS_PER_WAVE) * K_TOTAL + k0;
-	X17_UNROLL for (u32 u = 0; u < UNITS; ++u) {
-		__builtin_amdgcn_global_load_lds(
-			X17_GLOBAL_PTR(x_src + (size_t)(u * 8) * K_TOTAL + lo.x_src[u & 1]),
-			X17_LDS_PTR(x_lds + u * 8 * ROW_BYTES), 16, 0, 0);
-	}
-	// LDS weight row R = 128*wn + 32*bn + i holds weight row 128*wn + 64*((i/4)%2) + 16*bn + 4*(i/8) + i%4
-	// (see the header comment); for the 8 rows of one load the lane-dependent part is constant.
-	X17_UNROLL for (u32 u = 0; u < UNITS; ++u) {
-		u32 r0 = wave * ROWS_PER_WAVE + u * 8;
+	if constexpr (I < X_UNITS) {
+		constexpr u32 u = I;
+		u8 *x_lds = stage + (wave * X_UNITS + u) * UNIT_ROWS * ROW_BYTES;
+		u8 const *x_src = a_tile + (size_t)((wave * X_UNITS + u) * UNIT_ROWS) * K_TOTAL + k0;
+		__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(x_src + lo.x_src[u & 1]), X17_LDS_PTR(x_lds), 16, 0, 0);
+	} else {
+		constexpr u32 u = I - X_UNITS;
+		u32 r0 = (wave * W_UNITS + u) * UNIT_ROWS;
 		u32 n_uniform = 128 * (r0 / 128) + 16 * ((r0 % 128) / 32) + 4 * ((r0 % 32) / 8);
-		__builtin_amdgcn_global_load_lds(
-			X17_GLOBAL_PTR(b_tile + (size_t)n_uniform * K_TOTAL + k0 + lo.w_src[u & 1]),
-			X17_LDS_PTR(w_lds + u * 8 * ROW_BYTES), 16, 0, 0);
+		u8 *w_lds = stage + X_TILE_BYTES + r0 * ROW_BYTES;
+		u8 const *w_src = b_tile + (size_t)n_uniform * K_TOTAL + k0;
+		__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(w_src + lo.w_src[u & 1]), X17_LDS_PTR(w_lds), 16, 0, 0);
 	}
 }
 
-// One 16-byte operand chunk: row `row_off` (bytes), logical chunk `kc` of the 128-byte row.
+template <u32 FIRST, u32 LAST>
+X17_DEV void issue_stage_loads(
+	u8 const *a_tile, u8 const *b_tile, u8 *stage, u32 k0, u32 wave, LaneOffsets const &lo
+) {
+	if constexpr (FIRST < LAST) {
+		issue_stage_load<FIRST>(a_tile, b_tile, stage, k0, wave, lo);
+		issue_stage_loads<FIRST + 1, LAST>(a_tile, b_tile, stage, k0, wave, lo);
+	}
+}
+
+// s_waitcnt vmcnt(N) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14)
+template <u32 N>
+X17_DEV void wait_vmcnt() {
+	static_assert(N < 64);
+	__builtin_amdgcn_s_waitcnt((N & 15u) | ((N >> 4) << 14) | 0x0F70u);
+}
+// wait until at most `later` younger stages are still in flight
+X17_DEV void wait_stage(u32 later) {
+	if constexpr (gt::STAGES >= 4) {
+		if (later >= 2) { wait_vmcnt<2 * LOADS_PER_STAGE>(); return; }
+	}
+	if constexpr (gt::STAGES >= 3) {
+		if (later >= 1) { wait_vmcnt<LOADS_PER_STAGE>(); return; }
+	}
+	wait_vmcnt<0>();
+}
+
+// One 16-byte operand chunk: row `row_off` (bytes), logical chunk `kc` of the row.
 X17_DEV v4i lds_chunk(u8 const *tile, u32 row_off, u32 kc, u32 swz) {
 	return *reinterpret_cast<v4i const *>(tile + row_off + ((kc ^ swz) << 4));
 }
@@ -238,9 +276,94 @@ X17_DEV v8bf widen8(u32 lo, u32 hi, int kind) {
 	return __builtin_bit_cast(v8bf, packed);
 }
 
+// Operand fragments of one K slice (what one round of 4 x BM MFMA blocks consumes) and the MFMAs
+// themselves, per arithmetic: 32 bytes of K for int8 and for the bf16-widened mix, 64 for e4m3.
+constexpr u32 SLICE_BYTES = MMA == 1 ? 64 : 32;
+constexpr u32 SLICES = gt::K_STEP / SLICE_BYTES;
+constexpr u32 CHUNKS_PER_FRAG = SLICE_BYTES / 32;           // 16-byte chunks a lane fetches per operand row
+static_assert(SLICES % 2 == 0, "the fragment double buffer needs an even number of slices per step");
+
+struct Frags {
+	v4i w[4][CHUNKS_PER_FRAG];
+	v4i x[BM][CHUNKS_PER_FRAG];
+};
+
+X17_DEV void load_frags(Frags &f, u8 const *w_tile, u8 const *x_tile, u32 s, LaneOffsets const &lo) {
+	X17_UNROLL for (u32 c = 0; c < CHUNKS_PER_FRAG; ++c) {
+		u32 kc = CHUNKS_PER_FRAG * (2 * s + lo.half) + c;
+		X17_UNROLL for (int bn = 0; bn < 4; ++bn) f.w[bn][c] = lds_chunk(w_tile, bn * 32 * ROW_BYTES, kc, lo.swz);
+		X17_UNROLL for (int bm = 0; bm < BM; ++bm) f.x[bm][c] = lds_chunk(x_tile, bm * 32 * ROW_BYTES, kc, lo.swz);
+	}
+}
+
+X17_DEV void mma_slice(Frags const &f, Acc (&acc)[4][BM]) {
+	if constexpr (MMA == 0) {
+		X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
+			X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
+				acc[bn][bm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w[bn][0], f.x[bm][0], acc[bn][bm], 0, 0, 0);
+			}
+		}
+	} else if constexpr (MMA == 1) {
+		v8i wf[4], xf[BM];
+		X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
+			v4i l = f.w[bn][0], h = f.w[bn][CHUNKS_PER_FRAG - 1];
+			wf[bn] = v8i{l[0], l[1], l[2], l[3], h[0], h[1], h[2], h[3]};
+		}
+		X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
+			v4i l = f.x[bm][0], h = f.x[bm][CHUNKS_PER_FRAG - 1];
+			xf[bm] = v8i{l[0], l[1], l[2], l[3], h[0], h[1], h[2], h[3]};
+		}
+		X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
+			X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
+				v16f r = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+					wf[bn], xf[bm], __builtin_bit_cast(v16f, acc[bn][bm]), 0, 0, 0, 0, 0, 0);
+				acc[bn][bm] = __builtin_bit_cast(Acc, r);
+			}
+		}
+	} else {
+		X17_UNROLL for (int h = 0; h < 2; ++h) {                // two bf16 MFMAs of K = 16
+			v8bf wf[4], xf[BM];
+			X17_UNROLL for (int bn = 0; bn < 4; ++bn) wf[bn] = widen8(f.w[bn][0][2 * h], f.w[bn][0][2 * h + 1], B_KIND);
+			X17_UNROLL for (int bm = 0; bm < BM; ++bm) xf[bm] = widen8(f.x[bm][0][2 * h], f.x[bm][0][2 * h + 1], A_KIND);
+			X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
+				X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
+					v16f r = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+						wf[bn], xf[bm], __builtin_bit_cast(v16f, acc[bn][bm]), 0, 0, 0);
+					acc[bn][bm] = __builtin_bit_cast(Acc, r);
+				}
+			}
+		}
+	}
+}
+
+// Pin the issue order of one slice: the LDS reads of the next fragments and this slice's share of the
+// next stage's global loads are spread evenly between the MFMAs.  LDS latency then hides under
+// matrix-core time, and a wave never sits in a burst of loads waiting for the memory pipeline to
+// accept them (instructions issue in order: a queued load would hold back the MFMAs behind it).
+template <u32 N_LOADS>
+X17_DEV void interleave_slice(bool with_reads) {
+	if constexpr (MMA != 2) {
+		constexpr int READS = (4 + BM) * CHUNKS_PER_FRAG;
+		constexpr int MFMAS = 4 * BM;
+		constexpr int GROUPS = MFMAS < READS ? MFMAS : READS;
+		if (with_reads) {
+			X17_UNROLL for (int i = 0; i < GROUPS; ++i) {
+				__builtin_amdgcn_sched_group_barrier(0x008, MFMAS / GROUPS, 0);
+				__builtin_amdgcn_sched_group_barrier(0x100, READS / GROUPS, 0);
+				if (i < (int)N_LOADS) {
+					__builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+				}
+			}
+		} else {
+			__builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
+		}
+	}
+}
+
 } // namespace
 
 extern "C" __global__ __launch_bounds__(gt::THREADS_PER_BLOCK)
+__attribute__((amdgpu_waves_per_eu(gt::WAVES_PER_SIMD, gt::WAVES_PER_SIMD)))
 void kernel(
 	u8 const *a, u32 a_rows,
 	u8 const *b, u32 b_rows,
@@ -252,27 +375,32 @@ void kernel(
 #endif
 ) {
 	extern __shared__ __attribute__((aligned(1024))) u8 smem[];
-	(void)a_rows;
 	(void)b_rows;   // known at compile time, as in templates/basic_gemm/kernel.cu:18-21
 
-	// ---- which tile: remap the linear workgroup id so each XCD gets a compact block of tiles
-	u32 const tiles_m = gridDim.x;
-	u32 const tiles_n = gridDim.y;
+	// ---- which tiles.  The kernel is persistent: workgroup g of G works on tiles g, g + G, ... and
+	// any grid shape is accepted (with one workgroup per tile, as the reference launches it, every
+	// workgroup runs the loop once).  The linear tile id is remapped so that each XCD (own L2) gets a
+	// compact block of tiles -- the hardware deals workgroups round-robin to the 8 XCDs -- and tiles
+	// are walked in bands of token-tiles so that co-resident tiles share weight and token panels.
+	u32 const tiles_m = a_rows / gt::M_PER_BLOCK;
+	constexpr u32 tiles_n = N_RAW / gt::N_PER_BLOCK;
 	u32 const total = tiles_m * tiles_n;
-	u32 lin = blockIdx.x + blockIdx.y * tiles_m;
-	if (total % 8 == 0) {
-		lin = (lin % 8) * (total / 8) + lin / 8;      // hardware deals workgroups round-robin to 8 XCDs
-	}
-	// walk tiles in bands of 8 token-tiles so co-resident tiles share weight and token panels
-	constexpr u32 BAND = 8;
-	u32 tile_m, tile_n;
-	{
+	u32 const n_groups = gridDim.x * gridDim.y * gridDim.z;
+	u32 const group = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+	auto tile_coords = [&](u32 lin, u32 &tile_m, u32 &tile_n) {
+		constexpr u32 BAND = 2048 / gt::M_PER_BLOCK;
+		if (total % 8 == 0) {
+			lin = (lin % 8) * (total / 8) + lin / 8;
+		}
 		u32 band_tiles = BAND * tiles_n;
 		u32 band = lin / band_tiles;
 		u32 in_band = lin % band_tiles;
 		u32 rows_in_band = (tiles_m - band * BAND) < BAND ? (tiles_m - band * BAND) : BAND;
 		tile_m = band * BAND + in_band % rows_in_band;
 		tile_n = in_band / rows_in_band;
+	};
+	if (group >= total) {
+		return;
 	}
 
 	u32 const tid = threadIdx.x;
@@ -283,110 +411,113 @@ void kernel(
 
 	LaneOffsets lo;
 	{
-		u32 r = lane >> 3, p = lane & 7;
+		u32 j = lane / CHUNKS, p = lane % CHUNKS;     // row inside a load unit, stored chunk position
 		X17_UNROLL for (u32 odd = 0; odd < 2; ++odd) {
-			// the 8 rows of a load unit start at a multiple of 8: row pair index & 7 = 4 * (unit & 1) + r / 2
-			u32 chunk = p ^ (4 * odd + (r >> 1));
-			lo.x_src[odd] = r * K_TOTAL + 16 * chunk;
-			lo.w_src[odd] = (64 * ((lane >> 5) & 1) + ((lane >> 3) & 3)) * K_TOTAL + 16 * chunk;
+			u32 key = ((odd * UNIT_ROWS + j) >> SWZ_SHIFT) & (CHUNKS - 1);
+			u32 chunk = p ^ key;
+			lo.x_src[odd] = j * K_TOTAL + 16 * chunk;
+			lo.w_src[odd] = (64 * ((j >> 2) & 1) + 4 * (j >> 3) + (j & 3)) * K_TOTAL + 16 * chunk;
 		}
 		lo.frag_row = (lane % 32) * ROW_BYTES;
 		lo.half = lane / 32;
-		lo.swz = (lane >> 1) & 7;
+		lo.swz = ((lane % 32) >> SWZ_SHIFT) & (CHUNKS - 1);
 	}
 
+	// ---- main loop.  A ring of STAGES LDS buffers; step ks consumes buffer ks % STAGES while the
+	// loads of steps ks+1 .. ks+STAGES-1 are in flight.  The one barrier per step sits before the last
+	// slice's MFMAs: behind it the first fragments of the next step are fetched, so LDS latency is
+	// covered by matrix-core time across the step boundary too.  The load stream runs across tile
+	// boundaries: the last steps of a tile already fetch the first stages of the workgroup's next
+	// tile, which then land while the epilogue runs.
+	static_assert(K_STEPS + 1 >= gt::STAGES, "K too short for the LDS ring");
+	u32 const x_off = wm * gt::WAVE_M * ROW_BYTES + lo.frag_row;
+	u32 const w_off = X_TILE_BYTES + wn * 128 * ROW_BYTES + lo.frag_row;
+
+	// this wave's loads of one stage are dealt out over the first LOAD_SLICES slices of a step
+#ifndef X17_GEMM_LOAD_SLICES
+#define X17_GEMM_LOAD_SLICES (SLICES >= 4 ? 2 : 1)
+#endif
+	constexpr u32 LOAD_SLICES = X17_GEMM_LOAD_SLICES;
+	static_assert(LOAD_SLICES >= 1 && LOAD_SLICES < SLICES && LOAD_SLICES <= 3);
+	constexpr u32 LOADS_PER_SLICE = (LOADS_PER_STAGE + LOAD_SLICES - 1) / LOAD_SLICES;
+	constexpr u32 LOADS_END_1 = 2 * LOADS_PER_SLICE < LOADS_PER_STAGE ? 2 * LOADS_PER_SLICE : LOADS_PER_STAGE;
+
+	u32 tile_m, tile_n;
+	tile_coords(group, tile_m, tile_n);
 	u8 const *a_tile = a + (size_t)(tile_m * gt::M_PER_BLOCK) * K_TOTAL;
 	u8 const *b_tile = b + (size_t)(tile_n * gt::N_PER_BLOCK) * K_TOTAL;
-
-	Acc acc[4][BM];   // [bn][bm]
-	X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
-		X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
-			X17_UNROLL for (int r = 0; r < 16; ++r) acc[bn][bm][r] = 0;
-		}
+	X17_UNROLL for (u32 s = 0; s + 1 < gt::STAGES; ++s) {
+		issue_stage_loads<0, LOADS_PER_STAGE>(a_tile, b_tile, smem + s * STAGE_BYTES, s * gt::K_STEP, wave, lo);
 	}
 
-	issue_stage_loads(a_tile, b_tile, smem, 0, wave, lo);
-
-	for (u32 ks = 0; ks < K_STEPS; ++ks) {
-		__builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this step's tiles are in LDS
-		__syncthreads();                      // ... for every wave, and step ks-1 is fully consumed
-		if (ks + 1 < K_STEPS) {
-			issue_stage_loads(a_tile, b_tile, smem + ((ks + 1) % gt::STAGES) * STAGE_BYTES,
-			                  (ks + 1) * gt::K_STEP, wave, lo);
+	u32 buf = 0;                                   // ring position of the step being consumed
+	for (u32 lin = group; lin < total; lin += n_groups) {
+		bool const has_next = lin + n_groups < total;
+		u32 next_m = 0, next_n = 0;
+		if (has_next) {
+			tile_coords(lin + n_groups, next_m, next_n);
 		}
-		u8 const *x_tile = smem + (ks % gt::STAGES) * STAGE_BYTES + wm * gt::WAVE_M * ROW_BYTES + lo.frag_row;
-		u8 const *w_tile = smem + (ks % gt::STAGES) * STAGE_BYTES + X_TILE_BYTES + wn * 128 * ROW_BYTES + lo.frag_row;
+		u8 const *a_next = a + (size_t)(next_m * gt::M_PER_BLOCK) * K_TOTAL;
+		u8 const *b_next = b + (size_t)(next_n * gt::N_PER_BLOCK) * K_TOTAL;
 
-		if constexpr (MMA == 0) {
-			// 32 bytes of K per MFMA; operand fragments of slice s+1 are fetched before the
-			// MFMAs of slice s are issued, so LDS latency hides under matrix-core time
-			v4i wf[2][4], xf[2][BM];
-			X17_UNROLL for (int bn = 0; bn < 4; ++bn) wf[0][bn] = lds_chunk(w_tile, bn * 32 * ROW_BYTES, lo.half, lo.swz);
-			X17_UNROLL for (int bm = 0; bm < BM; ++bm) xf[0][bm] = lds_chunk(x_tile, bm * 32 * ROW_BYTES, lo.half, lo.swz);
-			X17_UNROLL for (u32 s = 0; s < 4; ++s) {
-				if (s + 1 < 4) {
-					u32 kc = 2 * (s + 1) + lo.half;
-					X17_UNROLL for (int bn = 0; bn < 4; ++bn) wf[(s + 1) & 1][bn] = lds_chunk(w_tile, bn * 32 * ROW_BYTES, kc, lo.swz);
-					X17_UNROLL for (int bm = 0; bm < BM; ++bm) xf[(s + 1) & 1][bm] = lds_chunk(x_tile, bm * 32 * ROW_BYTES, kc, lo.swz);
-				}
-				X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
-					X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
-						acc[bn][bm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[s & 1][bn], xf[s & 1][bm], acc[bn][bm], 0, 0, 0);
-					}
-				}
-				// pin the issue order: two MFMAs, then one of the eight LDS reads of the next slice
-				if (s + 1 < 4) {
-					X17_UNROLL for (int i = 0; i < 4 + BM; ++i) {
-						__builtin_amdgcn_sched_group_barrier(0x008, (4 * BM) / (4 + BM), 0);
-						__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-					}
+		Acc acc[4][BM];   // [bn][bm]
+		X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
+			X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
+				X17_UNROLL for (int r = 0; r < 16; ++r) acc[bn][bm][r] = 0;
+			}
+		}
+
+		// stage 0 of this tile has landed, for every wave, and nobody still reads the previous tile's buffers
+		// (vmcnt(0) rather than a stage count: the previous tile's output stores are in the same counter)
+		__builtin_amdgcn_s_waitcnt(0x0070);        // vmcnt(0) lgkmcnt(0)
+		__syncthreads();
+
+		Frags frags[2];
+		load_frags(frags[0], smem + buf * STAGE_BYTES + w_off, smem + buf * STAGE_BYTES + x_off, 0, lo);
+
+		for (u32 ks = 0; ks < K_STEPS; ++ks) {
+			u32 const load_buf = buf == 0 ? gt::STAGES - 1 : buf - 1;    // consumed by the previous step
+			u32 const next_buf = buf + 1 == gt::STAGES ? 0 : buf + 1;
+			u32 const load_step = ks + gt::STAGES - 1;
+			bool const this_tile = load_step < K_STEPS;
+			bool const more_loads = this_tile || has_next;
+			u8 const *la = this_tile ? a_tile : a_next;
+			u8 const *lb = this_tile ? b_tile : b_next;
+			u32 const load_k0 = (this_tile ? load_step : load_step - K_STEPS) * gt::K_STEP;
+			u8 *load_stage = smem + load_buf * STAGE_BYTES;
+			u8 const *stage = smem + buf * STAGE_BYTES;
+			X17_UNROLL for (u32 s = 0; s < SLICES; ++s) {
+				bool reads = true;
+				if (s + 1 < SLICES) {
+					load_frags(frags[(s + 1) & 1], stage + w_off, stage + x_off, s + 1, lo);
+				} else if (ks + 1 < K_STEPS) {
+					u32 remaining = has_next ? gt::STAGES : K_STEPS - 2 - ks;      // stages issued after ks+1
+					wait_stage(remaining < gt::STAGES - 2 ? remaining : gt::STAGES - 2);
+					__builtin_amdgcn_s_waitcnt(0xC07F);    // lgkmcnt(0): this wave is done reading buffer `buf`
+					__syncthreads();
+					u8 const *next = smem + next_buf * STAGE_BYTES;
+					load_frags(frags[(s + 1) & 1], next + w_off, next + x_off, 0, lo);
 				} else {
-					__builtin_amdgcn_sched_group_barrier(0x008, 4 * BM, 0);
+					reads = false;
 				}
-			}
-		} else if constexpr (MMA == 1) {
-			X17_UNROLL for (u32 s = 0; s < 2; ++s) {            // 64 bytes of K per MFMA
-				v8i wf[4], xf[BM];
-				u32 kc = 4 * s + 2 * lo.half;
-				X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
-					v4i lo4 = lds_chunk(w_tile, bn * 32 * ROW_BYTES, kc, lo.swz);
-					v4i hi4 = lds_chunk(w_tile, bn * 32 * ROW_BYTES, kc + 1, lo.swz);
-					wf[bn] = v8i{lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
-				}
-				X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
-					v4i lo4 = lds_chunk(x_tile, bm * 32 * ROW_BYTES, kc, lo.swz);
-					v4i hi4 = lds_chunk(x_tile, bm * 32 * ROW_BYTES, kc + 1, lo.swz);
-					xf[bm] = v8i{lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
-				}
-				X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
-					X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
-						v16f r = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-							wf[bn], xf[bm], __builtin_bit_cast(v16f, acc[bn][bm]), 0, 0, 0, 0, 0, 0);
-						acc[bn][bm] = __builtin_bit_cast(Acc, r);
+				if (more_loads) {
+					if (s == 0) issue_stage_loads<0, LOADS_PER_SLICE>(la, lb, load_stage, load_k0, wave, lo);
+					if constexpr (LOAD_SLICES >= 2) {
+						if (s == 1) issue_stage_loads<LOADS_PER_SLICE, LOADS_END_1>(la, lb, load_stage, load_k0, wave, lo);
+					}
+					if constexpr (LOAD_SLICES >= 3) {
+						if (s == 2) issue_stage_loads<LOADS_END_1, LOADS_PER_STAGE>(la, lb, load_stage, load_k0, wave, lo);
 					}
 				}
-			}
-		} else {
-			X17_UNROLL for (u32 s = 0; s < 4; ++s) {            // 32 bytes of K = two bf16 MFMAs of 16
-				u32 kc = 2 * s + lo.half;
-				v4i wraw[4], xraw[BM];
-				X17_UNROLL for (int bn = 0; bn < 4; ++bn) wraw[bn] = lds_chunk(w_tile, bn * 32 * ROW_BYTES, kc, lo.swz);
-				X17_UNROLL for (int bm = 0; bm < BM; ++bm) xraw[bm] = lds_chunk(x_tile, bm * 32 * ROW_BYTES, kc, lo.swz);
-				X17_UNROLL for (int h = 0; h < 2; ++h) {
-					v8bf wf[4], xf[BM];
-					X17_UNROLL for (int bn = 0; bn < 4; ++bn) wf[bn] = widen8(wraw[bn][2 * h], wraw[bn][2 * h + 1], B_KIND);
-					X17_UNROLL for (int bm = 0; bm < BM; ++bm) xf[bm] = widen8(xraw[bm][2 * h], xraw[bm][2 * h + 1], A_KIND);
-					X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
-						X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
-							v16f r = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-								wf[bn], xf[bm], __builtin_bit_cast(v16f, acc[bn][bm]), 0, 0, 0);
-							acc[bn][bm] = __builtin_bit_cast(Acc, r);
-						}
-					}
+				mma_slice(frags[s & 1], acc);
+				if (s < LOAD_SLICES) {
+					interleave_slice<(LOAD_SLICES == 1 ? 0 : LOADS_PER_SLICE)>(reads);
+				} else {
+					interleave_slice<0>(reads);
 				}
 			}
+			buf = next_buf;
 		}
-	}
 
 	// ---- epilogue.  Lane owns token (32*bm + lane%32) of its wave and raw columns
 	// 64*(lane/32) + 16*bn + r of its wave, r = accumulator register index.
@@ -490,5 +621,11 @@ void kernel(
 			}
 		}
 #endif
+	}
+
+		tile_m = next_m;
+		tile_n = next_n;
+		a_tile = a_next;
+		b_tile = b_next;
 	}
 }

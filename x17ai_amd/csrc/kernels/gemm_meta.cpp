@@ -10,6 +10,7 @@ int main() {
 	std::printf("\t\"THREADS_PER_BLOCK\": %u,\n", gt::THREADS_PER_BLOCK);
 	std::printf("\t\"SMEM_BYTES\": %u,\n", gt::SMEM_BYTES);
 	std::printf("\t\"M_PER_BLOCK\": %u,\n", gt::M_PER_BLOCK);
-	std::printf("\t\"N_PER_BLOCK\": %u\n", gt::N_PER_BLOCK);
+	std::printf("\t\"N_PER_BLOCK\": %u,\n", gt::N_PER_BLOCK);
+	std::printf("\t\"MAX_BLOCKS\": %u\n", gt::MAX_BLOCKS);
 	std::printf("}\n");
 }
