@@ -20,8 +20,8 @@
 //     a ring of LDS stages (gemm_tile.h: K_STEP bytes of K per step), one barrier per step;
 //     16-byte chunks are XOR-swizzled so that ds_read_b128 is conflict-free.
 //   * int8: v_mfma_i32_32x32x32_i8.  e4m3 x e4m3: v_mfma_f32_32x32x64_f8f6f4.  Mixed
-//     e4m3 x int8: both widened exactly to bf16 in registers, v_mfma_f32_32x32x16_bf16
-//     (int8 codes need 7 significand bits, e4m3 has 4).
+//     e4m3 x int8: both widened exactly to f16 in registers, v_mfma_f32_32x32x16_f16
+//     (int8 codes need 7 significand bits, e4m3 has 4; every e4m3 value is a normal f16).
 //   * Workgroup ids are remapped so that each XCD (own L2) works on a compact block of tiles.
 //
 // common.h (generated per kernel by the host-side kernel builder) provides:
@@ -46,7 +46,7 @@ constexpr int B_KIND = X17_B_KIND;
 constexpr int EPILOGUE = X17_EPILOGUE;
 constexpr int STORE = X17_STORE;
 
-// 0: int8 MFMA, 1: fp8 MFMA, 2: bf16 MFMA after widening
+// 0: int8 MFMA, 1: fp8 MFMA, 2: f16 MFMA after widening
 constexpr int MMA = (A_KIND == 0 && B_KIND == 0) ? 0 : ((A_KIND == 1 && B_KIND == 1) ? 1 : 2);
 constexpr bool ACC_F32 = MMA != 0;
 
@@ -255,29 +255,33 @@ X17_DEV v4i lds_chunk(u8 const *tile, u32 row_off, u32 kc, u32 swz) {
 	return *reinterpret_cast<v4i const *>(tile + row_off + ((kc ^ swz) << 4));
 }
 
-X17_DEV v8bf widen8(u32 lo, u32 hi, int kind) {
-	// eight 8-bit values -> eight bf16 (exact for int8 codes and for e4m3)
-	u32 w[2] = {lo, hi};
-	u32 out[4];
-	X17_UNROLL for (int i = 0; i < 4; ++i) {
-		u32 b0 = (w[i / 2] >> (16 * (i % 2))) & 0xFFu;
-		u32 b1 = (w[i / 2] >> (16 * (i % 2) + 8)) & 0xFFu;
-		u32 h0, h1;
-		if (kind == 1) {
-			h0 = e4m3_to_bf16_bits(b0);
-			h1 = e4m3_to_bf16_bits(b1);
-		} else {
-			h0 = f2u(f32((i32)(i8)b0)) >> 16;
-			h1 = f2u(f32((i32)(i8)b1)) >> 16;
+// Eight 8-bit values (two registers) -> eight f16, exact for both kinds.
+//   e4m3: the gfx950 packed fp8 -> f16 conversion (scale 1).  It reads OCP e4m3; the codes the
+//         reference's encoder produces (no subnormals, no NaN, no -0) mean the same in both.
+//   int8: flip the sign bit (b + 128 as an unsigned byte u), splice u under the f16 exponent of 1024
+//         (0x6400 | u == 1024 + u) and subtract 1152 -- five instructions per four bytes.
+X17_DEV v8h widen8(u32 lo, u32 hi, int kind) {
+	v2h p[4];
+	if (kind == 1) {
+		p[0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, false);
+		p[1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, true);
+		p[2] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, false);
+		p[3] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, true);
+	} else {
+		v2h const bias = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+		u32 w[2] = {lo ^ 0x80808080u, hi ^ 0x80808080u};
+		X17_UNROLL for (int i = 0; i < 2; ++i) {
+			u32 l = __builtin_amdgcn_perm(0x64646464u, w[i], 0x04010400u);
+			u32 h = __builtin_amdgcn_perm(0x64646464u, w[i], 0x04030402u);
+			p[2 * i] = __builtin_bit_cast(v2h, l) + bias;
+			p[2 * i + 1] = __builtin_bit_cast(v2h, h) + bias;
 		}
-		out[i] = h0 | (h1 << 16);
 	}
-	v4u packed = {out[0], out[1], out[2], out[3]};
-	return __builtin_bit_cast(v8bf, packed);
+	return v8h{p[0][0], p[0][1], p[1][0], p[1][1], p[2][0], p[2][1], p[3][0], p[3][1]};
 }
 
 // Operand fragments of one K slice (what one round of 4 x BM MFMA blocks consumes) and the MFMAs
-// themselves, per arithmetic: 32 bytes of K for int8 and for the bf16-widened mix, 64 for e4m3.
+// themselves, per arithmetic: 32 bytes of K for int8 and for the f16-widened mix, 64 for e4m3.
 constexpr u32 SLICE_BYTES = MMA == 1 ? 64 : 32;
 constexpr u32 SLICES = gt::K_STEP / SLICE_BYTES;
 constexpr u32 CHUNKS_PER_FRAG = SLICE_BYTES / 32;           // 16-byte chunks a lane fetches per operand row
@@ -321,13 +325,13 @@ X17_DEV void mma_slice(Frags const &f, Acc (&acc)[4][BM]) {
 			}
 		}
 	} else {
-		X17_UNROLL for (int h = 0; h < 2; ++h) {                // two bf16 MFMAs of K = 16
-			v8bf wf[4], xf[BM];
+		X17_UNROLL for (int h = 0; h < 2; ++h) {                // two f16 MFMAs of K = 16
+			v8h wf[4], xf[BM];
 			X17_UNROLL for (int bn = 0; bn < 4; ++bn) wf[bn] = widen8(f.w[bn][0][2 * h], f.w[bn][0][2 * h + 1], B_KIND);
 			X17_UNROLL for (int bm = 0; bm < BM; ++bm) xf[bm] = widen8(f.x[bm][0][2 * h], f.x[bm][0][2 * h + 1], A_KIND);
 			X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
 				X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
-					v16f r = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+					v16f r = __builtin_amdgcn_mfma_f32_32x32x16_f16(
 						wf[bn], xf[bm], __builtin_bit_cast(v16f, acc[bn][bm]), 0, 0, 0);
 					acc[bn][bm] = __builtin_bit_cast(Acc, r);
 				}
