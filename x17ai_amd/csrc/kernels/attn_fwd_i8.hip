@@ -14,20 +14,25 @@
 //
 // Design, MI355X-first:
 //   * One workgroup = 4 wavefronts = 128 queries of one head; a wavefront owns 32 queries.
-//     Keys/values are staged 32 keys per step (two 16-key tiles), double-buffered in LDS.
+//     Keys/values are staged 32 keys per step (two 16-key tiles) through rings in LDS.
 //   * S^T = K . Q^T on v_mfma_i32_32x32x32_i8 with the KEYS as the MFMA "A" operand: a lane then
 //     owns one query (lane % 32) and 8 keys of each 16-key tile; the other 8 keys sit in lane+32.
 //     Row max needs one cross-lane exchange per tile; the four per-quad partial sums of the
 //     reference fall two-and-two into the lane pair, so they need none until the very end.
-//   * P stays in registers: packed to bf16 it already IS the "B" operand of O^T = V^T . P^T.
-//     PV runs on v_mfma_f32_32x32x16_bf16: K = 16 is exactly one 16-key tile, P (0..255) and
-//     int8 V are exact in bf16 and every tile sum is below 2^24, so the f32 result equals the
+//   * P stays in registers: packed to f16 it already IS the "B" operand of O^T = V^T . P^T.
+//     PV runs on v_mfma_f32_32x32x16_f16: K = 16 is exactly one 16-key tile, P (0..255) and
+//     int8 V are exact in f16 and every tile sum is below 2^24, so the f32 result equals the
 //     reference's f32(int32 dot) bit for bit.  (CDNA4 has no unsigned x signed int8 MFMA; an
 //     int8 PV would need two MFMAs per tile for the 8-bit probabilities.)
-//   * V is widened to bf16 once per workgroup on its way into LDS and fetched transposed with
-//     ds_read_b64_tr_b16, so no register transposes; K goes global -> LDS directly.
+//   * K and V go global -> LDS directly, three 32-key steps ahead of their use.  V is widened to
+//     f16 once per workgroup, LDS -> LDS, one step ahead (sign-bit flip, byte splice under the
+//     exponent of 1024, subtract 1152: five instructions per four values) and fetched transposed
+//     with ds_read_b64_tr_b16, so no register transposes.
+//   * Three workgroups share a compute unit (register budget of 168 per lane), so one workgroup's
+//     waits for its tiles and its barrier are covered by the others' arithmetic.
 //   * X17_STRICT_MATH = 1: deterministic ex2 and one explicit f32 add per tile (parity build).
-//     X17_STRICT_MATH = 0: v_exp_f32 and accumulation inside the PV MFMA (speed build).
+//     X17_STRICT_MATH = 0: v_exp_f32 with the factor 255 folded into the exponent, and accumulation
+//     inside the PV MFMA (speed build).
 //
 // common.h (generated per kernel) provides X17_N_HEADS, X17_HEAD_DIM, X17_Q_STRIDE,
 // X17_KV_STRIDE, X17_O_STRIDE, X17_STRICT_MATH.
@@ -59,6 +64,7 @@ static_assert(HD == 32 || HD == 64 || HD == 128, "head_dim must be 32, 64 or 128
 static_assert(N_HEADS % HPK == 0, "n_heads must be divisible by heads_per_kernel");
 
 constexpr f32 PROB_SCALE = 255.0f;                                  // cuda/attn_fwd_i8.cuh:206
+constexpr f32 LOG2_PROB_SCALE = 7.9943534368588578f;                // lg2(255)
 constexpr f32 BASE_TEMPERATURE = f32(constexpr_inv_sqrt(f64(HD)) / 64.0);   // :47, :447-449
 
 typedef short v4s __attribute__((ext_vector_type(4)));
@@ -84,7 +90,7 @@ X17_DEV u32 k_chunk_offset(u32 key, u32 c) {
 	return (line << 7) | (((n & 7) ^ ((line >> 1) & 7)) << 4);
 }
 
-// V tile (bf16): linear 32-byte granule n = key * CPR + c (16 dims) lives in 256-byte line n / 8
+// V tile (f16): linear 32-byte granule n = key * CPR + c (16 dims) lives in 256-byte line n / 8
 // at position (n % 8) ^ ((line & 3) << 1): the 4 keys x 2 granules that 32 lanes of a transposed
 // read touch then cover all 64 banks exactly once (checked exhaustively for head_dim 32/64/128).
 X17_DEV u32 v_granule_offset(u32 key, u32 c) {
@@ -93,14 +99,15 @@ X17_DEV u32 v_granule_offset(u32 key, u32 c) {
 	return (line << 8) | (((n & 7) ^ ((line & 3) << 1)) << 5);
 }
 
-X17_DEV u32 pack_bf16(f32 lo, f32 hi) {
-	// both values are exactly representable in bf16: keep the upper halves
-	return __builtin_amdgcn_perm(f2u(hi), f2u(lo), 0x07060302u);
+X17_DEV u32 pack_f16(f32 lo, f32 hi) {
+	// both values are integers below 2048: exact in f16 whatever the rounding mode
+	return __builtin_bit_cast(u32, __builtin_amdgcn_cvt_pkrtz(lo, hi));
 }
 
 } // namespace
 
 extern "C" __global__ __launch_bounds__(at::THREADS_PER_BLOCK)
+__attribute__((amdgpu_waves_per_eu(at::WAVES_PER_SIMD, at::WAVES_PER_SIMD)))
 void kernel(
 	u32 seq_len,
 	i8 const *q,
@@ -140,41 +147,58 @@ void kernel(
 		i8 const *q_head = q + row_base * Q_STRIDE + (size_t)head * HD;
 		i8 const *kv_head = kv + row_base * KV_STRIDE + (size_t)head * 2 * HD;
 
-		// ---- staging helpers for one 32-key block
-		auto issue_k_load = [&](u32 kb, u32 stage) {
-			if (tid < 32 * CPR) {
-				// lane `tid` fills stored chunk `tid` of the K tile; find which logical chunk lives there
-				u32 line = tid >> 3;
-				u32 n = (line << 3) | ((tid & 7) ^ ((line >> 1) & 7));
-				u32 key = n / CPR, c = n % CPR;
-				i8 const *src = kv_head + (size_t)(kb * at::KV_PER_STEP + key) * KV_STRIDE + c * 16;
-				u8 *dst = smem + stage * at::STAGE_BYTES + (tid / 64) * 1024;
-				__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(src), X17_LDS_PTR(dst), 16, 0, 0);
+		// ---- staging helpers for one 32-key block.  Both K and V travel global -> LDS without passing
+		// through registers (thread t fetches 16-byte chunk t of each tile), PREFETCH steps ahead; one step
+		// before its use a V tile is widened LDS -> LDS by the threads that fetched it.
+		bool const stager = tid < 32 * CPR;
+		u32 stage_k_src = 0, stage_v_src = 0, widen_dst = 0;
+		if (stager) {
+			// lane `tid` fills stored chunk `tid` of the K tile; find which logical chunk lives there
+			u32 line = tid >> 3;
+			u32 n = (line << 3) | ((tid & 7) ^ ((line >> 1) & 7));
+			stage_k_src = (n / CPR) * KV_STRIDE + (n % CPR) * 16;
+			stage_v_src = (tid / CPR) * KV_STRIDE + HD + (tid % CPR) * 16;
+			widen_dst = v_granule_offset(tid / CPR, tid % CPR);
+		}
+		u32 const stage_lds = (tid / 64) * 1024;          // wave-uniform part of the direct-to-LDS address
+		auto issue_kv_load = [&](u32 kb, u32 slot) {
+			if (stager) {
+				i8 const *src = kv_head + (size_t)(kb * at::KV_PER_STEP) * KV_STRIDE;
+				u8 *k_dst = smem + at::K_RING_OFFSET + slot * at::K_TILE_BYTES + stage_lds;
+				u8 *v_dst = smem + at::RAW_V_RING_OFFSET + slot * at::RAW_V_TILE_BYTES + stage_lds;
+				__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(src + stage_k_src), X17_LDS_PTR(k_dst), 16, 0, 0);
+				__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(src + stage_v_src), X17_LDS_PTR(v_dst), 16, 0, 0);
 			}
 		};
-		auto load_v = [&](u32 kb) -> v4i {
-			v4i v = {0, 0, 0, 0};
-			if (tid < 32 * CPR) {
-				u32 key = tid / CPR, c = tid % CPR;
-				v = *reinterpret_cast<v4i const *>(kv_head + (size_t)(kb * at::KV_PER_STEP + key) * KV_STRIDE + HD + c * 16);
-			}
-			return v;
-		};
-		auto store_v = [&](v4i raw, u32 stage) {
-			if (tid < 32 * CPR) {
-				u32 key = tid / CPR, c = tid % CPR;
+		auto widen_v = [&](u32 slot, u32 tile) {
+			if (stager) {
+				v4u raw = *reinterpret_cast<v4u const *>(smem + at::RAW_V_RING_OFFSET + slot * at::RAW_V_TILE_BYTES + tid * 16);
+				// int8 -> f16: b + 128 as an unsigned byte u, 0x6400 | u == 1024 + u, minus 1152
+				v2h const bias = {(_Float16)-1152.0f, (_Float16)-1152.0f};
 				u32 w[8];
-				X17_UNROLL for (int i = 0; i < 8; ++i) {
-					u32 word = (u32)raw[i / 2];
-					u32 b0 = (word >> (16 * (i % 2))) & 0xFFu;
-					u32 b1 = (word >> (16 * (i % 2) + 8)) & 0xFFu;
-					w[i] = (f2u(f32((i32)(i8)b0)) >> 16) | (f2u(f32((i32)(i8)b1)) & 0xFFFF0000u);
+				X17_UNROLL for (int i = 0; i < 4; ++i) {
+					u32 word = raw[i] ^ 0x80808080u;
+					u32 l = __builtin_amdgcn_perm(0x64646464u, word, 0x04010400u);
+					u32 h = __builtin_amdgcn_perm(0x64646464u, word, 0x04030402u);
+					w[2 * i] = __builtin_bit_cast(u32, __builtin_bit_cast(v2h, l) + bias);
+					w[2 * i + 1] = __builtin_bit_cast(u32, __builtin_bit_cast(v2h, h) + bias);
 				}
-				u8 *dst = smem + stage * at::STAGE_BYTES + at::K_TILE_BYTES + v_granule_offset(key, c);
+				u8 *dst = smem + at::V_TILES_OFFSET + tile * at::V_TILE_BYTES + widen_dst;
 				*reinterpret_cast<v4u *>(dst) = v4u{w[0], w[1], w[2], w[3]};
 				*reinterpret_cast<v4u *>(dst + 16) = v4u{w[4], w[5], w[6], w[7]};
 			}
 		};
+		// each staging thread has two loads in flight per prefetched step; they complete in issue order
+		auto wait_steps_in_flight = [&](u32 steps) {
+			if (steps >= 2) {
+				__builtin_amdgcn_s_waitcnt(0x0F74);          // vmcnt(4)
+			} else if (steps == 1) {
+				__builtin_amdgcn_s_waitcnt(0x0F72);          // vmcnt(2)
+			} else {
+				__builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0)
+			}
+		};
+		static_assert(at::PREFETCH == 3, "the waits below are written for a prefetch distance of 3");
 
 		// ---- per-query setup (cuda/attn_fwd_i8.cuh:444-517)
 		v4i qf[K_SLICES];
@@ -207,24 +231,31 @@ void kernel(
 		}
 
 		// ---- pipeline prologue
+		u32 const n_steps = kb_end - kb_begin;
 		__syncthreads();                      // previous head's tiles are no longer read
-		issue_k_load(kb_begin, 0);
-		store_v(load_v(kb_begin), 0);
+		X17_UNROLL for (u32 j = 0; j < at::PREFETCH; ++j) {
+			if (j < n_steps) issue_kv_load(kb_begin + j, j);
+		}
+		wait_steps_in_flight((n_steps < at::PREFETCH ? n_steps : at::PREFETCH) - 1);
+		widen_v(0, 0);
 
-		for (u32 kb = kb_begin; kb < kb_end; ++kb) {
-			u32 const stage = (kb - kb_begin) % at::STAGES;
-			__builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): this block's K tile has landed
-			__syncthreads();
-			v4i v_next = {0, 0, 0, 0};
-			bool const has_next = kb + 1 < kb_end;
-			if (has_next) {
-				issue_k_load(kb + 1, stage ^ 1);
-				v_next = load_v(kb + 1);
+		for (u32 i = 0; i < n_steps; ++i) {
+			u32 const kb = kb_begin + i;
+			u32 const slot = i % at::RING;
+			// K tile i and raw V tile i+1 have landed (this thread's chunks), at most step i+2 stays in flight
+			wait_steps_in_flight(i + 2 < n_steps ? 1 : 0);
+			__builtin_amdgcn_s_waitcnt(0xC07F);          // lgkmcnt(0): own LDS traffic of step i-1 is complete
+			__builtin_amdgcn_s_barrier();                // ... and so is everybody else's: tiles i are visible
+			if (i + at::PREFETCH < n_steps) {
+				issue_kv_load(kb + at::PREFETCH, (i + at::PREFETCH) % at::RING);
+			}
+			if (i + 1 < n_steps) {
+				widen_v((i + 1) % at::RING, (i + 1) & 1);
 			}
 
 			if (kb >= wave_kb_first && kb <= wave_kb_last) {
-				u8 const *k_tile = smem + stage * at::STAGE_BYTES;
-				u8 const *v_tile = k_tile + at::K_TILE_BYTES;
+				u8 const *k_tile = smem + at::K_RING_OFFSET + slot * at::K_TILE_BYTES;
+				u8 const *v_tile = smem + at::V_TILES_OFFSET + (i & 1) * at::V_TILE_BYTES;
 
 				// S^T block: rows = 32 keys, columns = this wave's 32 queries
 				v16i s_acc = {0};
@@ -264,7 +295,12 @@ void kernel(
 
 					// :265-290 -- p = ex2(s - max) * 255; partial sums over key quads; P = rne(p)
 					f32 p[8];
-					X17_UNROLL for (u32 r = 0; r < 8; ++r) p[r] = sfu::ex2(s[r] - m) * PROB_SCALE;
+					if constexpr (STRICT) {
+						X17_UNROLL for (u32 r = 0; r < 8; ++r) p[r] = sfu::ex2(s[r] - m) * PROB_SCALE;
+					} else {
+						f32 const shift = m - LOG2_PROB_SCALE;        // 255 * 2^(s - m) = 2^(s - (m - lg2 255))
+						X17_UNROLL for (u32 r = 0; r < 8; ++r) p[r] = sfu::ex2(s[r] - shift);
+					}
 					f32 add_lo = (p[0] + p[1]) + (p[2] + p[3]);
 					f32 add_hi = (p[4] + p[5]) + (p[6] + p[7]);
 					sum_lo = fmaf32(sum_lo, resc, add_lo);
@@ -272,9 +308,9 @@ void kernel(
 
 					v4u pp;
 					X17_UNROLL for (int w = 0; w < 4; ++w) {
-						pp[w] = pack_bf16(__builtin_rintf(p[2 * w]), __builtin_rintf(p[2 * w + 1]));
+						pp[w] = pack_f16(__builtin_rintf(p[2 * w]), __builtin_rintf(p[2 * w + 1]));
 					}
-					v8bf const pfrag = __builtin_bit_cast(v8bf, pp);
+					v8h const pfrag = __builtin_bit_cast(v8h, pp);
 
 					// :588-605 -- O += f32(P . V) for this 16-key tile
 					X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
@@ -291,21 +327,18 @@ void kernel(
 						}
 						typedef short v8s __attribute__((ext_vector_type(8)));
 						v8s both = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
-						v8bf const vfrag = __builtin_bit_cast(v8bf, both);
+						v8h const vfrag = __builtin_bit_cast(v8h, both);
 						if constexpr (STRICT) {
 							v16f zero = {0};
-							v16f pv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfrag, pfrag, zero, 0, 0, 0);
+							v16f pv = __builtin_amdgcn_mfma_f32_32x32x16_f16(vfrag, pfrag, zero, 0, 0, 0);
 							X17_UNROLL for (int r = 0; r < 16; ++r) o_acc[db][r] = o_acc[db][r] + pv[r];
 						} else {
-							o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfrag, pfrag, o_acc[db], 0, 0, 0);
+							o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vfrag, pfrag, o_acc[db], 0, 0, 0);
 						}
 					}
 				}
 			}
 
-			if (has_next) {
-				store_v(v_next, stage ^ 1);
-			}
 		}
 
 		// ---- finish (cuda/attn_fwd_i8.cuh:293-351): the lane pair holds partial sums (s0, s2) and (s1, s3)
@@ -322,13 +355,21 @@ void kernel(
 		f32 inv = strict::rcp(total);
 		i8 *o_row = out + (row_base + qi) * O_STRIDE + (size_t)head * HD;
 		X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
-			X17_UNROLL for (int r4 = 0; r4 < 4; ++r4) {
-				u32 word = 0;
+			// word g of this lane = dims 32*db + 8*g + 4*half .. +3
+			u32 word[4];
+			X17_UNROLL for (int g = 0; g < 4; ++g) {
+				word[g] = 0;
 				X17_UNROLL for (int b = 0; b < 4; ++b) {
-					word |= ((u32)f32_to_fixedi8(o_acc[db][4 * r4 + b] * inv) & 0xFFu) << (8 * b);
+					word[g] |= ((u32)f32_to_fixedi8(o_acc[db][4 * g + b] * inv) & 0xFFu) << (8 * b);
 				}
-				*reinterpret_cast<u32 *>(o_row + 32 * db + 8 * r4 + 4 * half) = word;
 			}
+			// The lane pair (lane, lane + 32) holds the 32 bytes of this block interleaved word by word; two
+			// cross-half swaps give the lower lane bytes 0..15 and the upper lane bytes 16..31, so that each
+			// lane writes one 16-byte vector.
+			auto a = __builtin_amdgcn_permlane32_swap(word[0], word[2], false, false);
+			auto b = __builtin_amdgcn_permlane32_swap(word[1], word[3], false, false);
+			v4u vec = {a[0], a[1], b[0], b[1]};
+			*reinterpret_cast<v4u *>(o_row + 32 * db + 16 * half) = vec;
 		}
 	}
 }

@@ -15,11 +15,23 @@ constexpr unsigned Q_PER_WAVE = 32;
 constexpr unsigned Q_PER_BLOCK = Q_WAVES * Q_PER_WAVE;      // 128 queries per workgroup
 constexpr unsigned KV_PER_STEP = 32;                         // keys staged per pipeline step
 constexpr unsigned THREADS_PER_BLOCK = WAVE * Q_WAVES;
-constexpr unsigned STAGES = 2;
+// K/V tiles are fetched PREFETCH steps ahead of their use into rings of PREFETCH + 1 slots
+constexpr unsigned PREFETCH = 3;
+constexpr unsigned RING = PREFETCH + 1;
+// Register budget: this many wavefronts (= workgroups) share a SIMD, so that one workgroup's waits for
+// its K/V tiles and its barrier are covered by the others' arithmetic.
+#ifndef X17_ATTN_WAVES_PER_SIMD
+#define X17_ATTN_WAVES_PER_SIMD (X17_STRICT_MATH ? 2 : 3)   // the deterministic transcendentals need more registers
+#endif
+constexpr unsigned WAVES_PER_SIMD = X17_ATTN_WAVES_PER_SIMD;
 
 constexpr unsigned K_TILE_BYTES = KV_PER_STEP * HEAD_DIM;        // int8 keys, row = one key
-constexpr unsigned V_TILE_BYTES = KV_PER_STEP * HEAD_DIM * 2;    // values widened to bf16
-constexpr unsigned STAGE_BYTES = K_TILE_BYTES + V_TILE_BYTES;
-constexpr unsigned SMEM_BYTES = STAGES * STAGE_BYTES;
+constexpr unsigned RAW_V_TILE_BYTES = KV_PER_STEP * HEAD_DIM;    // int8 values as they arrive
+constexpr unsigned V_TILE_BYTES = KV_PER_STEP * HEAD_DIM * 2;    // values widened to f16
+// LDS map: K ring | raw V ring | two f16 V tiles (the tile in use and the one being widened)
+constexpr unsigned K_RING_OFFSET = 0;
+constexpr unsigned RAW_V_RING_OFFSET = RING * K_TILE_BYTES;
+constexpr unsigned V_TILES_OFFSET = RAW_V_RING_OFFSET + RING * RAW_V_TILE_BYTES;
+constexpr unsigned SMEM_BYTES = V_TILES_OFFSET + 2 * V_TILE_BYTES;
 
 }} // namespace x17::attn_tile

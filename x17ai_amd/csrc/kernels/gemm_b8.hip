@@ -474,7 +474,7 @@ void kernel(
 		// stage 0 of this tile has landed, for every wave, and nobody still reads the previous tile's buffers
 		// (vmcnt(0) rather than a stage count: the previous tile's output stores are in the same counter)
 		__builtin_amdgcn_s_waitcnt(0x0070);        // vmcnt(0) lgkmcnt(0)
-		__syncthreads();
+		__builtin_amdgcn_s_barrier();
 
 		Frags frags[2];
 		load_frags(frags[0], smem + buf * STAGE_BYTES + w_off, smem + buf * STAGE_BYTES + x_off, 0, lo);
@@ -498,7 +498,7 @@ void kernel(
 					u32 remaining = has_next ? gt::STAGES : K_STEPS - 2 - ks;      // stages issued after ks+1
 					wait_stage(remaining < gt::STAGES - 2 ? remaining : gt::STAGES - 2);
 					__builtin_amdgcn_s_waitcnt(0xC07F);    // lgkmcnt(0): this wave is done reading buffer `buf`
-					__syncthreads();
+					__builtin_amdgcn_s_barrier();
 					u8 const *next = smem + next_buf * STAGE_BYTES;
 					load_frags(frags[(s + 1) & 1], next + w_off, next + x_off, 0, lo);
 				} else {
