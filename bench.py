@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized block-forward path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] [--only KERNEL] [--copy-probe]
 
 Headline (the JSON line's `value`): BASELINE config 2, the int8 FFN GEMM pair
   ffn_f_fwd   x[8192, 2048] i8 . W1[16384, 2048]^T  -> GeGLU   -> f[8192, 8192] FixedI8
@@ -269,6 +269,68 @@ def extras(dev, X, recipes):
 	return out
 
 
+def single(dev, X, recipes, name, iters):
+	"""One kernel of one BASELINE workload, launched `iters` times: what the rocprofv3 summaries under
+	profiles/ are taken from (every code object exports the entry `kernel`, so a profile of several
+	kernels at once cannot tell them apart by name)."""
+	rng = np.random.default_rng(3000)
+	D, F = 2048, 8192
+	if name == "ffn_f_config2":
+		M = 8192
+		a = X.Tensor.from_numpy(dev, _rand_codes(rng, (M, D)), X.INT8)
+		b = X.Tensor.from_numpy(dev, _rand_codes(rng, (2 * F, D)), X.INT8)
+		c = X.Tensor(dev, (M, F), X.INT8)
+		k = recipes.ffn_f_kernel(dev, D, 2 * F, False, X.INT8)
+		fn, work, unit = (lambda: k.launch(a, b, c)), k.n_ops(a, b) / 1e12, "TOPS"
+	elif name == "ffn_y_f8_config4":
+		M = 32768
+		a = X.Tensor.from_numpy(dev, rng.integers(0x20, 0x50, (M, F), dtype=np.uint8), X.E4M3)
+		b = X.Tensor.from_numpy(dev, _rand_codes(rng, (2 * D, F)), X.INT8)
+		r = X.Tensor.from_numpy(dev, _rand_codes(rng, (M, D)), X.INT8)
+		c = X.Tensor(dev, (M, D), X.E4M3)
+		k = recipes.ffn_y_kernel(dev, D, F, False)
+		fn, work, unit = (lambda: k.launch(a, b, c, r)), k.n_ops(a, b) / 1e12, "TFLOP/s"
+	elif name in ("attn_config4", "attn_config5"):
+		T, B, H, HD, W = (8192, 4, 16, 128, 512) if name == "attn_config4" else (65536, 1, 32, 128, 4096)
+		rows = T * B
+		q = X.Tensor.from_numpy(dev, _rand_codes(rng, (rows, H * HD)), X.INT8)
+		kv = X.Tensor.from_numpy(dev, _rand_codes(rng, (rows, 2 * H * HD)), X.INT8)
+		sk = X.Tensor.from_numpy(dev, _rand_codes(rng, (H, HD)), X.INT8)
+		sv = X.Tensor.from_numpy(dev, _rand_codes(rng, (H, HD)), X.INT8)
+		tp = X.Tensor.from_numpy(dev, (0.5 + rng.random(H)).astype(np.float32), X.F32)
+		o = X.Tensor(dev, (rows, H * HD), X.INT8)
+		l = X.Tensor(dev, (H, rows), X.F32)
+		k = recipes.attn_kernel(dev, H, HD, False)
+		pairs = W * (W - 1) // 2 + (T - W) * W
+		fn, work, unit = (lambda: k.launch(q, kv, sk, sv, tp, o, l, W, B)), 4.0 * HD * H * B * pairs / 1e12, "TOPS"
+	elif name == "decode_config5":
+		S5, CAP, H, HD, W = 64, 4096, 32, 128, 4096
+		one = _rand_codes(rng, (1, CAP, 2 * H * HD))
+		cache = X.Tensor.from_numpy(dev, np.ascontiguousarray(np.broadcast_to(one, (S5, CAP, 2 * H * HD))), X.INT8)
+		qd = X.Tensor.from_numpy(dev, _rand_codes(rng, (S5, H * HD)), X.INT8)
+		lens = X.Tensor.from_numpy(dev, np.full(S5, CAP, np.uint32).view(np.float32), X.F32)
+		sk = X.Tensor.from_numpy(dev, _rand_codes(rng, (H, HD)), X.INT8)
+		sv = X.Tensor.from_numpy(dev, _rand_codes(rng, (H, HD)), X.INT8)
+		tp = X.Tensor.from_numpy(dev, np.ones(H, np.float32), X.F32)
+		od = X.Tensor(dev, (S5, H * HD), X.INT8)
+		k = recipes.attn_decode_kernel(dev, H, HD, CAP, False)
+		fn, work, unit = (lambda: k.launch(qd, cache, lens, sk, sv, tp, od, None, W)), S5 * CAP * 2 * H * HD / 1e9, "GB/s"
+	elif name == "rms_norm_config4":
+		rows = 32768
+		xb = X.Tensor.from_numpy(dev, (rng.standard_normal((rows, D), dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16), X.BF16)
+		xi = X.Tensor(dev, (rows, D), X.INT8)
+		k = recipes.rms_norm_kernel(dev, D, X.BF16)
+		fn, work, unit = (lambda: k.launch(xb, xi)), rows * D * 3 / 1e9, "GB/s"
+	else:
+		raise SystemExit(f"bench.py: unknown --only target {name!r}")
+	med, mn = _median_launch(dev, X, fn, iters, 3)
+	print(json.dumps({"only": name, "launches": iters, "median_us": med * 1e6, "min_us": mn * 1e6,
+	                  "rate": work / med, "unit": unit}))
+
+
+ONLY_TARGETS = ("ffn_f_config2", "ffn_y_f8_config4", "attn_config4", "attn_config5", "decode_config5", "rms_norm_config4")
+
+
 def main():
 	ap = argparse.ArgumentParser()
 	ap.add_argument("--gpus", type=int, default=1)
@@ -278,6 +340,8 @@ def main():
 	ap.add_argument("--no-cpu", action="store_true")
 	ap.add_argument("--copy-probe", action="store_true",
 	                help="only run a 1 GiB device-to-device copy kernel (calibrates the HBM traffic counters)")
+	ap.add_argument("--only", choices=ONLY_TARGETS,
+	                help="launch one kernel of one workload --steps times and print its median (used for the profiles)")
 	args = ap.parse_args()
 	if args.gpus != 1:
 		print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -297,6 +361,9 @@ def main():
 			probe.launch(src, dst)
 		dev.synchronize()
 		print(json.dumps({"copy_probe_bytes_read": n, "copy_probe_bytes_written": n, "launches": 5}))
+		return
+	if args.only:
+		single(dev, X, recipes, args.only, args.steps)
 		return
 	h = headline(dev, X, recipes, args.steps, args.warmup)
 	value = h["ops_per_step"] * args.steps / h["wall_s"] / 1e12

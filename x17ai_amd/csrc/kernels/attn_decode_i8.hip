@@ -9,7 +9,8 @@
 // of the int32 P.V per tile.  So appending a token and decoding it gives bit for bit what a
 // prefill over the longer sequence gives for that row.
 //
-// The work is bandwidth: every cached K byte and V byte is read exactly once.  One workgroup
+// The work is bandwidth: every cached K byte is read exactly once, and so is every V row whose
+// 8-bit probability is not zero (rows with probability 0 contribute nothing and are not fetched).  One workgroup
 // per (sequence, head); the recurrence is cut into phases so that only two cheap scans remain
 // sequential:
 //   1  scores: HD/16 lanes per key row (16-byte coalesced loads), v_dot4 + lane reduction
@@ -90,21 +91,30 @@ void kernel(
 	}
 	f32 const m0 = f32(sink_dot) * temperature;
 
-	// ---- phase 1: scores of all keys of the walked tiles
+	// ---- phase 1: scores of all keys of the walked tiles.  A thread keeps BATCH independent 16-byte
+	// loads in flight (a load per pass would leave the kernel waiting on memory latency).
 	u32 const n_keys = n_tiles * 16;
-	for (u32 base = 0; base < n_keys; base += KEYS_PER_PASS) {
-		u32 kidx = base + tid / CPR;
-		u32 j = t0 * 16 + kidx;
-		bool in_range = kidx < n_keys;
-		bool vis = in_range && j >= j_lo && j < pos;
-		i32 dot = 0;
-		if (vis) {
-			v4i kc = *reinterpret_cast<v4i const *>(kv_head + (size_t)j * ROW + 16 * c);
-			X17_UNROLL for (int w = 0; w < 4; ++w) dot = __builtin_amdgcn_sdot4(qc[w], kc[w], dot, false);
+	constexpr u32 BATCH = 8;
+	for (u32 base = 0; base < n_keys; base += KEYS_PER_PASS * BATCH) {
+		v4i kc[BATCH];
+		X17_UNROLL for (u32 bb = 0; bb < BATCH; ++bb) {
+			u32 kidx = base + bb * KEYS_PER_PASS + tid / CPR;
+			u32 j = t0 * 16 + kidx;
+			bool vis = kidx < n_keys && j >= j_lo && j < pos;
+			u32 j_safe = vis ? j : pos - 1;                   // a row that exists (n_tiles > 0 means pos >= 1)
+			kc[bb] = *reinterpret_cast<v4i const *>(kv_head + (size_t)j_safe * ROW + 16 * c);
 		}
-		X17_UNROLL for (u32 mask = 1; mask < CPR; mask <<= 1) dot += __shfl_xor(dot, (int)mask, 64);
-		if (in_range && c == 0) {
-			s_score[kidx] = vis ? f32(dot) * temperature : -__builtin_inff();
+		X17_UNROLL for (u32 bb = 0; bb < BATCH; ++bb) {
+			u32 kidx = base + bb * KEYS_PER_PASS + tid / CPR;
+			u32 j = t0 * 16 + kidx;
+			bool in_range = kidx < n_keys;
+			bool vis = in_range && j >= j_lo && j < pos;
+			i32 dot = 0;
+			X17_UNROLL for (int w = 0; w < 4; ++w) dot = __builtin_amdgcn_sdot4(qc[w], kc[bb][w], dot, false);
+			X17_UNROLL for (u32 mask = 1; mask < CPR; mask <<= 1) dot += __shfl_xor(dot, (int)mask, 64);
+			if (in_range && c == 0) {
+				s_score[kidx] = vis ? f32(dot) * temperature : -__builtin_inff();
+			}
 		}
 	}
 	__syncthreads();
@@ -163,10 +173,17 @@ void kernel(
 	}
 	__syncthreads();
 
-	// ---- phase 3: the four partial-sum chains
+	// ---- phase 3: the four partial-sum chains (operands fetched eight tiles at a time, so the chain
+	// itself is the only serial part)
 	if (tid < 4) {
 		f32 sum = 63.75f;
-		for (u32 t = 0; t < n_tiles; ++t) sum = fmaf32(sum, s_resc[t], s_quad[t * 4 + tid]);
+		u32 t = 0;
+		for (; t + 8 <= n_tiles; t += 8) {
+			f32 r[8], a[8];
+			X17_UNROLL for (int i = 0; i < 8; ++i) { r[i] = s_resc[t + i]; a[i] = s_quad[(t + i) * 4 + tid]; }
+			X17_UNROLL for (int i = 0; i < 8; ++i) sum = fmaf32(sum, r[i], a[i]);
+		}
+		for (; t < n_tiles; ++t) sum = fmaf32(sum, s_resc[t], s_quad[t * 4 + tid]);
 		s_sum[tid] = sum;
 	}
 
@@ -184,13 +201,22 @@ void kernel(
 			i32 acc[16];
 			X17_UNROLL for (int i = 0; i < 16; ++i) acc[i] = 0;
 			v4u probs = *reinterpret_cast<v4u const *>(s_prob + t * 16);
+			// all loads of the tile first (only rows with a nonzero probability are fetched: masked keys have
+			// p == 0 and may lie outside the cache), then the arithmetic
+			v4i vv[16];
+			X17_UNROLL for (int k = 0; k < 16; ++k) {
+				u32 p = (probs[k / 4] >> (8 * (k % 4))) & 0xFFu;
+				u32 j = (t0 + t) * 16 + k;
+				vv[k] = v4i{0, 0, 0, 0};
+				if (p != 0) {
+					vv[k] = *reinterpret_cast<v4i const *>(kv_head + (size_t)j * ROW + HD + 16 * c);
+				}
+			}
 			X17_UNROLL for (int k = 0; k < 16; ++k) {
 				i32 p = (i32)((probs[k / 4] >> (8 * (k % 4))) & 0xFFu);
-				u32 j = (t0 + t) * 16 + k;
-				if (p != 0) {     // masked keys have p == 0 (and may lie outside the cache)
-					v4i vv = *reinterpret_cast<v4i const *>(kv_head + (size_t)j * ROW + HD + 16 * c);
+				if (p != 0) {     // after the 8-bit quantisation most keys far below the maximum carry no weight
 					X17_UNROLL for (int i = 0; i < 16; ++i) {
-						acc[i] += p * (i32)(i8)(((u32)vv[i / 4] >> (8 * (i % 4))) & 0xFFu);
+						acc[i] += p * (i32)(i8)(((u32)vv[k][i / 4] >> (8 * (i % 4))) & 0xFFu);
 					}
 				}
 			}
@@ -201,7 +227,17 @@ void kernel(
 		__syncthreads();
 		// 4b: one f32 multiply (rescale) and one f32 add per tile (:247-252, :588-605)
 		if (tid < HD) {
-			for (u32 tl2 = 0; tl2 < tiles_here; ++tl2) {
+			u32 tl2 = 0;
+			for (; tl2 + 8 <= tiles_here; tl2 += 8) {
+				f32 r[8];
+				i32 a[8];
+				X17_UNROLL for (int i = 0; i < 8; ++i) { r[i] = s_resc[chunk + tl2 + i]; a[i] = s_pv[(tl2 + i) * HD + tid]; }
+				X17_UNROLL for (int i = 0; i < 8; ++i) {
+					o = o * r[i];
+					o = o + f32(a[i]);
+				}
+			}
+			for (; tl2 < tiles_here; ++tl2) {
 				o = o * s_resc[chunk + tl2];
 				o = o + f32(s_pv[tl2 * HD + tid]);
 			}
