@@ -31,8 +31,8 @@
 //   * Three workgroups share a compute unit (register budget of 168 per lane), so one workgroup's
 //     waits for its tiles and its barrier are covered by the others' arithmetic.
 //   * X17_STRICT_MATH = 1: deterministic ex2 and one explicit f32 add per tile (parity build).
-//     X17_STRICT_MATH = 0: v_exp_f32 with the factor 255 folded into the exponent, and accumulation
-//     inside the PV MFMA (speed build).
+//     X17_STRICT_MATH = 0: v_exp_f32 with the factor 255 folded into the exponent, accumulation
+//     inside the PV MFMA, and lazy rescaling of O (speed build; results stay within one output code).
 //
 // common.h (generated per kernel) provides X17_N_HEADS, X17_HEAD_DIM, X17_Q_STRIDE,
 // X17_KV_STRIDE, X17_O_STRIDE, X17_STRICT_MATH.
@@ -65,6 +65,7 @@ static_assert(N_HEADS % HPK == 0, "n_heads must be divisible by heads_per_kernel
 
 constexpr f32 PROB_SCALE = 255.0f;                                  // cuda/attn_fwd_i8.cuh:206
 constexpr f32 LOG2_PROB_SCALE = 7.9943534368588578f;                // lg2(255)
+constexpr f32 MAX_LIFT = 64.0f;                                     // 255 * 64 stays far inside f16
 constexpr f32 BASE_TEMPERATURE = f32(constexpr_inv_sqrt(f64(HD)) / 64.0);   // :47, :447-449
 
 typedef short v4s __attribute__((ext_vector_type(4)));
@@ -129,7 +130,14 @@ void kernel(
 
 	u32 const seq = blockIdx.z;
 	size_t const row_base = (size_t)seq * seq_len;          // first row of this sequence
-	u32 const q_block0 = blockIdx.x * at::Q_PER_BLOCK;      // position of the block's first query
+	// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  When the number of query
+	// blocks is a multiple of 8, XCD k gets a contiguous eighth of the sequence, so that the query blocks
+	// resident on one XCD at a time are neighbours and share their K/V windows in its L2.
+	u32 q_block_index = blockIdx.x;
+	if (gridDim.x % 8 == 0) {
+		q_block_index = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
+	}
+	u32 const q_block0 = q_block_index * at::Q_PER_BLOCK;   // position of the block's first query
 	u32 const q_wave0 = q_block0 + wave * at::Q_PER_WAVE;
 	u32 const qi = q_wave0 + qlane;                         // this lane's query position
 
@@ -217,6 +225,9 @@ void kernel(
 		sink_dot += partner_i32(sink_dot, half);
 
 		f32 m = f32(sink_dot) * temperature;
+		f32 m_ref = m;                       // speed build: the maximum O's scale refers to, and 2^(m - m_ref)
+		f32 lift = 1.0f;
+		v2h lift2 = {(_Float16)1.0f, (_Float16)1.0f};
 		f32 sum_lo = 0.25f * PROB_SCALE;     // partial sum of key quad `half` of every tile
 		f32 sum_hi = 0.25f * PROB_SCALE;     // partial sum of key quad `2 + half`
 		// (the lane pair holds the reference's four partial sums two-and-two; each starts at 63.75)
@@ -288,8 +299,24 @@ void kernel(
 						f32 new_m = __builtin_fmaxf(tmax, m);
 						resc = sfu::ex2(m - new_m);      // exactly 1 for rows whose max did not move
 						m = new_m;
-						X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
-							X17_UNROLL for (int r = 0; r < 16; ++r) o_acc[db][r] = o_acc[db][r] * resc;
+						if constexpr (STRICT) {
+							X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
+								X17_UNROLL for (int r = 0; r < 16; ++r) o_acc[db][r] = o_acc[db][r] * resc;
+							}
+						} else {
+							// Speed build: O stays at the scale of an older maximum m_ref and the new probabilities are
+							// lifted to that scale instead (8 values instead of the 2 * head_dim / 4 accumulators);
+							// O is brought down only when the lift factor 2^(m - m_ref) of some query passes 64.
+							lift = sfu::ex2(m - m_ref);
+							if (__any(lift > MAX_LIFT)) {
+								f32 const down = sfu::rcp(lift);
+								X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
+									X17_UNROLL for (int r = 0; r < 16; ++r) o_acc[db][r] = o_acc[db][r] * down;
+								}
+								m_ref = m;
+								lift = 1.0f;
+							}
+							lift2 = v2h{(_Float16)lift, (_Float16)lift};      // round to nearest
 						}
 					}
 
@@ -308,7 +335,13 @@ void kernel(
 
 					v4u pp;
 					X17_UNROLL for (int w = 0; w < 4; ++w) {
-						pp[w] = pack_f16(__builtin_rintf(p[2 * w]), __builtin_rintf(p[2 * w + 1]));
+						u32 word = pack_f16(__builtin_rintf(p[2 * w]), __builtin_rintf(p[2 * w + 1]));
+						if constexpr (!STRICT) {
+							// integers up to 255 times a factor up to 64: in range, rounded to 11 bits
+							// (bit-casting a vector ELEMENT in place reads element 0, hence the scalar temporary)
+							word = __builtin_bit_cast(u32, __builtin_bit_cast(v2h, word) * lift2);
+						}
+						pp[w] = word;
 					}
 					v8h const pfrag = __builtin_bit_cast(v8h, pp);
 
@@ -353,6 +386,9 @@ void kernel(
 			l_out[(size_t)head * ((size_t)gridDim.z * seq_len) + row_base + qi] = strict::lg2(total) + m;
 		}
 		f32 inv = strict::rcp(total);
+		if constexpr (!STRICT) {
+			inv = inv * sfu::rcp(lift);
+		}
 		i8 *o_row = out + (row_base + qi) * O_STRIDE + (size_t)head * HD;
 		X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
 			// word g of this lane = dims 32*db + 8*g + 4*half .. +3
