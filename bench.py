@@ -37,7 +37,10 @@ PEAK_BF16_TFLOPS = 2500.0    # dense bf16
 PEAK_HBM_GBS = 8000.0        # HBM3E
 
 # HBM bytes per ffn_f launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), or None
-FFN_F_TRAFFIC_BYTES = int((196803 * 2.0 + 65536 * 1.0) * 1024)
+FFN_F_TRAFFIC_BYTES = int((196791 * 2.0 + 65536 * 1.0) * 1024)
+# HBM bytes one decode launch of config 5 fetches (profiles/attn_decode_i8_config5.txt): all K rows plus the
+# V rows with a nonzero 8-bit probability -- about half of the 2 GiB cache for the synthetic Gaussian codes
+DECODE_TRAFFIC_BYTES = int(529497 * 2.0 * 1024)
 
 
 def _rand_i8(rng, shape):
@@ -263,8 +266,9 @@ def extras(dev, X, recipes):
 		nbytes = S5 * CAP * 2 * H5 * HD5
 		tag = "strict" if strict else "fast"
 		c5[f"decode_{tag}_us"] = med * 1e6
-		c5[f"decode_{tag}_gbs"] = nbytes / med / 1e9
-		c5[f"decode_{tag}_frac_of_hbm"] = nbytes / med / 1e9 / PEAK_HBM_GBS
+		c5[f"decode_{tag}_cache_gbs"] = nbytes / med / 1e9            # whole cache / time: counts the V rows skipped
+		c5[f"decode_{tag}_hbm_gbs"] = DECODE_TRAFFIC_BYTES / med / 1e9  # bytes actually fetched (rocprofv3) / time
+		c5[f"decode_{tag}_frac_of_hbm"] = DECODE_TRAFFIC_BYTES / med / 1e9 / PEAK_HBM_GBS
 	out["config5_long_context"] = c5
 	return out
 
@@ -314,7 +318,7 @@ def single(dev, X, recipes, name, iters):
 		tp = X.Tensor.from_numpy(dev, np.ones(H, np.float32), X.F32)
 		od = X.Tensor(dev, (S5, H * HD), X.INT8)
 		k = recipes.attn_decode_kernel(dev, H, HD, CAP, False)
-		fn, work, unit = (lambda: k.launch(qd, cache, lens, sk, sv, tp, od, None, W)), S5 * CAP * 2 * H * HD / 1e9, "GB/s"
+		fn, work, unit = (lambda: k.launch(qd, cache, lens, sk, sv, tp, od, None, W)), S5 * CAP * 2 * H * HD / 1e9, "GB/s of cache (rows with zero probability are not fetched)"
 	elif name == "rms_norm_config4":
 		rows = 32768
 		xb = X.Tensor.from_numpy(dev, (rng.standard_normal((rows, D), dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16), X.BF16)
