@@ -1,0 +1,164 @@
+"""GPU parity at the full BASELINE sizes.
+
+The CPU oracle cannot redo these workloads whole in test time, so each check uses a property that does
+not depend on the size: a GEMM output row depends only on its own token row and the weights, an attention
+head only on its own columns, a decoded (sequence, head) only on its own cache slice.  The kernels run at
+full size (persistent grid, every tile / query block / workgroup exercised); a sample of rows / heads /
+sequences is then recomputed by the oracle and compared to the strict builds bit for bit.
+"""
+import math
+
+import numpy as np
+import pytest
+
+import x17ai_amd as X
+from x17ai_amd import recipes
+from oracle import strict as S
+from tests.gpu_common import i8_codes, rng_for
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+	d = X.Device(0)
+	yield d
+	d.synchronize()
+
+
+def _up(dev, arr, dtype):
+	return X.Tensor.from_numpy(dev, arr, dtype)
+
+
+def _sample_rows(rng, m, count):
+	# first and last rows, the rows around every 256-row tile edge of the first tiles, and random ones
+	fixed = [0, 1, 255, 256, 257, m - 257, m - 256, m - 1]
+	return np.unique(np.concatenate((np.array(fixed), rng.integers(0, m, count - len(fixed)))))
+
+
+def test_config2_ffn_pair_sampled_rows(dev):
+	"""BASELINE config 2: tokens 8192, d_model 2048, d_ff 8192 -- ffn_f (GeGLU -> FixedI8) and the int8
+	ffn_y (gated residual -> e4m3), strict builds, 96 sampled token rows of each against the oracle."""
+	m, d, f = 8192, 2048, 8192
+	rng = rng_for("full-config2")
+	x, w1, w2 = i8_codes(rng, (m, d)), i8_codes(rng, (2 * f, d)), i8_codes(rng, (2 * d, f))
+	k1 = recipes.ffn_f_kernel(dev, d, 2 * f, True, X.INT8)
+	k2 = recipes.ffn_y_kernel(dev, d, f, True, X.INT8, X.INT8)
+	xt = _up(dev, x, X.INT8)
+	ft = X.Tensor(dev, (m, f), X.INT8)
+	yt = X.Tensor(dev, (m, d), X.E4M3)
+	k1.launch(xt, _up(dev, w1, X.INT8), ft)
+	k2.launch(ft, _up(dev, w2, X.INT8), yt, xt)
+	got_f, got_y = ft.download(), yt.download()
+	rows = _sample_rows(rng, m, 96)
+	want_f = S.epilogue_geglu(S.gemm_i32(x[rows], w1), 1.0 / math.sqrt(d) / 64.0, 8.0, S.STORE_I8)
+	assert np.array_equal(got_f[rows], want_f)
+	inp_y = math.sqrt(recipes.GELU_VAR_FIX_2 / f) / 64.0
+	want_y = S.epilogue_residual(S.gemm_i32(got_f[rows], w2), x[rows], inp_y, 1.0, S.STORE_E4M3)
+	assert np.array_equal(got_y[rows], want_y)
+	# every tile wrote something plausible: no output row is left at the allocator's fill
+	assert np.count_nonzero(np.abs(got_f.astype(np.int32)).sum(axis=1) == 0) == 0
+
+
+def test_config2_checksum_of_checksums(dev):
+	"""Column sums of an int8 GEMM are linear in the token rows: sum_m C[m, n] = (sum_m A[m, :]) . B[n, :].
+	With +-1/0 operands sparse enough that no accumulator leaves the FixedI8 range, a scale-1 epilogue
+	returns the accumulators themselves, and the whole 8192 x 16384 output is checked through one vector."""
+	m, k, n = 8192, 2048, 16384
+	rng = rng_for("full-checksum")
+	a = (rng.integers(-1, 2, (m, k)) * (rng.random((m, k)) < 0.02)).astype(np.int8)
+	b = (rng.integers(-1, 2, (n, k)) * (rng.random((n, k)) < 0.3)).astype(np.int8)
+	cfg = X.GemmConfig(X.GemmInputConfig(X.INT8, k, None, False), X.GemmInputConfig(X.INT8, k, n, True), X.INT8)
+	kern = X.GemmKernel(dev, f"acc_probe-k{k}-n{n}", cfg, X.ScaleConfig(1.0, 1.0))
+	c = X.Tensor(dev, (m, n), X.INT8)
+	kern.launch(_up(dev, a, X.INT8), _up(dev, b, X.INT8), c)
+	got = c.download().astype(np.int64)
+	assert np.abs(got).max() < 127                      # nothing saturated, so got IS the accumulator
+	col = a.astype(np.int64).sum(axis=0)
+	assert np.array_equal(got.sum(axis=0), b.astype(np.int64) @ col)
+	row = b.astype(np.int64).sum(axis=0)
+	assert np.array_equal(got.sum(axis=1), a.astype(np.int64) @ row)
+
+
+def _attn_inputs(rng, rows, h, hd):
+	q = i8_codes(rng, (rows, h * hd))
+	k = rng.standard_normal((rows, h, hd), dtype=np.float32)
+	k /= np.sqrt((k * k).mean(-1, keepdims=True))
+	v = rng.standard_normal((rows, h, hd), dtype=np.float32) * 1.3
+	kv = S.f32_to_fixedi8((np.concatenate((k, v), axis=2).reshape(rows, 2 * h * hd) * 8).astype(np.float32))
+	sk = rng.standard_normal((h, hd))
+	sk /= np.sqrt((sk * sk).mean(-1, keepdims=True))
+	return q, kv, S.f32_to_fixedi8((sk * 8).astype(np.float32)), i8_codes(rng, (h, hd), 1.3), (0.5 + rng.random(h)).astype(np.float32)
+
+
+def _head_columns(arr, heads, width):
+	return np.ascontiguousarray(np.concatenate([arr[:, h * width:(h + 1) * width] for h in heads], axis=1))
+
+
+def test_config4_attention_sampled_heads(dev):
+	"""BASELINE config 4 attention: 4 sequences x 8192 tokens, 16 heads x 128, window 512.  Heads are
+	independent, so three heads of two of the sequences are recomputed by the oracle (all 8192 queries)."""
+	t, b, h, hd, w = 8192, 4, 16, 128, 512
+	rng = rng_for("full-config4-attn")
+	q, kv, sk, sv, temp = _attn_inputs(rng, t * b, h, hd)
+	kern = recipes.attn_kernel(dev, h, hd, True)
+	out = X.Tensor(dev, q.shape, X.INT8)
+	l = X.Tensor(dev, (h, t * b), X.F32)
+	kern.launch(_up(dev, q, X.INT8), _up(dev, kv, X.INT8), _up(dev, sk, X.INT8), _up(dev, sv, X.INT8),
+	            _up(dev, temp, X.F32), out, l, w, b)
+	got, got_l = out.download(), l.download()
+	heads = [0, 7, 15]
+	for seq in (0, 3):
+		rows = slice(seq * t, (seq + 1) * t)
+		want, want_l = S.attn_fwd_i8(_head_columns(q[rows], heads, hd), _head_columns(kv[rows], heads, 2 * hd),
+		                             sk[heads], sv[heads], temp[heads], len(heads), hd, w)
+		assert np.array_equal(_head_columns(got[rows], heads, hd), want)
+		assert np.array_equal(got_l[heads][:, rows].view(np.uint32), want_l.view(np.uint32))
+
+
+def test_config5_prefill_sampled_heads(dev):
+	"""BASELINE config 5 prefill: one sequence of 65536 tokens, 32 heads x 128, window 4096; two heads
+	recomputed by the oracle.  Also the speed build against the strict one over the whole output."""
+	t, h, hd, w = 65536, 32, 128, 4096
+	rng = rng_for("full-config5-attn")
+	q, kv, sk, sv, temp = _attn_inputs(rng, t, h, hd)
+	qt, kvt = _up(dev, q, X.INT8), _up(dev, kv, X.INT8)
+	skt, svt, tt = _up(dev, sk, X.INT8), _up(dev, sv, X.INT8), _up(dev, temp, X.F32)
+	out = X.Tensor(dev, q.shape, X.INT8)
+	l = X.Tensor(dev, (h, t), X.F32)
+	recipes.attn_kernel(dev, h, hd, True).launch(qt, kvt, skt, svt, tt, out, l, w, 1)
+	got, got_l = out.download(), l.download()
+	heads = [3, 31]
+	want, want_l = S.attn_fwd_i8(_head_columns(q, heads, hd), _head_columns(kv, heads, 2 * hd),
+	                             sk[heads], sv[heads], temp[heads], len(heads), hd, w)
+	assert np.array_equal(_head_columns(got, heads, hd), want)
+	assert np.array_equal(got_l[heads].view(np.uint32), want_l.view(np.uint32))
+	out_fast = X.Tensor(dev, q.shape, X.INT8)
+	recipes.attn_kernel(dev, h, hd, False).launch(qt, kvt, skt, svt, tt, out_fast, None, w, 1)
+	d = np.abs(out_fast.download().astype(np.int32) - got.astype(np.int32))
+	assert d.max() <= 1 and np.mean(d > 0) < 0.02, (d.max(), np.mean(d > 0))
+
+
+def test_config5_decode_sampled_sequences(dev):
+	"""BASELINE config 5 decode: 64 sequences against 4096 cached positions, 32 heads x 128.  Ragged
+	lengths (0, 1, 15, 16, 17, ..., 4096); four heads of every sequence recomputed by the oracle."""
+	s, cap, h, hd, w = 64, 4096, 32, 128, 4096
+	rng = rng_for("full-config5-decode")
+	q, _, sk, sv, temp = _attn_inputs(rng, s, h, hd)
+	cache = np.empty((s, cap, 2 * h * hd), np.int8)
+	for i in range(s):
+		cache[i] = i8_codes(rng, (cap, 2 * h * hd))
+	lens = rng.integers(1, cap + 1, s).astype(np.uint32)
+	lens[:8] = [0, 1, 15, 16, 17, 4095, 4096, 2048]
+	kern = recipes.attn_decode_kernel(dev, h, hd, cap, True)
+	out = X.Tensor(dev, (s, h * hd), X.INT8)
+	l = X.Tensor(dev, (s, h), X.F32)
+	kern.launch(_up(dev, q, X.INT8), _up(dev, cache, X.INT8), _up(dev, lens.view(np.float32), X.F32),
+	            _up(dev, sk, X.INT8), _up(dev, sv, X.INT8), _up(dev, temp, X.F32), out, l, w)
+	got, got_l = out.download(), l.download()
+	heads = [0, 5, 17, 31]
+	sub_cache = np.ascontiguousarray(np.concatenate([cache[:, :, hh * 2 * hd:(hh + 1) * 2 * hd] for hh in heads], axis=2))
+	want, want_l = S.attn_decode_i8(_head_columns(q, heads, hd), sub_cache, lens, sk[heads], sv[heads], temp[heads],
+	                                len(heads), hd, w)
+	assert np.array_equal(_head_columns(got, heads, hd), want)
+	assert np.array_equal(got_l[:, heads].view(np.uint32), np.asarray(want_l).reshape(s, len(heads)).view(np.uint32))

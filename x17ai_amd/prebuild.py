@@ -64,6 +64,9 @@ def _specs():
 	add(("ffn_y", 2048, 8192, False, E4M3, INT8))
 	add(("attn", 8, 64, False))
 	add(("copy_probe",))
+	# ---- tests/test_gpu_fullsize.py (the strict ffn pair, attention and decode kernels are listed above)
+	add(("attn", 16, 128, True))
+	add(("acc_probe_full",))
 	return s
 
 
@@ -96,6 +99,10 @@ def _build_one(spec) -> str:
 		cfg = GemmConfig(GemmInputConfig(INT8, k, None, False), GemmInputConfig(INT8, k, n, True), INT8)
 		GemmKernel(None, f"acc_probe-k{k}-n{n}", cfg, ScaleConfig(1.0, 1.0))
 		return GemmKernel(None, f"acc_probe2-k{k}-n{n}", cfg, ScaleConfig(1.0 / (k * 127.0), 1.0)).name
+	if kind == "acc_probe_full":
+		k, n = 2048, 16384
+		cfg = GemmConfig(GemmInputConfig(INT8, k, None, False), GemmInputConfig(INT8, k, n, True), INT8)
+		return GemmKernel(None, f"acc_probe-k{k}-n{n}", cfg, ScaleConfig(1.0, 1.0)).name
 	raise ValueError(spec)
 
 
