@@ -392,7 +392,11 @@ void kernel(
 	u32 const n_groups = gridDim.x * gridDim.y * gridDim.z;
 	u32 const group = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
 	auto tile_coords = [&](u32 lin, u32 &tile_m, u32 &tile_n) {
+#ifdef X17_GEMM_BAND
+		constexpr u32 BAND = X17_GEMM_BAND;
+#else
 		constexpr u32 BAND = 2048 / gt::M_PER_BLOCK;
+#endif
 		if (total % 8 == 0) {
 			lin = (lin % 8) * (total / 8) + lin / 8;
 		}
@@ -427,42 +431,55 @@ void kernel(
 		lo.swz = ((lane % 32) >> SWZ_SHIFT) & (CHUNKS - 1);
 	}
 
-	// ---- main loop.  A ring of STAGES LDS buffers; step ks consumes buffer ks % STAGES while the
-	// loads of steps ks+1 .. ks+STAGES-1 are in flight.  The one barrier per step sits before the last
-	// slice's MFMAs: behind it the first fragments of the next step are fetched, so LDS latency is
-	// covered by matrix-core time across the step boundary too.  The load stream runs across tile
-	// boundaries: the last steps of a tile already fetch the first stages of the workgroup's next
-	// tile, which then land while the epilogue runs.
-	static_assert(K_STEPS + 1 >= gt::STAGES, "K too short for the LDS ring");
+	// ---- main loop.  A ring of STAGES LDS buffers; step ks consumes buffer ks % STAGES while the loads of
+	// steps ks+1 .. ks+STAGES-1 are in flight.  The one barrier per step sits before the last slice's
+	// MFMAs, when every wave holds the last fragments of the step in registers: behind it the buffer is
+	// free, so the loads of step ks+STAGES are issued there -- a full step before they are waited for --
+	// and the first fragments of step ks+1 are fetched, so LDS latency is covered by matrix-core time across
+	// the step boundary too.  The load stream runs across tile boundaries: the last steps of a tile
+	// already fetch the first stages of the workgroup's next tile, which land while the epilogue runs.
+	// (a K shorter than the ring cannot prefetch across tiles: each tile then starts with its own prologue)
+	constexpr bool CROSS_TILE = K_STEPS >= gt::STAGES;
+	constexpr u32 PROLOGUE_STAGES = CROSS_TILE ? gt::STAGES : K_STEPS;
 	u32 const x_off = wm * gt::WAVE_M * ROW_BYTES + lo.frag_row;
 	u32 const w_off = X_TILE_BYTES + wn * 128 * ROW_BYTES + lo.frag_row;
-
-	// this wave's loads of one stage are dealt out over the first LOAD_SLICES slices of a step
-#ifndef X17_GEMM_LOAD_SLICES
-#define X17_GEMM_LOAD_SLICES (SLICES >= 4 ? 2 : 1)
-#endif
-	constexpr u32 LOAD_SLICES = X17_GEMM_LOAD_SLICES;
-	static_assert(LOAD_SLICES >= 1 && LOAD_SLICES < SLICES && LOAD_SLICES <= 3);
-	constexpr u32 LOADS_PER_SLICE = (LOADS_PER_STAGE + LOAD_SLICES - 1) / LOAD_SLICES;
-	constexpr u32 LOADS_END_1 = 2 * LOADS_PER_SLICE < LOADS_PER_STAGE ? 2 * LOADS_PER_SLICE : LOADS_PER_STAGE;
 
 	u32 tile_m, tile_n;
 	tile_coords(group, tile_m, tile_n);
 	u8 const *a_tile = a + (size_t)(tile_m * gt::M_PER_BLOCK) * K_TOTAL;
 	u8 const *b_tile = b + (size_t)(tile_n * gt::N_PER_BLOCK) * K_TOTAL;
-	X17_UNROLL for (u32 s = 0; s + 1 < gt::STAGES; ++s) {
-		issue_stage_loads<0, LOADS_PER_STAGE>(a_tile, b_tile, smem + s * STAGE_BYTES, s * gt::K_STEP, wave, lo);
-	}
+	auto prologue = [&]() {
+		X17_UNROLL for (u32 s = 0; s < PROLOGUE_STAGES; ++s) {
+			issue_stage_loads<0, LOADS_PER_STAGE>(a_tile, b_tile, smem + s * STAGE_BYTES, s * gt::K_STEP, wave, lo);
+		}
+		if constexpr (CROSS_TILE) {
+			wait_stage(gt::STAGES - 1);                // stage 0 has landed ...
+		} else {
+			wait_vmcnt<0>();
+		}
+		__builtin_amdgcn_s_barrier();                  // ... for every wave
+	};
+	prologue();
 
 	u32 buf = 0;                                   // ring position of the step being consumed
 	for (u32 lin = group; lin < total; lin += n_groups) {
-		bool const has_next = lin + n_groups < total;
+		bool const first_tile = lin == group;
+		bool const more_tiles = lin + n_groups < total;
+		bool const has_next = CROSS_TILE && more_tiles;      // prefetch the next tile's first stages
 		u32 next_m = 0, next_n = 0;
-		if (has_next) {
+		if (more_tiles) {
 			tile_coords(lin + n_groups, next_m, next_n);
 		}
 		u8 const *a_next = a + (size_t)(next_m * gt::M_PER_BLOCK) * K_TOTAL;
 		u8 const *b_next = b + (size_t)(next_n * gt::N_PER_BLOCK) * K_TOTAL;
+		if constexpr (!CROSS_TILE) {
+			if (!first_tile) {
+				__builtin_amdgcn_s_waitcnt(0xC07F);        // lgkmcnt(0)
+				__builtin_amdgcn_s_barrier();              // nobody still reads the previous tile's buffers
+				buf = 0;
+				prologue();
+			}
+		}
 
 		Acc acc[4][BM];   // [bn][bm]
 		X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
@@ -471,53 +488,48 @@ void kernel(
 			}
 		}
 
-		// stage 0 of this tile has landed, for every wave, and nobody still reads the previous tile's buffers
-		// (vmcnt(0) rather than a stage count: the previous tile's output stores are in the same counter)
-		__builtin_amdgcn_s_waitcnt(0x0070);        // vmcnt(0) lgkmcnt(0)
-		__builtin_amdgcn_s_barrier();
-
+		// (stage 0 of this tile is visible: the wait and the barrier were the previous tile's last ones)
 		Frags frags[2];
 		load_frags(frags[0], smem + buf * STAGE_BYTES + w_off, smem + buf * STAGE_BYTES + x_off, 0, lo);
 
 		for (u32 ks = 0; ks < K_STEPS; ++ks) {
-			u32 const load_buf = buf == 0 ? gt::STAGES - 1 : buf - 1;    // consumed by the previous step
 			u32 const next_buf = buf + 1 == gt::STAGES ? 0 : buf + 1;
-			u32 const load_step = ks + gt::STAGES - 1;
+			u32 const load_step = ks + gt::STAGES;                       // the step whose loads go out behind this barrier
 			bool const this_tile = load_step < K_STEPS;
 			bool const more_loads = this_tile || has_next;
 			u8 const *la = this_tile ? a_tile : a_next;
 			u8 const *lb = this_tile ? b_tile : b_next;
 			u32 const load_k0 = (this_tile ? load_step : load_step - K_STEPS) * gt::K_STEP;
-			u8 *load_stage = smem + load_buf * STAGE_BYTES;
-			u8 const *stage = smem + buf * STAGE_BYTES;
+			u8 *stage = smem + buf * STAGE_BYTES;
 			X17_UNROLL for (u32 s = 0; s < SLICES; ++s) {
 				bool reads = true;
 				if (s + 1 < SLICES) {
 					load_frags(frags[(s + 1) & 1], stage + w_off, stage + x_off, s + 1, lo);
-				} else if (ks + 1 < K_STEPS) {
-					u32 remaining = has_next ? gt::STAGES : K_STEPS - 2 - ks;      // stages issued after ks+1
-					wait_stage(remaining < gt::STAGES - 2 ? remaining : gt::STAGES - 2);
+				} else if (ks + 1 < K_STEPS || has_next) {
+					// step ks+1 (or the next tile's step 0) must have landed; younger stages may stay in flight.
+					// After an epilogue its stores share the counter with the loads: wait for everything then.
+					u32 in_flight = has_next ? gt::STAGES : K_STEPS - 2 - ks;     // stages issued after the awaited one
+					bool const stores_pending = !first_tile && ks + 1 < gt::STAGES;
+					wait_stage(stores_pending ? 0 : (in_flight < gt::STAGES - 2 ? in_flight : gt::STAGES - 2));
 					__builtin_amdgcn_s_waitcnt(0xC07F);    // lgkmcnt(0): this wave is done reading buffer `buf`
 					__builtin_amdgcn_s_barrier();
-					u8 const *next = smem + next_buf * STAGE_BYTES;
-					load_frags(frags[(s + 1) & 1], next + w_off, next + x_off, 0, lo);
+					if (more_loads) {
+						issue_stage_loads<0, LOADS_PER_STAGE>(la, lb, stage, load_k0, wave, lo);
+					}
+					if (ks + 1 < K_STEPS) {
+						u8 const *next = smem + next_buf * STAGE_BYTES;
+						load_frags(frags[(s + 1) & 1], next + w_off, next + x_off, 0, lo);
+					} else {
+						reads = false;
+					}
 				} else {
 					reads = false;
 				}
-				if (more_loads) {
-					if (s == 0) issue_stage_loads<0, LOADS_PER_SLICE>(la, lb, load_stage, load_k0, wave, lo);
-					if constexpr (LOAD_SLICES >= 2) {
-						if (s == 1) issue_stage_loads<LOADS_PER_SLICE, LOADS_END_1>(la, lb, load_stage, load_k0, wave, lo);
-					}
-					if constexpr (LOAD_SLICES >= 3) {
-						if (s == 2) issue_stage_loads<LOADS_END_1, LOADS_PER_STAGE>(la, lb, load_stage, load_k0, wave, lo);
-					}
-				}
 				mma_slice(frags[s & 1], acc);
-				if (s < LOAD_SLICES) {
-					interleave_slice<(LOAD_SLICES == 1 ? 0 : LOADS_PER_SLICE)>(reads);
-				} else {
+				if (s + 1 < SLICES) {
 					interleave_slice<0>(reads);
+				} else {
+					interleave_slice<LOADS_PER_STAGE>(reads);
 				}
 			}
 			buf = next_buf;
