@@ -394,10 +394,8 @@ void kernel(
 			// word g of this lane = dims 32*db + 8*g + 4*half .. +3
 			u32 word[4];
 			X17_UNROLL for (int g = 0; g < 4; ++g) {
-				word[g] = 0;
-				X17_UNROLL for (int b = 0; b < 4; ++b) {
-					word[g] |= ((u32)f32_to_fixedi8(o_acc[db][4 * g + b] * inv) & 0xFFu) << (8 * b);
-				}
+				word[g] = pack4_fixedi8(o_acc[db][4 * g] * inv, o_acc[db][4 * g + 1] * inv,
+				                        o_acc[db][4 * g + 2] * inv, o_acc[db][4 * g + 3] * inv);
 			}
 			// The lane pair (lane, lane + 32) holds the 32 bytes of this block interleaved word by word; two
 			// cross-half swaps give the lower lane bytes 0..15 and the upper lane bytes 16..31, so that each

@@ -79,11 +79,9 @@ struct ScaleEpilogue {
 		X17_UNROLL for (int v = 0; v < 4; ++v) {
 			v4u pack;
 			X17_UNROLL for (int w = 0; w < 4; ++w) {
-				u32 word = 0;
-				X17_UNROLL for (int b = 0; b < 4; ++b) {
-					word |= store_convert<STORE>(x[16 * v + 4 * w + b] * f32(SCALE)) << (8 * b);
-				}
-				pack[w] = word;
+				f32 y[4];
+				X17_UNROLL for (int b = 0; b < 4; ++b) y[b] = x[16 * v + 4 * w + b] * f32(SCALE);
+				pack[w] = pack4_store<STORE>(y[0], y[1], y[2], y[3]);
 			}
 			*reinterpret_cast<v4u *>(dst + 16 * v) = pack;
 		}
@@ -108,17 +106,32 @@ struct GeGluEpilogue {
 		f32 t = sfu::tanh(s);
 		return fmaf32(f32(Y) * x, t, f32(Y) * x);
 	}
+	// gate(g) * v.  The speed build uses 1 + tanh(s) = 2 / (1 + 2^(-2 s lg e)) and folds the constants:
+	// g * v / (c + c * 2^(g * (A1 + A3 g^2))), c = 1 / (2 Y) -- two transcendentals and seven plain
+	// operations; an overflowing exponential gives +inf and a quotient of zero, the right limit.
+	static constexpr f64 LOG2E = 1.4426950408889634;
+	X17_DEV static f32 gated(f32 g, f32 v) {
+		if constexpr (X17_STRICT_MATH != 0) {
+			return gate(g) * v;
+		} else {
+			f32 g2 = g * g;
+			f32 t = fmaf32(g2, f32(-2.0 * LOG2E * CK3), f32(-2.0 * LOG2E * CK));
+			f32 e = hw::ex2(t * g);
+			f32 d = fmaf32(e, f32(0.5 / Y), f32(0.5 / Y));
+			return (g * v) * hw::rcp(d);
+		}
+	}
 	X17_DEV static void run(f32 const (&x)[64], u8 *c, u32 row, u32 n, void const *) {
 		u8 *dst = c + (size_t)row * OUT_COLS + n / 2;
 		X17_UNROLL for (int v = 0; v < 2; ++v) {
 			v4u pack;
 			X17_UNROLL for (int w = 0; w < 4; ++w) {
-				u32 word = 0;
+				f32 y[4];
 				X17_UNROLL for (int b = 0; b < 4; ++b) {
 					int j = 16 * v + 4 * w + b;
-					word |= store_convert<STORE>(gate(x[2 * j]) * x[2 * j + 1]) << (8 * b);
+					y[b] = gated(x[2 * j], x[2 * j + 1]);
 				}
-				pack[w] = word;
+				pack[w] = pack4_store<STORE>(y[0], y[1], y[2], y[3]);
 			}
 			*reinterpret_cast<v4u *>(dst + 16 * v) = pack;
 		}
@@ -156,13 +169,13 @@ struct ResidualEpilogue {
 			v4u rv = *reinterpret_cast<v4u const *>(res + 16 * v);
 			v4u pack;
 			X17_UNROLL for (int w = 0; w < 4; ++w) {
-				u32 word = 0;
+				f32 y[4];
 				X17_UNROLL for (int b = 0; b < 4; ++b) {
 					int j = 16 * v + 4 * w + b;
 					f32 r = f32((i32)(i8)((rv[w] >> (8 * b)) & 0xFFu));
-					word |= store_convert<STORE>(mix(x[2 * j], x[2 * j + 1], r)) << (8 * b);
+					y[b] = mix(x[2 * j], x[2 * j + 1], r);
 				}
-				pack[w] = word;
+				pack[w] = pack4_store<STORE>(y[0], y[1], y[2], y[3]);
 			}
 			*reinterpret_cast<v4u *>(dst + 16 * v) = pack;
 		}
@@ -582,12 +595,8 @@ void kernel(
 			X17_UNROLL for (int v = 0; v < count / 16; ++v) {
 				v4u pack;
 				X17_UNROLL for (int w = 0; w < 4; ++w) {
-					u32 word = 0;
-					X17_UNROLL for (int bb = 0; bb < 4; ++bb) {
-						int d = first + 16 * v + 4 * w + bb;
-						word |= ((u32)f32_to_fixedi8(x[d] * scale) & 0xFFu) << (8 * bb);
-					}
-					pack[w] = word;
+					int d = first + 16 * v + 4 * w;
+					pack[w] = pack4_fixedi8(x[d] * scale, x[d + 1] * scale, x[d + 2] * scale, x[d + 3] * scale);
 				}
 				*reinterpret_cast<v4u *>(dst + first + 16 * v) = pack;
 			}

@@ -89,6 +89,28 @@ X17_DEV u32 e4m3_to_bf16_bits(u32 c) {
 	return rest == 0 ? 0u : ((sign | rest) + (120u << 7));
 }
 
+// Four FixedI8 codes packed into one word (a in the low byte).  Same values as f32_to_fixedi8:
+// clamp, then add 1.5 * 2^23 -- the add rounds to an integer, ties to even, exactly like rint, and
+// leaves the two's-complement code in the low byte of the float -- then gather the four low bytes.
+X17_DEV u32 pack4_fixedi8(f32 a, f32 b, f32 c, f32 d) {
+	constexpr f32 MAGIC = 12582912.0f;
+	u32 ua = f2u(__builtin_amdgcn_fmed3f(a, -127.0f, 127.0f) + MAGIC);
+	u32 ub = f2u(__builtin_amdgcn_fmed3f(b, -127.0f, 127.0f) + MAGIC);
+	u32 uc = f2u(__builtin_amdgcn_fmed3f(c, -127.0f, 127.0f) + MAGIC);
+	u32 ud = f2u(__builtin_amdgcn_fmed3f(d, -127.0f, 127.0f) + MAGIC);
+	u32 lo = __builtin_amdgcn_perm(ub, ua, 0x0c0c0400u);     // bytes: a0, b0, 0, 0
+	u32 hi = __builtin_amdgcn_perm(ud, uc, 0x04000c0cu);     // bytes: 0, 0, c0, d0
+	return lo | hi;
+}
+
+template<int STORE> X17_DEV u32 pack4_store(f32 a, f32 b, f32 c, f32 d) {
+	if constexpr (STORE == 1) {
+		return f32_to_e4m3(a) | (f32_to_e4m3(b) << 8) | (f32_to_e4m3(c) << 16) | (f32_to_e4m3(d) << 24);
+	} else {
+		return pack4_fixedi8(a, b, c, d);
+	}
+}
+
 template<int STORE> X17_DEV u32 store_convert(f32 v) {
 	if constexpr (STORE == 1) {
 		return f32_to_e4m3(v);
