@@ -37,6 +37,11 @@ enum { X17H_EPI_SCALE = 0, X17H_EPI_GEGLU = 1, X17H_EPI_RESIDUAL = 2, X17H_EPI_R
 char const *x17h_last_error(void);
 /* text of the warnings/errors collected by the last *_new call (kernel generation diagnostics) */
 char const *x17h_last_diagnostics(void);
+/* For callers of the raw shim that cannot implement the FfiBuffer callbacks themselves: hands `diag`
+ * (a non-NULL X17DiagnosticBuffer* returned by an x17ai_hip_* function) to x17ai_move_diagnostic
+ * through the operator layer's own growable buffer (the twin of src/util/ffi_buffer.rs:13-103) and
+ * APPENDS the text to the NUL-terminated string in out[capacity].  Returns the new string length. */
+size_t x17h_move_diagnostic_text(void *diag, char *out, size_t capacity);
 
 /* CudaDevice::new, src/device/cuda.rs:31-38 */
 int x17h_device_new(size_t device_id, X17hDevice **out);

@@ -39,7 +39,7 @@ def test_host_library_exports_every_declared_entry_point():
 	assert declared and not [s for s in declared if s not in exported]
 
 
-def test_struct_layouts_match_the_reference_ffi():
+def test_struct_layouts_match_the_reference_ffi(tmp_path):
 	# CudaKernelAttrs: nine int32 (cuda_shim.rs:51-63); PtrResult: two pointers (cuda_shim.rs:70-74)
 	src = open(os.path.join(ROOT, "include", "x17ai_hip_shim.h")).read()
 	body = src[src.index("typedef struct X17HipKernelAttrs {"):src.index("} X17HipKernelAttrs;")]
@@ -49,8 +49,7 @@ def test_struct_layouts_match_the_reference_ffi():
 	#include <stdio.h>
 	int main(void) { printf("%zu %zu %zu %zu\n", sizeof(X17HipKernelAttrs), sizeof(X17StreamResult), sizeof(X17FfiBuffer), sizeof(X17FfiSpan)); return 0; }
 	'''
-	exe = os.path.join(ROOT, "_work", "layout_probe")
-	os.makedirs(os.path.dirname(exe), exist_ok=True)
+	exe = str(tmp_path / "layout_probe")
 	subprocess.run(["gcc", "-x", "c", "-", "-I", os.path.join(ROOT, "include"), "-o", exe], input=prog, text=True, check=True)
 	assert subprocess.run([exe], capture_output=True, text=True, check=True).stdout.split() == ["36", "16", "16", "16"]
 

@@ -19,6 +19,11 @@ def lib_paths() -> dict:
 	}
 
 
+def kernel_cache_dir() -> str:
+	"""Where the operator layer keeps one directory per built kernel (common.h, kernel.hsaco, meta.json)."""
+	return os.environ.get("X17AI_KERNEL_CACHE") or os.path.join(_HERE, "cache", "kernels")
+
+
 class GemmConfigC(ctypes.Structure):
 	_fields_ = [
 		("a_dtype", ctypes.c_int), ("a_cols", ctypes.c_size_t), ("a_rows", ctypes.c_size_t), ("a_trans", ctypes.c_int),

@@ -1013,6 +1013,20 @@ extern "C" {
 char const *x17h_last_error(void) { return g_last_error.c_str(); }
 char const *x17h_last_diagnostics(void) { return g_last_diag.c_str(); }
 
+size_t x17h_move_diagnostic_text(void *diag, char *out, size_t capacity) {
+	if (out == nullptr || capacity == 0) return 0;
+	size_t have = strnlen(out, capacity - 1);
+	FfiBufferImpl buf;
+	buf.data.assign(out, have);
+	if (diag != nullptr) {
+		x17ai_move_diagnostic(reinterpret_cast<X17DiagnosticBuffer *>(diag), buf.as_ffi());
+	}
+	size_t n = buf.data.size() < capacity - 1 ? buf.data.size() : capacity - 1;
+	std::memcpy(out, buf.data.data(), n);
+	out[n] = 0;
+	return n;
+}
+
 int x17h_device_new(size_t device_id, X17hDevice **out) {
 	try {
 		auto r = HipDevice::create(device_id);

@@ -37,6 +37,14 @@
 using namespace x17;
 namespace gt = x17::gemm_tile;
 
+// The compiler fully unrolls a K loop of up to 8 steps and then runs out of registers; longer loops it
+// unrolls by a small factor on its own, which measures 5 % faster than a rolled loop.
+#if (X17_A_COLS / X17_GEMM_K_STEP) <= 8
+#define X17_K_LOOP_PRAGMA _Pragma("clang loop unroll(disable)")
+#else
+#define X17_K_LOOP_PRAGMA
+#endif
+
 namespace {
 
 constexpr u32 K_TOTAL = X17_A_COLS;
@@ -505,6 +513,7 @@ void kernel(
 		Frags frags[2];
 		load_frags(frags[0], smem + buf * STAGE_BYTES + w_off, smem + buf * STAGE_BYTES + x_off, 0, lo);
 
+		X17_K_LOOP_PRAGMA
 		for (u32 ks = 0; ks < K_STEPS; ++ks) {
 			u32 const next_buf = buf + 1 == gt::STAGES ? 0 : buf + 1;
 			u32 const load_step = ks + gt::STAGES;                       // the step whose loads go out behind this barrier
