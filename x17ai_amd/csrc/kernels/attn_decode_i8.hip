@@ -51,15 +51,16 @@ void kernel(
 	i8 *out, f32 *l_out, u32 window_size
 ) {
 	extern __shared__ __attribute__((aligned(16))) u8 smem[];
+	// the scores are dead once the probabilities exist, so the P.V partials of phase 4 reuse their space
 	f32 *s_score = reinterpret_cast<f32 *>(smem);                               // [CAP]
-	u8 *s_prob = smem + CAP * 4;                                                 // [CAP]
-	f32 *s_quad = reinterpret_cast<f32 *>(smem + CAP * 5);                       // [CAP / 4]
-	f32 *s_tmax = reinterpret_cast<f32 *>(smem + CAP * 6);                       // [MAX_TILES]
+	i32 *s_pv = reinterpret_cast<i32 *>(smem);                                   // [CHUNK_TILES][HD]
+	u8 *s_prob = smem + dt::SCORE_PV_BYTES;                                      // [CAP]
+	f32 *s_quad = reinterpret_cast<f32 *>(s_prob + CAP);                         // [CAP / 4]
+	f32 *s_tmax = s_quad + CAP / 4;                                              // [MAX_TILES]
 	f32 *s_resc = s_tmax + dt::MAX_TILES;                                        // [MAX_TILES]
 	f32 *s_mrun = s_resc + dt::MAX_TILES;                                        // [MAX_TILES]
 	f32 *s_bmax = s_mrun + dt::MAX_TILES;                                        // [256]
-	i32 *s_pv = reinterpret_cast<i32 *>(s_bmax + 256);                           // [CHUNK_TILES][HD]
-	f32 *s_sum = reinterpret_cast<f32 *>(s_pv + dt::CHUNK_TILES * HD);           // [4]
+	f32 *s_sum = s_bmax + 256;                                                   // [4]
 
 	u32 const tid = threadIdx.x;
 	u32 const head = blockIdx.x;

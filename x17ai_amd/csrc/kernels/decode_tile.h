@@ -11,10 +11,11 @@ constexpr unsigned HEADS_PER_BLOCK = 1;
 constexpr unsigned MAX_TILES = CAPACITY / 16;           // 16-key tiles
 constexpr unsigned CHUNK_TILES = 32;                    // tiles whose P.V partials are staged at once
 
-// LDS: scores f32[CAPACITY] | probabilities u8[CAPACITY] | quad sums f32[CAPACITY/4]
-//      | per tile: max, running max, rescale f32[3 * MAX_TILES] | block maxima f32[256]
-//      | P.V partials i32[CHUNK_TILES * HEAD_DIM] | final partial sums f32[4]
-constexpr unsigned SMEM_BYTES =
-	CAPACITY * 4 + CAPACITY + CAPACITY + 3 * MAX_TILES * 4 + 256 * 4 + CHUNK_TILES * HEAD_DIM * 4 + 16;
+// LDS: scores f32[CAPACITY], later reused for the P.V partials i32[CHUNK_TILES * HEAD_DIM]
+//      | probabilities u8[CAPACITY] | quad sums f32[CAPACITY/4]
+//      | per tile: max, rescale, running max f32[3 * MAX_TILES] | block maxima f32[256] | final partial sums f32[4]
+constexpr unsigned SCORE_PV_BYTES =
+	CAPACITY * 4 > CHUNK_TILES * HEAD_DIM * 4 ? CAPACITY * 4 : CHUNK_TILES * HEAD_DIM * 4;
+constexpr unsigned SMEM_BYTES = SCORE_PV_BYTES + CAPACITY + CAPACITY + 3 * MAX_TILES * 4 + 256 * 4 + 16;
 
 }} // namespace x17::decode_tile
