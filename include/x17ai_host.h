@@ -32,7 +32,10 @@ typedef struct X17hDecodeKernel X17hDecodeKernel;   /* single-token decode; no r
 /* DType, src/dtype.rs:1-15 */
 enum { X17H_E4M3 = 0, X17H_INT8 = 1, X17H_BF16 = 2, X17H_F32 = 3 };
 /* epilogues, src/device/cuda/gemm.rs:322-349 */
-enum { X17H_EPI_SCALE = 0, X17H_EPI_GEGLU = 1, X17H_EPI_RESIDUAL = 2, X17H_EPI_RMSNORM = 3 };
+enum { X17H_EPI_SCALE = 0, X17H_EPI_GEGLU = 1, X17H_EPI_RESIDUAL = 2, X17H_EPI_RMSNORM = 3,
+       /* no counterpart in gemm.rs: run-time per-row x per-column f32 scales, bf16 output */
+       X17H_EPI_DEQUANT = 4 };
+enum { X17H_ACT_NONE = 0, X17H_ACT_GEGLU = 1 };
 
 char const *x17h_last_error(void);
 /* text of the warnings/errors collected by the last *_new call (kernel generation diagnostics) */
@@ -78,6 +81,7 @@ typedef struct X17hGemmConfig {
 	size_t head_dim;         /* RMSNorm only */
 	size_t sep_dim;          /* RMSNorm only */
 	int strict_math;         /* 1: deterministic transcendentals (parity build), 0: hardware ones */
+	int activation;          /* Dequant only: X17H_ACT_* */
 } X17hGemmConfig;
 
 /* GemmKernel::<E>::new, gemm.rs:368-437.  dev == NULL: generate and compile only. */
@@ -85,6 +89,10 @@ int x17h_gemm_kernel_new(X17hDevice *dev, char const *kernel_name, X17hGemmConfi
 void x17h_gemm_kernel_free(X17hGemmKernel *k);
 /* GemmKernel::launch, gemm.rs:439-443; extra = rrms (RMSNorm) / residual (Residual) / NULL */
 int x17h_gemm_kernel_launch(X17hGemmKernel *k, X17hTensor *a, X17hTensor *b, X17hTensor *c, X17hTensor *extra);
+/* Dequant epilogue: c[m, n] = bf16((acc * row_scale[m]) * col_scale[n]), or GeGLU over column pairs of that;
+ * row_scale f32 [M], col_scale f32 [N_raw].  No counterpart in the reference (its scales are constants). */
+int x17h_gemm_kernel_launch_dequant(X17hGemmKernel *k, X17hTensor *a, X17hTensor *b, X17hTensor *c,
+                                    X17hTensor *row_scale, X17hTensor *col_scale);
 /* GemmKernel::n_ops, gemm.rs:445-449 */
 double x17h_gemm_kernel_n_ops(X17hGemmKernel *k, X17hTensor *a, X17hTensor *b);
 /* launch geometry read back from meta.json: THREADS_PER_BLOCK, SMEM_BYTES, M_PER_BLOCK, N_PER_BLOCK */

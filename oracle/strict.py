@@ -171,6 +171,19 @@ def epilogue_residual(acc, residual, inp_scale: float, out_scale: float, store: 
 	return c
 
 
+def epilogue_dequant(acc, row_scale, col_scale, geglu: bool = False) -> np.ndarray:
+	"""bf16 bits (uint16) of (f32(acc) * row_scale[m]) * col_scale[n], optionally through GeGLU over column pairs."""
+	acc, is_f32 = _acc_args(acc)
+	m, n = acc.shape
+	row_scale = np.ascontiguousarray(row_scale, dtype=np.float32).reshape(-1)
+	col_scale = np.ascontiguousarray(col_scale, dtype=np.float32).reshape(-1)
+	assert row_scale.shape == (m,) and col_scale.shape == (n,)
+	out = np.empty((m, n // 2 if geglu else n), dtype=np.uint16)
+	lib().x17o_epilogue_dequant(_p(acc), ctypes.c_int(is_f32), _p(row_scale), _p(col_scale), _p(out), _sz(m), _sz(n),
+	                            ctypes.c_int(int(geglu)))
+	return out
+
+
 def epilogue_l2norm(acc, head_dim: int, eps: float, inp_scale: float, out_scale: float):
 	"""Returns (kv codes int8 [M, N_raw], rrms float32 [M, N_raw / (2*head_dim)]).
 

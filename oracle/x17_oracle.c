@@ -314,6 +314,40 @@ X17_EXPORT void x17o_epilogue_geglu(const void *acc, int acc_is_f32, uint8_t *C,
 	}
 }
 
+/* Dequantising writer with per-row and per-column scales (no counterpart in the reference, whose
+ * scales are compile-time constants; precedent for the bf16 store: cuda/gemm_b16.cuh:264-294).
+ * t = (f32(acc) * row_scale[m]) * col_scale[n], two f32 multiplies in that order; optional GeGLU over
+ * column pairs with the gelu of cuda/utils_core.cuh:426-448 at unit scales; round to nearest even bf16. */
+static inline uint16_t bf16_rne(float v) {
+	uint32_t b = f2u(v);
+	return (uint16_t)((b + 0x7FFFu + ((b >> 16) & 1u)) >> 16);
+}
+X17_EXPORT void x17o_epilogue_dequant(const void *acc, int acc_is_f32, const float *row_scale,
+                                      const float *col_scale, uint16_t *C, size_t M, size_t N_raw, int geglu) {
+	double ck = constexpr_sqrt(2.0 * X17_INV_PI);
+	float fck = (float)ck, fck3 = (float)(0.044715 * ck), fy = 0.5f;
+	#pragma omp parallel for schedule(static)
+	for (size_t m = 0; m < M; ++m) {
+		if (!geglu) {
+			for (size_t n = 0; n < N_raw; ++n) {
+				float t = (acc_at(acc, acc_is_f32, m * N_raw + n) * row_scale[m]) * col_scale[n];
+				C[m * N_raw + n] = bf16_rne(t);
+			}
+		} else {
+			size_t N = N_raw / 2;
+			for (size_t j = 0; j < N; ++j) {
+				float x = (acc_at(acc, acc_is_f32, m * N_raw + 2 * j) * row_scale[m]) * col_scale[2 * j];
+				float lin = (acc_at(acc, acc_is_f32, m * N_raw + 2 * j + 1) * row_scale[m]) * col_scale[2 * j + 1];
+				float x2 = x * x;
+				float s = fmaf(fck3 * x, x2, fck * x);
+				float t = sfu_tanh(s);
+				float gate = fmaf(fy * x, t, fy * x);
+				C[m * N + j] = bf16_rne(gate * lin);
+			}
+		}
+	}
+}
+
 /* ResidualMatrixWriter cuda/gemm_b8.cuh:443-622 (residual_gate :484-505),
  * sigmoid_base4 cuda/utils_core.cuh:397-405, imprecise_softplus_base4 :468-483. */
 X17_EXPORT void x17o_epilogue_residual(const void *acc, int acc_is_f32, const int8_t *R,

@@ -60,6 +60,47 @@ def test_config2_ffn_pair_sampled_rows(dev):
 	assert np.count_nonzero(np.abs(got_f.astype(np.int32)).sum(axis=1) == 0) == 0
 
 
+def test_config2_literal_per_token_per_channel_scales(dev):
+	"""BASELINE config 2 as worded: x ~ N(0,1) per-token int8 (absmax / 127), W1 [2048 x 8192 (x2 gated)] and
+	W2 [8192 x 2048] ~ N(0, 1/sqrt(fan_in)) per-output-channel int8, int32 accumulate, fused dequantisation +
+	GeGLU, bf16 out; the bf16 activations are re-quantised per token for the second GEMM.  Sampled rows
+	against the oracle, bit for bit, and the whole against the float64 computation it approximates."""
+	m, d, f = 8192, 2048, 8192
+	rng = rng_for("full-config2-literal")
+
+	def quant(x):
+		scale = (np.abs(x).max(axis=1, keepdims=True) / np.float32(127.0)).astype(np.float32)
+		return np.clip(np.rint(x / scale), -127, 127).astype(np.int8), scale.reshape(-1)
+
+	xf = rng.standard_normal((m, d), dtype=np.float32)
+	w1f = rng.standard_normal((2 * f, d), dtype=np.float32) / np.float32(math.sqrt(d))
+	w2f = rng.standard_normal((d, f), dtype=np.float32) / np.float32(math.sqrt(f))
+	x, xs = quant(xf)
+	w1, w1s = quant(w1f)
+	w2, w2s = quant(w2f)
+	k1 = recipes.dequant_gemm_kernel(dev, d, 2 * f, X.INT8, X.INT8, True, True)
+	k2 = recipes.dequant_gemm_kernel(dev, f, d, X.INT8, X.INT8, False, True)
+	h_t = X.Tensor(dev, (m, f), X.BF16)
+	k1.launch_dequant(_up(dev, x, X.INT8), _up(dev, w1, X.INT8), h_t, _up(dev, xs, X.F32), _up(dev, w1s, X.F32))
+	h_bits = h_t.download()
+	hf = (h_bits.astype(np.uint32) << 16).view(np.float32)
+	h, hs = quant(hf)                                       # host-side requantisation between the two GEMMs
+	y_t = X.Tensor(dev, (m, d), X.BF16)
+	k2.launch_dequant(_up(dev, h, X.INT8), _up(dev, w2, X.INT8), y_t, _up(dev, hs, X.F32), _up(dev, w2s, X.F32))
+	y_bits = y_t.download()
+	rows = _sample_rows(rng, m, 64)
+	assert np.array_equal(h_bits[rows], S.epilogue_dequant(S.gemm_i32(x[rows], w1), xs[rows], w1s, True))
+	assert np.array_equal(y_bits[rows], S.epilogue_dequant(S.gemm_i32(h[rows], w2), hs[rows], w2s, False))
+	# dequantised outputs against the float computation on a row sample: relative L2 and max-abs error
+	g = xf[rows].astype(np.float64) @ w1f.astype(np.float64).T
+	gate, lin = g[:, 0::2], g[:, 1::2]
+	h_ref = 0.5 * gate * (1.0 + np.tanh(math.sqrt(2.0 / math.pi) * (gate + 0.044715 * gate ** 3))) * lin
+	y_ref = h_ref @ w2f.astype(np.float64).T
+	y_got = (y_bits[rows].astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+	rel_l2 = np.linalg.norm(y_got - y_ref) / np.linalg.norm(y_ref)
+	assert rel_l2 < 0.05 and np.abs(y_got - y_ref).max() < 0.25, (rel_l2, np.abs(y_got - y_ref).max())
+
+
 def test_config2_checksum_of_checksums(dev):
 	"""Column sums of an int8 GEMM are linear in the token rows: sum_m C[m, n] = (sum_m A[m, :]) . B[n, :].
 	With +-1/0 operands sparse enough that no accumulator leaves the FixedI8 range, a scale-1 epilogue

@@ -168,6 +168,73 @@ def test_fp8_geglu(dev, m, k, n):
 	assert neq < 5e-3 and beyond == 0.0, (neq, beyond)
 
 
+def _absmax_quantize(x, axis):
+	"""Symmetric int8 with scale = absmax / 127 along `axis` (f32 arithmetic)."""
+	x = x.astype(np.float32)
+	scale = (np.abs(x).max(axis=axis, keepdims=True) / np.float32(127.0)).astype(np.float32)
+	codes = np.clip(np.rint(x / scale), -127, 127).astype(np.int8)
+	return codes, scale.reshape(-1)
+
+
+@pytest.mark.parametrize("geglu", [False, True])
+def test_dequant_epilogue_per_row_per_channel_scales(dev, geglu):
+	"""Run-time per-token x per-output-channel scales, bf16 out (no counterpart in the reference: defined by
+	the oracle's two-multiply order).  Strict build bit-exact; speed build within bf16 ulps; and the
+	dequantised product close to the float matmul it approximates."""
+	m, k, n = 512, 1024, 512
+	rng = rng_for("dequant", geglu)
+	xf = rng.standard_normal((m, k), dtype=np.float32)
+	wf = rng.standard_normal((n, k), dtype=np.float32) / np.float32(math.sqrt(k))
+	a, rs = _absmax_quantize(xf, 1)
+	b, cs = _absmax_quantize(wf, 1)
+	acc = S.gemm_i32(a, b)
+	want = S.epilogue_dequant(acc, rs, cs, geglu)
+	outs = {}
+	for strict in (True, False):
+		kern = recipes.dequant_gemm_kernel(dev, k, n, X.INT8, X.INT8, geglu, strict)
+		c = X.Tensor(dev, (m, n // 2 if geglu else n), X.BF16)
+		kern.launch_dequant(_up(dev, a, X.INT8), _up(dev, b, X.INT8), c, _up(dev, rs, X.F32), _up(dev, cs, X.F32))
+		outs[strict] = c.download()
+	assert np.array_equal(outs[True], want)
+	d = np.abs(outs[False].astype(np.int32) - want.astype(np.int32))
+	# one bf16 ulp, except where 1 + tanh cancels: there the two gelu formulations differ by several ulps of a
+	# tiny value, bounded absolutely
+	assert np.mean(d > 1) < 1e-3 and np.mean(d > 0) < 0.02, (d.max(), np.mean(d > 1), np.mean(d > 0))
+	fast_f = (outs[False].astype(np.uint32) << 16).view(np.float32)
+	want_f = (want.astype(np.uint32) << 16).view(np.float32)
+	assert np.allclose(fast_f, want_f, rtol=2.0 ** -7, atol=float(np.abs(want_f).max()) * 1e-5)
+	# what it approximates: x @ w^T (then GeGLU) in float64; int8 quantisation noise only
+	got_f = (outs[True].astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+	ref = xf.astype(np.float64) @ wf.astype(np.float64).T
+	if geglu:
+		g, l = ref[:, 0::2], ref[:, 1::2]
+		ref = 0.5 * g * (1.0 + np.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g ** 3))) * l
+	rel_l2 = np.linalg.norm(got_f - ref) / np.linalg.norm(ref)
+	assert rel_l2 < 0.03, rel_l2
+
+
+def test_dequant_epilogue_fp8_per_tensor_scales(dev):
+	"""e4m3 x e4m3 with per-tensor scales (constant scale vectors), f32 accumulate, bf16 out."""
+	m, k, n = 256, 512, 256
+	rng = rng_for("dequant-f8")
+	a, b = e4m3_bytes(rng, (m, k)), e4m3_bytes(rng, (n, k))
+	rs = np.full(m, 0.75, np.float32)
+	cs = np.full(n, 1.0 / math.sqrt(k), np.float32)
+	want = S.epilogue_dequant(S.gemm_f32_seq(a, True, b, True), rs, cs, False)
+	kern = recipes.dequant_gemm_kernel(dev, k, n, X.E4M3, X.E4M3, False, True)
+	c = X.Tensor(dev, (m, n), X.BF16)
+	kern.launch_dequant(_up(dev, a, X.E4M3), _up(dev, b, X.E4M3), c, _up(dev, rs, X.F32), _up(dev, cs, X.F32))
+	got_bits = c.download()
+	got = (got_bits.astype(np.uint32) << 16).view(np.float32)
+	ref = (want.astype(np.uint32) << 16).view(np.float32)
+	# the matrix cores add the f32 products in another order than the oracle: one bf16 ulp, plus an absolute
+	# slack of 1e-4 of the largest output for sums that cancel
+	assert np.allclose(got, ref, rtol=2.0 ** -7, atol=float(np.abs(ref).max()) * 1e-4)
+	assert np.mean(got_bits != want) < 0.05
+	with pytest.raises(X.X17Error, match="row-scale and a column-scale"):
+		kern.launch(_up(dev, a, X.E4M3), _up(dev, b, X.E4M3), c)
+
+
 def test_launch_rejects_bad_arguments(dev):
 	"""Shape / dtype / device checks of the launcher (src/device/cuda/tensor_check.rs, gemm.rs:591-616)."""
 	k, n = 128, 256

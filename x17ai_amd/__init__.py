@@ -10,12 +10,12 @@ kernel launch and raises X17Error if the libraries, the code objects or a GPU ar
 from ._ffi import X17Error, lib_paths
 from .api import (
 	BF16, E4M3, F32, INT8,
-	AttnDecodeKernel, AttnKernel, AttnKernelConfig, Device, GeGluConfig, GemmConfig, GemmInputConfig,
+	AttnDecodeKernel, AttnKernel, AttnKernelConfig, DequantConfig, Device, GeGluConfig, GemmConfig, GemmInputConfig,
 	GemmKernel, ResidualConfig, RMSNormConfig, RmsNormKernel, ScaleConfig, Tensor, Timer,
 )
 
 __all__ = [
 	"X17Error", "lib_paths", "BF16", "E4M3", "F32", "INT8", "AttnDecodeKernel", "AttnKernel", "AttnKernelConfig",
-	"Device", "GeGluConfig", "GemmConfig", "GemmInputConfig", "GemmKernel", "ResidualConfig", "RMSNormConfig",
+	"DequantConfig", "Device", "GeGluConfig", "GemmConfig", "GemmInputConfig", "GemmKernel", "ResidualConfig", "RMSNormConfig",
 	"RmsNormKernel", "ScaleConfig", "Tensor", "Timer",
 ]

@@ -36,6 +36,7 @@ class GemmConfigC(ctypes.Structure):
 		("head_dim", ctypes.c_size_t),
 		("sep_dim", ctypes.c_size_t),
 		("strict_math", ctypes.c_int),
+		("activation", ctypes.c_int),
 	]
 
 
@@ -94,6 +95,7 @@ def host() -> ctypes.CDLL:
 	h.x17h_gemm_kernel_free.argtypes = [P]
 	h.x17h_gemm_kernel_free.restype = None
 	h.x17h_gemm_kernel_launch.argtypes = [P, P, P, P, P]
+	h.x17h_gemm_kernel_launch_dequant.argtypes = [P, P, P, P, P, P]
 	h.x17h_gemm_kernel_n_ops.argtypes = [P, P, P]
 	h.x17h_gemm_kernel_n_ops.restype = ctypes.c_double
 	h.x17h_gemm_kernel_metadata.argtypes = [P, ctypes.POINTER(SZ)]

@@ -193,7 +193,17 @@ class RMSNormConfig:            # gemm.rs:38-45
 	kind = 3
 
 
-EpilogueConfig = Union[ScaleConfig, GeGluConfig, ResidualConfig, RMSNormConfig]
+@dataclasses.dataclass
+class DequantConfig:
+	"""No counterpart in gemm.rs: run-time per-row (token) and per-column (output channel) f32 scales,
+	bf16 output, optionally GeGLU over column pairs -- symmetric per-row / per-channel int8 quantisation."""
+	geglu: bool = False
+	inp_scale: float = 1.0
+	out_scale: float = 1.0
+	kind = 4
+
+
+EpilogueConfig = Union[ScaleConfig, GeGluConfig, ResidualConfig, RMSNormConfig, DequantConfig]
 
 
 def _attrs_dict(raw) -> dict:
@@ -222,6 +232,7 @@ class GemmKernel:
 		c.head_dim = getattr(epilogue_config, "head_dim", 0)
 		c.sep_dim = getattr(epilogue_config, "sep_dim", 0)
 		c.strict_math = int(strict_math)
+		c.activation = int(bool(getattr(epilogue_config, "geglu", False)))
 		self.device = device
 		self.name = kernel_name
 		self.epilogue_kind = epilogue_config.kind
@@ -232,6 +243,9 @@ class GemmKernel:
 
 	def launch(self, a: Tensor, b: Tensor, c: Tensor, extra: Optional[Tensor] = None) -> None:
 		check(_ffi.host().x17h_gemm_kernel_launch(self._h, a._h, b._h, c._h, extra._h if extra is not None else None))
+
+	def launch_dequant(self, a: Tensor, b: Tensor, c: Tensor, row_scale: Tensor, col_scale: Tensor) -> None:
+		check(_ffi.host().x17h_gemm_kernel_launch_dequant(self._h, a._h, b._h, c._h, row_scale._h, col_scale._h))
 
 	def n_ops(self, a: Tensor, b: Tensor) -> float:
 		return float(_ffi.host().x17h_gemm_kernel_n_ops(self._h, a._h, b._h))

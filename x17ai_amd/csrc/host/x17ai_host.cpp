@@ -570,7 +570,7 @@ std::unique_ptr<GemmKernel> GemmKernel::create(std::shared_ptr<HipDevice> device
 	common << "#define X17_A_COLS " << g.a.cols << "\n#define X17_B_ROWS " << b_rows << "\n";
 	common << "#define X17_A_KIND " << kind_of(g.a.dtype) << "\n#define X17_B_KIND " << kind_of(g.b.dtype) << "\n";
 	common << "#define X17_EPILOGUE " << kind << "\n";
-	common << "#define X17_STORE " << (g.c_dtype == DType::E4m3 ? 1 : 0) << "\n";
+	common << "#define X17_STORE " << (g.c_dtype == DType::E4m3 ? 1 : (g.c_dtype == DType::Bf16 ? 2 : 0)) << "\n";
 	common << "#define X17_STRICT_MATH " << (strict_math ? 1 : 0) << "\n";
 
 	auto finite_pos = [](double v) { return std::isfinite(v) && v > 0.0; };
@@ -592,6 +592,11 @@ std::unique_ptr<GemmKernel> GemmKernel::create(std::shared_ptr<HipDevice> device
 		if (b_rows % 2 != 0) { diag.add_error("Residual GEMM requires an even raw output column count"); return nullptr; }
 		common << "#define X17_INP_SCALE " << format_cpp_f64(c->inp_scale.value) << " // " << c->inp_scale.description << "\n";
 		common << "#define X17_OUT_SCALE " << format_cpp_f64(c->out_scale.value) << " // " << c->out_scale.description << "\n";
+	} else if (auto const *c = std::get_if<DequantConfig>(&e)) {
+		if (g.c_dtype != DType::Bf16) { diag.add_error("Dequant epilogue requires a bf16 output"); return nullptr; }
+		if (c->geglu && b_rows % 2 != 0) { diag.add_error("Dequant GeGLU GEMM requires an even raw output column count"); return nullptr; }
+		common << "#define X17_DEQ_GEGLU " << (c->geglu ? 1 : 0) << "\n";
+		common << "#define X17_INP_SCALE 1.0\n#define X17_OUT_SCALE 1.0\n";      // the scales arrive at run time
 	} else if (auto const *c = std::get_if<RMSNormConfig>(&e)) {
 		if (g.c_dtype != DType::Int8) { diag.add_error("RMSNorm epilogue requires an i8 output"); return nullptr; }
 		if (g.a.dtype != DType::Int8 || g.b.dtype != DType::Int8) { diag.add_error("RMSNorm epilogue requires i8 inputs"); return nullptr; }
@@ -645,6 +650,7 @@ std::unique_ptr<GemmKernel> GemmKernel::create(std::shared_ptr<HipDevice> device
 	out->c_dtype = g.c_dtype;
 	out->head_dim = head_dim;
 	out->sep_dim = sep_dim;
+	if (auto const *c = std::get_if<DequantConfig>(&e)) out->dequant_geglu = c->geglu;
 	if (device) {
 		out->kernel = kernel_build::load_kernel(*device->stream, built->code_object_path, "kernel", out->metadata.SMEM_BYTES, diag);
 		if (!out->kernel) return nullptr;
@@ -668,7 +674,7 @@ Status GemmKernel::launch(GemmArgs const &args) {
 	s = tensor_check::matrix_shape(op, "b", *args.b, b_rows, a_cols, *device, b_dtype, b_shape);
 	if (!s.is_ok()) return s;
 	size_t const a_rows = a_shape[0], b_rows_v = b_shape[0];
-	bool const halves = epilogue_kind == 1 || epilogue_kind == 2;
+	bool const halves = epilogue_kind == 1 || epilogue_kind == 2 || (epilogue_kind == 4 && dequant_geglu);
 	if (halves && b_rows_v % 2 != 0) {
 		return Status::err(TensorOpError::Other, std::string(epilogue_kind == 2 ? "Residual" : "GeGLU")
 			+ " GEMM requires an even raw output column count, got " + std::to_string(b_rows_v));
@@ -685,6 +691,15 @@ Status GemmKernel::launch(GemmArgs const &args) {
 		return Status::err(TensorOpError::Other, std::string(op) + " raw output shape [" + std::to_string(a_rows) + ", "
 			+ std::to_string(b_rows_v) + "] must be divisible by tile shape [" + std::to_string(metadata.M_PER_BLOCK) + ", "
 			+ std::to_string(metadata.N_PER_BLOCK) + "]");
+	}
+	if (epilogue_kind == 4) {
+		if (args.extra == nullptr || args.extra2 == nullptr) {
+			return Status::err(TensorOpError::Other, "Dequant GEMM needs a row-scale and a column-scale tensor");
+		}
+		s = tensor_check::vector_shape(op, "row_scale", *args.extra, a_rows, *device, DType::F32);
+		if (!s.is_ok()) return s;
+		s = tensor_check::vector_shape(op, "col_scale", *args.extra2, b_rows_v, *device, DType::F32);
+		if (!s.is_ok()) return s;
 	}
 	if (epilogue_kind == 3) {
 		if (args.extra == nullptr) return Status::err(TensorOpError::Other, "RMSNorm GEMM needs an rrms tensor");
@@ -703,7 +718,8 @@ Status GemmKernel::launch(GemmArgs const &args) {
 	size_t b_rows_arg = b_rows_v;
 	void *c_ptr = args.c->ptr;
 	void *extra_ptr = args.extra != nullptr ? args.extra->ptr : nullptr;
-	void *raw_args[6] = {&a_ptr, &a_rows_arg, &b_ptr, &b_rows_arg, &c_ptr, &extra_ptr};
+	void *extra2_ptr = args.extra2 != nullptr ? args.extra2->ptr : nullptr;
+	void *raw_args[7] = {&a_ptr, &a_rows_arg, &b_ptr, &b_rows_arg, &c_ptr, &extra_ptr, &extra2_ptr};
 	size_t grid[3] = {grid_x, grid_y, 1};
 	if (metadata.MAX_BLOCKS != 0 && grid_x * grid_y > metadata.MAX_BLOCKS) {
 		// persistent kernel: the workgroups share the tiles out among themselves
@@ -1099,6 +1115,7 @@ int x17h_gemm_kernel_new(X17hDevice *dev, char const *kernel_name, X17hGemmConfi
 			case X17H_EPI_GEGLU: e = GeGluConfig{inp, outs}; break;
 			case X17H_EPI_RESIDUAL: e = ResidualConfig{inp, outs}; break;
 			case X17H_EPI_RMSNORM: e = RMSNormConfig{c->eps, c->head_dim, c->sep_dim, inp, outs}; break;
+			case X17H_EPI_DEQUANT: e = DequantConfig{c->activation == X17H_ACT_GEGLU}; break;
 			default: return fail("unknown epilogue");
 		}
 		Diagnostics diag;
@@ -1113,6 +1130,14 @@ void x17h_gemm_kernel_free(X17hGemmKernel *k) { delete k; }
 int x17h_gemm_kernel_launch(X17hGemmKernel *k, X17hTensor *a, X17hTensor *b, X17hTensor *c, X17hTensor *extra) {
 	if (a == nullptr || b == nullptr || c == nullptr) return fail("GEMM launch needs a, b and c");
 	GemmArgs args{a->t.get(), b->t.get(), c->t.get(), extra != nullptr ? extra->t.get() : nullptr};
+	return from_status(k->k->launch(args));
+}
+int x17h_gemm_kernel_launch_dequant(X17hGemmKernel *k, X17hTensor *a, X17hTensor *b, X17hTensor *c,
+                                    X17hTensor *row_scale, X17hTensor *col_scale) {
+	if (a == nullptr || b == nullptr || c == nullptr || row_scale == nullptr || col_scale == nullptr) {
+		return fail("dequant GEMM launch needs a, b, c, row_scale and col_scale");
+	}
+	GemmArgs args{a->t.get(), b->t.get(), c->t.get(), row_scale->t.get(), col_scale->t.get()};
 	return from_status(k->k->launch(args));
 }
 double x17h_gemm_kernel_n_ops(X17hGemmKernel *k, X17hTensor *a, X17hTensor *b) { return k->k->n_ops(*a->t, *b->t); }

@@ -187,7 +187,10 @@ struct ScaleConfig { Scale inp_scale, out_scale; };
 struct RMSNormConfig { double eps; size_t head_dim; size_t sep_dim; Scale inp_scale, out_scale; };
 struct ResidualConfig { Scale inp_scale, out_scale; };
 struct GeGluConfig { Scale inp_scale, out_scale; };
-using EpilogueConfig = std::variant<ScaleConfig, GeGluConfig, ResidualConfig, RMSNormConfig>;   // index = X17_EPILOGUE
+// Run-time per-row and per-column dequantisation scales, bf16 output, optional GeGLU over column pairs
+// (no counterpart in gemm.rs: the superset for symmetric per-row / per-channel int8 quantisation).
+struct DequantConfig { bool geglu; };
+using EpilogueConfig = std::variant<ScaleConfig, GeGluConfig, ResidualConfig, RMSNormConfig, DequantConfig>;   // index = X17_EPILOGUE
 
 struct GemmInputConfig { DType dtype; size_t cols; std::optional<size_t> rows; bool trans; };
 struct GemmConfig { GemmInputConfig a, b; DType c_dtype; };
@@ -197,7 +200,8 @@ struct GemmLauncherMetadata { size_t THREADS_PER_BLOCK, SMEM_BYTES, M_PER_BLOCK,
 
 struct GemmArgs {
 	Tensor const *a; Tensor const *b; Tensor const *c;
-	Tensor const *extra;     // rrms (RMSNorm epilogue) or residual (Residual epilogue), else null
+	Tensor const *extra;     // rrms (RMSNorm epilogue), residual (Residual epilogue) or row scales (Dequant), else null
+	Tensor const *extra2 = nullptr;   // column scales (Dequant epilogue)
 };
 
 struct GemmKernel {
@@ -208,6 +212,7 @@ struct GemmKernel {
 	std::optional<size_t> b_rows;
 	DType a_dtype, b_dtype, c_dtype;
 	size_t head_dim = 0, sep_dim = 0;
+	bool dequant_geglu = false;
 	GemmLauncherMetadata metadata{};
 	std::shared_ptr<HipDevice> device;    // null for a build-only kernel
 	std::unique_ptr<HipKernel> kernel;

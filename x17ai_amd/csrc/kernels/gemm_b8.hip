@@ -26,7 +26,8 @@
 //
 // common.h (generated per kernel by the host-side kernel builder) provides:
 //   X17_A_COLS (K), X17_B_ROWS (N_raw), X17_A_KIND / X17_B_KIND (0 = int8, 1 = e4m3),
-//   X17_EPILOGUE (0 scale, 1 geglu, 2 residual, 3 l2norm), X17_STORE (0 FixedI8, 1 e4m3),
+//   X17_EPILOGUE (0 scale, 1 geglu, 2 residual, 3 l2norm, 4 dequant), X17_STORE (0 FixedI8, 1 e4m3; dequant
+//   always stores bf16), X17_DEQ_GEGLU (dequant only: 0 plain, 1 GeGLU over column pairs),
 //   X17_INP_SCALE, X17_OUT_SCALE, and for l2norm X17_HEAD_DIM, X17_EPS, X17_HEAD_SCALE,
 //   X17_SEP_SCALE (doubles), X17_STRICT_MATH.
 
@@ -189,6 +190,48 @@ struct ResidualEpilogue {
 		}
 	}
 };
+
+// Dequantising writer: per-row (token) and per-column (output channel) f32 scales, bf16 output, optional
+// GeGLU over column pairs.  The reference folds its scales into compile-time constants; this is the
+// run-time-scale superset for symmetric per-row / per-channel int8 quantisation (bf16 store precedent:
+// cuda/gemm_b16.cuh:264-294).  t = (x * row_scale) * col_scale, two f32 multiplies in that order.
+#if X17_EPILOGUE == 4
+struct DequantEpilogue {
+	static constexpr bool GEGLU = X17_DEQ_GEGLU != 0;
+	static constexpr u32 OUT_COLS = GEGLU ? N_RAW / 2 : N_RAW;
+	X17_DEV static void run(f32 const (&x)[64], u8 *c, u32 row, u32 n, f32 const *row_scale, f32 const *col_scale) {
+		f32 const rs = row_scale[row];
+		f32 t[64];
+		X17_UNROLL for (int v = 0; v < 16; ++v) {
+			v4f cs = *reinterpret_cast<v4f const *>(col_scale + n + 4 * v);
+			X17_UNROLL for (int i = 0; i < 4; ++i) t[4 * v + i] = (x[4 * v + i] * rs) * cs[i];
+		}
+		if constexpr (GEGLU) {
+			u8 *dst = c + ((size_t)row * OUT_COLS + n / 2) * 2;
+			X17_UNROLL for (int v = 0; v < 4; ++v) {
+				v4u pack;
+				X17_UNROLL for (int w = 0; w < 4; ++w) {
+					int j = 8 * v + 2 * w;
+					u32 lo = f32_to_bf16_rne(GeGluEpilogue::gated(t[2 * j], t[2 * j + 1]));
+					u32 hi = f32_to_bf16_rne(GeGluEpilogue::gated(t[2 * j + 2], t[2 * j + 3]));
+					pack[w] = lo | (hi << 16);
+				}
+				*reinterpret_cast<v4u *>(dst + 16 * v) = pack;
+			}
+		} else {
+			u8 *dst = c + ((size_t)row * OUT_COLS + n) * 2;
+			X17_UNROLL for (int v = 0; v < 8; ++v) {
+				v4u pack;
+				X17_UNROLL for (int w = 0; w < 4; ++w) {
+					int j = 8 * v + 2 * w;
+					pack[w] = f32_to_bf16_rne(t[j]) | (f32_to_bf16_rne(t[j + 1]) << 16);
+				}
+				*reinterpret_cast<v4u *>(dst + 16 * v) = pack;
+			}
+		}
+	}
+};
+#endif
 
 // The l2norm epilogue needs more than one lane for head_dim > 64 and is handled in the kernel body.
 #if X17_EPILOGUE == 3
@@ -397,6 +440,8 @@ void kernel(
 	, f32 *rrms
 #elif X17_EPILOGUE == 2
 	, i8 const *residual
+#elif X17_EPILOGUE == 4
+	, f32 const *row_scale, f32 const *col_scale
 #endif
 ) {
 	extern __shared__ __attribute__((aligned(1024))) u8 smem[];
@@ -582,6 +627,8 @@ void kernel(
 		GeGluEpilogue::run(x, c, row, n0, nullptr);
 #elif X17_EPILOGUE == 2
 		ResidualEpilogue::run(x, c, row, n0, residual);
+#elif X17_EPILOGUE == 4
+		DequantEpilogue::run(x, c, row, n0, row_scale, col_scale);
 #else
 		// L2NormMatrixWriter, cuda/gemm_b8.cuh:861-949 with kv_helpers::l2_norm :767-830.
 		// Per head the columns are [K (hd) | V (hd)].  Sum of squares of the K half: four partial

@@ -89,6 +89,12 @@ X17_DEV u32 e4m3_to_bf16_bits(u32 c) {
 	return rest == 0 ? 0u : ((sign | rest) + (120u << 7));
 }
 
+// f32 -> bf16 bits, round to nearest even (finite inputs)
+X17_DEV u32 f32_to_bf16_rne(f32 v) {
+	u32 b = f2u(v);
+	return (b + 0x7FFFu + ((b >> 16) & 1u)) >> 16;
+}
+
 // Four FixedI8 codes packed into one word (a in the low byte).  Same values as f32_to_fixedi8:
 // clamp, then add 1.5 * 2^23 -- the add rounds to an integer, ties to even, exactly like rint, and
 // leaves the two's-complement code in the low byte of the float -- then gather the four low bytes.

@@ -67,6 +67,14 @@ def _specs():
 	# ---- tests/test_gpu_fullsize.py (the strict ffn pair, attention and decode kernels are listed above)
 	add(("attn", 16, 128, True))
 	add(("acc_probe_full",))
+	# ---- tests/test_gpu_gemm.py: run-time dequantisation scales, bf16 out
+	for strict in (True, False):
+		add(("dequant", 1024, 512, INT8, INT8, False, strict))
+		add(("dequant", 1024, 512, INT8, INT8, True, strict))
+	add(("dequant", 512, 256, E4M3, E4M3, False, True))
+	# ---- tests/test_gpu_fullsize.py: BASELINE config 2 in its literal form (per-token / per-channel scales)
+	add(("dequant", 2048, 16384, INT8, INT8, True, True))
+	add(("dequant", 8192, 2048, INT8, INT8, False, True))
 	return s
 
 
@@ -90,6 +98,8 @@ def _build_one(spec) -> str:
 		return recipes.attn_decode_kernel(None, spec[1], spec[2], spec[3], spec[4]).name
 	if kind == "rms_norm":
 		return recipes.rms_norm_kernel(None, spec[1], spec[2]).name
+	if kind == "dequant":
+		return recipes.dequant_gemm_kernel(None, spec[1], spec[2], spec[3], spec[4], spec[5], spec[6]).name
 	if kind == "copy_probe":
 		from .api import CopyProbe
 		CopyProbe(None)

@@ -10,8 +10,8 @@ import math
 from typing import Optional
 
 from .api import (
-	E4M3, INT8,
-	AttnDecodeKernel, AttnKernel, AttnKernelConfig, Device, GeGluConfig, GemmConfig, GemmInputConfig, GemmKernel,
+	BF16, E4M3, INT8,
+	AttnDecodeKernel, AttnKernel, AttnKernelConfig, Device, DequantConfig, GeGluConfig, GemmConfig, GemmInputConfig, GemmKernel,
 	ResidualConfig, RMSNormConfig, RmsNormKernel, ScaleConfig,
 )
 
@@ -95,6 +95,16 @@ def ffn_f_f8_kernel(device: Optional[Device], model_dim: int, ffn_f_proj_outputs
 	cfg = GeGluConfig(_inv_sqrt(model_dim), 1.0)
 	return GemmKernel(device, f"ffn_f_fwd_f8-k{model_dim}-n{ffn_f_proj_outputs}-{_mode(strict)}",
 	                  _gemm(E4M3, E4M3, E4M3, model_dim, ffn_f_proj_outputs), cfg, strict)
+
+
+def dequant_gemm_kernel(device: Optional[Device], k: int, n_raw: int, a_dtype: int = INT8, b_dtype: int = INT8,
+                        geglu: bool = False, strict: bool = True) -> GemmKernel:
+	"""No counterpart in src/main.rs: a[M, k] . b[n_raw, k]^T with run-time per-row and per-column f32
+	dequantisation scales -> bf16 [M, n_raw] (or GeGLU over column pairs -> bf16 [M, n_raw / 2]).  This is
+	the literal form of symmetric per-token / per-output-channel int8 (scale = absmax / 127) and of e4m3
+	operands with per-tensor scales."""
+	name = f"dequant_gemm-a{a_dtype}b{b_dtype}-k{k}-n{n_raw}-{'geglu' if geglu else 'plain'}-{_mode(strict)}"
+	return GemmKernel(device, name, _gemm(a_dtype, b_dtype, BF16, k, n_raw), DequantConfig(geglu), strict)
 
 
 def rms_norm_kernel(device: Optional[Device], model_dim: int, in_dtype: int = E4M3, eps: float = L2_NORM_EPS) -> RmsNormKernel:
