@@ -141,7 +141,22 @@ def extras(dev, X, recipes):
 		tag = "strict" if strict else "fast"
 		c2[f"ffn_f_{tag}"] = gemm_entry(recipes.ffn_f_kernel(dev, D, 2 * F, strict, X.INT8), x, w1, f, None, PEAK_INT8_TOPS)
 		c2[f"ffn_y_{tag}"] = gemm_entry(recipes.ffn_y_kernel(dev, D, F, strict, X.INT8, X.INT8), f, w2, y, x, PEAK_INT8_TOPS)
+	# the same pair in the literal form of the config text: per-token / per-output-channel scale vectors
+	# applied in the epilogue, bf16 out (W2 ungated: N_raw = d_model)
+	rs = X.Tensor.from_numpy(dev, (0.01 + 0.01 * rng.random(M)).astype(np.float32), X.F32)
+	cs1 = X.Tensor.from_numpy(dev, (0.01 + 0.01 * rng.random(2 * F)).astype(np.float32), X.F32)
+	cs2 = X.Tensor.from_numpy(dev, (0.01 + 0.01 * rng.random(D)).astype(np.float32), X.F32)
+	w2l = X.Tensor.from_numpy(dev, _rand_codes(rng, (D, F)), X.INT8)
+	hb = X.Tensor(dev, (M, F), X.BF16)
+	yb = X.Tensor(dev, (M, D), X.BF16)
+	kd1 = recipes.dequant_gemm_kernel(dev, D, 2 * F, X.INT8, X.INT8, True, False)
+	kd2 = recipes.dequant_gemm_kernel(dev, F, D, X.INT8, X.INT8, False, False)
+	for name, kern, a_, b_, c_, cs_ in (("dequant_geglu_bf16", kd1, x, w1, hb, cs1), ("dequant_bf16", kd2, f, w2l, yb, cs2)):
+		med, mn = _median_launch(dev, X, lambda: kern.launch_dequant(a_, b_, c_, rs, cs_), 20, 5)
+		ops = kern.n_ops(a_, b_)
+		c2[name] = {"median_us": med * 1e6, "min_us": mn * 1e6, "tops": ops / med / 1e12, "frac_of_peak": ops / med / 1e12 / PEAK_INT8_TOPS}
 	out["config2_int8_ffn"] = c2
+	del rs, cs1, cs2, w2l, hb, yb
 	del w1, w2, f, y
 
 	# ---- config 3: all-fp8 FFN, tokens=16384, d_model=4096, d_ff=16384

@@ -124,6 +124,31 @@ def test_geglu_epilogue_against_float64():
 	assert np.abs(got8 - want8).max() <= 1 and np.mean(got8 != want8) < 1e-3
 
 
+def test_dequant_epilogue_against_torch_bf16_and_tanh_gelu():
+	"""The run-time-scale writer: bf16 rounding against torch's float32 -> bfloat16 cast (a library routine,
+	round to nearest even), the plain form against the same products formed in float32 by torch, and the
+	GeGLU form against torch's tanh-approximated gelu in float64 (within bf16 resolution)."""
+	rng = np.random.default_rng(31)
+	m, n = 48, 64
+	acc = rng.integers(-200000, 200000, (m, n), dtype=np.int32)
+	rs = (rng.random(m) * 1e-3 + 1e-4).astype(np.float32)
+	cs = (rng.random(n) * 1e-2 + 1e-3).astype(np.float32)
+	got = S.epilogue_dequant(acc, rs, cs, False)
+	prod = (torch.from_numpy(acc).to(torch.float32) * torch.from_numpy(rs)[:, None]) * torch.from_numpy(cs)[None, :]
+	want = prod.to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+	assert np.array_equal(got, want)
+	# exact ties round to even: 1 + 2^-8 -> 1.0, 1 + 3 * 2^-8 -> 1 + 2^-6
+	ties = np.array([[1 << 24 | 1 << 16, 1 << 24 | 3 << 16]], dtype=np.int32)        # as integers: 2^24 + 2^16 k
+	one = np.array([2.0 ** -24], np.float32)
+	bits = S.epilogue_dequant(ties, one, np.ones(2, np.float32), False)
+	assert bits.tolist() == [[0x3F80, 0x3F82]]
+	gg = S.epilogue_dequant(acc, rs, cs, True)
+	x = prod.to(torch.float64)
+	ref = torch.nn.functional.gelu(x[:, 0::2], approximate="tanh") * x[:, 1::2]
+	gg_f = (gg.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+	assert np.allclose(gg_f, ref.numpy(), rtol=2.0 ** -7, atol=1e-6 * float(ref.abs().max()))
+
+
 def test_residual_epilogue_against_float64_and_identities():
 	acc = _acc(8, 256, 1024)
 	r = _rng(9)
