@@ -216,6 +216,8 @@ void kernel(
 		u32 const visible = qi < wr ? qi : wr;
 		f32 temperature = BASE_TEMPERATURE * strict::lg2(f32(visible + 4u));
 		temperature = temperature * attn_temperature[head];
+		// (the sign is the head's: lg2(visible + 4) >= 2)
+		bool const positive_temperature = __builtin_amdgcn_readfirstlane(f2u(attn_temperature[head])) - 1u < 0x7F7FFFFFu;
 
 		i32 sink_dot = 0;
 		X17_UNROLL for (u32 s = 0; s < K_SLICES; ++s) {
@@ -280,18 +282,32 @@ void kernel(
 				bool const need_mask = !(key0 + 31 < q_wave0 && (q_wave0 + 31 - key0) <= wr);
 
 				X17_UNROLL for (u32 tile = 0; tile < 2; ++tile) {
+					// Speed build, tile fully visible, positive temperature: the row maximum is taken over the
+					// integer dots (the scaling is monotone, so f32(max) * temperature IS the maximum score) and
+					// the scaling is fused into the exponent's subtraction further down.
+					bool const int_path = !STRICT && !need_mask && positive_temperature;
 					f32 s[8];
-					X17_UNROLL for (u32 r = 0; r < 8; ++r) s[r] = f32(s_acc[8 * tile + r]) * temperature;
-					if (need_mask) {
-						X17_UNROLL for (u32 r = 0; r < 8; ++r) {
-							u32 j = key0 + 16 * tile + 8 * (r / 4) + 4 * half + (r % 4);
-							bool vis = j < qi && (qi - j) <= wr;
-							s[r] = vis ? s[r] : -__builtin_inff();
+					f32 tmax;
+					if (int_path) {
+						i32 const *a = reinterpret_cast<i32 const *>(&s_acc) + 8 * tile;
+						auto mx = [](i32 x, i32 y) { return x > y ? x : y; };     // pairs of these become v_max3_i32
+						i32 imax = mx(mx(mx(a[0], a[1]), mx(a[2], a[3])), mx(mx(a[4], a[5]), mx(a[6], a[7])));
+						i32 other = partner_i32(imax, half);
+						imax = imax > other ? imax : other;
+						tmax = f32(imax) * temperature;
+					} else {
+						X17_UNROLL for (u32 r = 0; r < 8; ++r) s[r] = f32(s_acc[8 * tile + r]) * temperature;
+						if (need_mask) {
+							X17_UNROLL for (u32 r = 0; r < 8; ++r) {
+								u32 j = key0 + 16 * tile + 8 * (r / 4) + 4 * half + (r % 4);
+								bool vis = j < qi && (qi - j) <= wr;
+								s[r] = vis ? s[r] : -__builtin_inff();
+							}
 						}
+						f32 lmax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fmaxf(s[0], s[1]), __builtin_fmaxf(s[2], s[3])),
+						                           __builtin_fmaxf(__builtin_fmaxf(s[4], s[5]), __builtin_fmaxf(s[6], s[7])));
+						tmax = __builtin_fmaxf(lmax, partner_f32(lmax, half));
 					}
-					f32 lmax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fmaxf(s[0], s[1]), __builtin_fmaxf(s[2], s[3])),
-					                           __builtin_fmaxf(__builtin_fmaxf(s[4], s[5]), __builtin_fmaxf(s[6], s[7])));
-					f32 tmax = __builtin_fmaxf(lmax, partner_f32(lmax, half));
 
 					// cuda/attn_fwd_i8.cuh:233-256 -- rescale only when some row's max grew
 					f32 resc = 1.0f;
@@ -326,7 +342,13 @@ void kernel(
 						X17_UNROLL for (u32 r = 0; r < 8; ++r) p[r] = sfu::ex2(s[r] - m) * PROB_SCALE;
 					} else {
 						f32 const shift = m - LOG2_PROB_SCALE;        // 255 * 2^(s - m) = 2^(s - (m - lg2 255))
-						X17_UNROLL for (u32 r = 0; r < 8; ++r) p[r] = sfu::ex2(s[r] - shift);
+						if (int_path) {
+							X17_UNROLL for (u32 r = 0; r < 8; ++r) {
+								p[r] = sfu::ex2(fmaf32(f32(s_acc[8 * tile + r]), temperature, -shift));
+							}
+						} else {
+							X17_UNROLL for (u32 r = 0; r < 8; ++r) p[r] = sfu::ex2(s[r] - shift);
+						}
 					}
 					f32 add_lo = (p[0] + p[1]) + (p[2] + p[3]);
 					f32 add_hi = (p[4] + p[5]) + (p[6] + p[7]);
