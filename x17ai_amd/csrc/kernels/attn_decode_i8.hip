@@ -61,6 +61,8 @@ void kernel(
 	f32 *s_mrun = s_resc + dt::MAX_TILES;                                        // [MAX_TILES]
 	f32 *s_bmax = s_mrun + dt::MAX_TILES;                                        // [256]
 	f32 *s_sum = s_bmax + 256;                                                   // [4]
+	u32 *s_nact = reinterpret_cast<u32 *>(s_sum + 4);                            // [4] (one used)
+	u16 *s_act = reinterpret_cast<u16 *>(s_nact + 4);                            // [MAX_TILES] tiles that move O
 
 	u32 const tid = threadIdx.x;
 	u32 const head = blockIdx.x;
@@ -189,16 +191,42 @@ void kernel(
 	}
 
 	// ---- phase 4: O chains.  Lane d < HD owns output dim d.
+	// A tile whose sixteen probabilities all rounded to zero and whose rescale factor is exactly 1 leaves O
+	// untouched (O * 1 + 0), and after the first few tiles that is most of them: the last wave lists the
+	// other tiles, in order, and only those are walked.
+	if (tid >= dt::THREADS_PER_BLOCK - 64) {
+		u32 const lane = tid % 64;
+		u32 count = 0;
+		for (u32 base = 0; base < n_tiles; base += 64) {
+			u32 t = base + lane;
+			bool active = false;
+			if (t < n_tiles) {
+				v4u probs = *reinterpret_cast<v4u const *>(s_prob + t * 16);
+				active = (probs[0] | probs[1] | probs[2] | probs[3]) != 0 || s_resc[t] != 1.0f;
+			}
+			unsigned long long const mask = __ballot(active);
+			if (active) {
+				s_act[count + __builtin_popcountll(mask & ((1ull << lane) - 1ull))] = (u16)t;
+			}
+			count += (u32)__builtin_popcountll(mask);
+		}
+		if (lane == 0) {
+			s_nact[0] = count;
+		}
+	}
+	__syncthreads();
+	u32 const n_act = s_nact[0];
+
 	f32 o = 0.0f;
 	if (tid < HD) {
 		o = f32((i32)sink_v[(size_t)head * HD + tid] * 255);
 	}
-	for (u32 chunk = 0; chunk < n_tiles; chunk += dt::CHUNK_TILES) {
-		u32 const tiles_here = n_tiles - chunk < dt::CHUNK_TILES ? n_tiles - chunk : dt::CHUNK_TILES;
+	for (u32 chunk = 0; chunk < n_act; chunk += dt::CHUNK_TILES) {
+		u32 const tiles_here = n_act - chunk < dt::CHUNK_TILES ? n_act - chunk : dt::CHUNK_TILES;
 		// 4a: int32 P.V of one tile x 16 dims per thread
 		u32 const tl = tid / CPR;
 		if (tl < tiles_here) {
-			u32 const t = chunk + tl;
+			u32 const t = s_act[chunk + tl];
 			i32 acc[16];
 			X17_UNROLL for (int i = 0; i < 16; ++i) acc[i] = 0;
 			v4u probs = *reinterpret_cast<v4u const *>(s_prob + t * 16);
@@ -232,14 +260,14 @@ void kernel(
 			for (; tl2 + 8 <= tiles_here; tl2 += 8) {
 				f32 r[8];
 				i32 a[8];
-				X17_UNROLL for (int i = 0; i < 8; ++i) { r[i] = s_resc[chunk + tl2 + i]; a[i] = s_pv[(tl2 + i) * HD + tid]; }
+				X17_UNROLL for (int i = 0; i < 8; ++i) { r[i] = s_resc[s_act[chunk + tl2 + i]]; a[i] = s_pv[(tl2 + i) * HD + tid]; }
 				X17_UNROLL for (int i = 0; i < 8; ++i) {
 					o = o * r[i];
 					o = o + f32(a[i]);
 				}
 			}
 			for (; tl2 < tiles_here; ++tl2) {
-				o = o * s_resc[chunk + tl2];
+				o = o * s_resc[s_act[chunk + tl2]];
 				o = o + f32(s_pv[tl2 * HD + tid]);
 			}
 		}

@@ -16,6 +16,7 @@ constexpr unsigned CHUNK_TILES = 32;                    // tiles whose P.V parti
 //      | per tile: max, rescale, running max f32[3 * MAX_TILES] | block maxima f32[256] | final partial sums f32[4]
 constexpr unsigned SCORE_PV_BYTES =
 	CAPACITY * 4 > CHUNK_TILES * HEAD_DIM * 4 ? CAPACITY * 4 : CHUNK_TILES * HEAD_DIM * 4;
-constexpr unsigned SMEM_BYTES = SCORE_PV_BYTES + CAPACITY + CAPACITY + 3 * MAX_TILES * 4 + 256 * 4 + 16;
+//      | number of listed tiles u32[4] | listed tiles u16[MAX_TILES]
+constexpr unsigned SMEM_BYTES = SCORE_PV_BYTES + CAPACITY + CAPACITY + 3 * MAX_TILES * 4 + 256 * 4 + 16 + 16 + MAX_TILES * 2;
 
 }} // namespace x17::decode_tile
