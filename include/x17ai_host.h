@@ -58,6 +58,11 @@ int x17h_tensor_new_empty(X17hDevice *dev, size_t const *shape, size_t ndim, int
 void x17h_tensor_free(X17hTensor *t);
 int x17h_tensor_upload(X17hTensor *t, void const *src, size_t bytes);      /* async on the device stream */
 int x17h_tensor_download(X17hTensor *t, void *dst, size_t bytes);          /* async; synchronize before reading */
+/* Tensor::from_safetensors_file, src/tensor.rs:155-179: exactly one tensor, dtype F8_E4M3 / I8 / BF16 / F32,
+ * bytes uploaded unchanged.  dev == NULL loads onto the CPU.  shape must have room for 8 dimensions. */
+int x17h_tensor_from_safetensors_file(X17hDevice *dev, char const *path, X17hTensor **out, int *dtype, size_t *shape, size_t *ndim);
+/* Tensor::save_safetensors_file, src/tensor.rs:213-249: CPU tensors only, single entry "tensor" */
+int x17h_tensor_save_safetensors_file(X17hTensor *t, char const *path);
 void *x17h_tensor_device_ptr(X17hTensor *t);
 size_t x17h_tensor_bytes(X17hTensor *t);
 int x17h_tensor_reshape(X17hTensor *t, size_t const *shape, size_t ndim);  /* Tensor::reshape, in place */

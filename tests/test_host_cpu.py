@@ -146,6 +146,89 @@ def test_cpu_tensors_round_trip():
 		t.reshape((5, 5))
 
 
+def test_safetensors_files_round_trip_against_the_safetensors_package(tmp_path):
+	"""The on-disk format of the reference's tensors (src/tensor.rs:155-249, block_utils.py:163-199): one tensor per
+	file, dtype I8 / F8_E4M3 / BF16 / F32.  Files written by the `safetensors` package load here byte for byte,
+	files written here load there, and the reference's error cases are errors."""
+	import numpy as np
+	import torch
+	from safetensors.torch import load_file, save_file
+	rng = np.random.default_rng(5)
+	cases = {
+		X.INT8: torch.from_numpy(rng.integers(-127, 128, (6, 32), dtype=np.int8)),
+		X.E4M3: torch.from_numpy(rng.integers(0, 0x7F, (4, 16), dtype=np.uint8)).view(torch.float8_e4m3fn),
+		X.BF16: torch.from_numpy(rng.standard_normal((3, 8), dtype=np.float32)).to(torch.bfloat16),
+		X.F32: torch.from_numpy(rng.standard_normal((2, 5, 7), dtype=np.float32)),
+	}
+	for dtype, tensor in cases.items():
+		theirs = str(tmp_path / f"t{dtype}_theirs.safetensors")
+		save_file({"x_i8": tensor}, theirs, metadata={"note": "written by the package, with a metadata block"})
+		t = X.Tensor.from_safetensors_file(theirs, None)
+		assert t.dtype == dtype and t.shape == tuple(tensor.shape)
+		raw = tensor.view(torch.uint8).numpy() if dtype != X.F32 else tensor.numpy().view(np.uint8)
+		assert t.download(np.uint8 if dtype in (X.E4M3,) else None).tobytes() == raw.tobytes()
+		ours = str(tmp_path / "sub" / "dir" / f"t{dtype}_ours.safetensors")      # parent directories are created
+		t.save_safetensors_file(ours)
+		back = load_file(ours)
+		assert list(back) == ["tensor"] and back["tensor"].dtype == tensor.dtype and back["tensor"].shape == tensor.shape
+		assert back["tensor"].view(torch.uint8).numpy().tobytes() == raw.tobytes()
+	two = str(tmp_path / "two.safetensors")
+	save_file({"a": cases[X.INT8], "b": cases[X.INT8].clone()}, two)
+	with pytest.raises(X.X17Error, match="expected exactly one tensor, found 2"):
+		X.Tensor.from_safetensors_file(two, None)
+	f16 = str(tmp_path / "f16.safetensors")
+	save_file({"a": torch.zeros(4, dtype=torch.float16)}, f16)
+	with pytest.raises(X.X17Error, match="unsupported dtype F16"):
+		X.Tensor.from_safetensors_file(f16, None)
+	with pytest.raises(X.X17Error, match="cannot open"):
+		X.Tensor.from_safetensors_file(str(tmp_path / "missing.safetensors"), None)
+	junk = tmp_path / "junk.safetensors"
+	junk.write_bytes(b"\x10\x00\x00\x00\x00\x00\x00\x00not json at all!")
+	with pytest.raises(X.X17Error, match="invalid safetensors file"):
+		X.Tensor.from_safetensors_file(str(junk), None)
+
+
+def test_reference_tensor_file_conventions(tmp_path):
+	"""`<name>_<tag>.safetensors|.bin` (block_utils.py:47-124): the tag names the dtype, .bin needs a shape,
+	i8 codes are value * 8 with -128 = NaN, f8 codes decode as the kernels decode them."""
+	import numpy as np
+	import torch
+	from safetensors.torch import save_file
+	from x17ai_amd import tensor_files as TF
+	assert TF.storage_dtype_tag("tmp/block_torch/ffn_y_f8.bin") == "f8"
+	assert TF.storage_dtype_tag("attn_out_i8.safetensors") == "i8"
+	for bad in ("x.safetensors", "x_i8.npy", "_i8.bin", "x_u8.bin"):
+		with pytest.raises(X.X17Error):
+			TF.storage_dtype_tag(bad)
+	rng = np.random.default_rng(9)
+	real = rng.standard_normal((8, 16)).astype(np.float32) * 4
+	codes = np.clip(np.rint(real * 8), -127, 127).astype(np.int8)            # block_utils.py:163-166
+	codes[0, 0] = -128
+	p = str(tmp_path / "x_i8.safetensors")
+	save_file({"x": torch.from_numpy(codes)}, p)
+	t = TF.load_tensor_file(p, None)
+	assert t.dtype == X.INT8 and t.shape == (8, 16)
+	vals = TF.real_values(t.download(), t.dtype)
+	assert np.isnan(vals[0, 0]) and np.array_equal(vals.ravel()[1:], codes.ravel()[1:].astype(np.float32) / 8)
+	raw = str(tmp_path / "x_i8.bin")
+	codes.tofile(raw)
+	assert np.array_equal(TF.load_tensor_file(raw, None, (8, 16)).download(), codes)
+	with pytest.raises(X.X17Error, match="carries no shape"):
+		TF.load_tensor_file(raw, None)
+	with pytest.raises(X.X17Error, match="needs 256"):
+		TF.load_tensor_file(raw, None, (16, 16))
+	wrong = str(tmp_path / "y_f8.safetensors")
+	save_file({"y": torch.from_numpy(codes)}, wrong)
+	with pytest.raises(X.X17Error, match="declares f8"):
+		TF.load_tensor_file(wrong, None)
+	# every e4m3 code the reference's encoder emits decodes like torch's float8_e4m3fn (normal codes, zero)
+	all_codes = np.array([c for c in range(256) if (c & 0x7F) == 0 or (c & 0x78) != 0 and (c & 0x7F) != 0x7F], np.uint8)
+	want = torch.from_numpy(all_codes).view(torch.float8_e4m3fn).to(torch.float32).numpy()
+	assert np.array_equal(TF.real_values(all_codes, X.E4M3), np.abs(want) * np.where(np.signbit(want) & (want != 0), -1, 1))
+	bf = torch.from_numpy(real).to(torch.bfloat16)
+	assert np.array_equal(TF.real_values(bf.view(torch.int16).numpy().view(np.uint16), X.BF16), bf.to(torch.float32).numpy())
+
+
 def test_bench_refuses_more_than_one_gpu():
 	r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
 	assert r.returncode != 0 and "one GPU" in r.stderr

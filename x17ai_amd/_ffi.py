@@ -80,6 +80,8 @@ def host() -> ctypes.CDLL:
 	h.x17h_tensor_free.restype = None
 	h.x17h_tensor_upload.argtypes = [P, P, SZ]
 	h.x17h_tensor_download.argtypes = [P, P, SZ]
+	h.x17h_tensor_from_safetensors_file.argtypes = [P, ctypes.c_char_p, PP, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(SZ), ctypes.POINTER(SZ)]
+	h.x17h_tensor_save_safetensors_file.argtypes = [P, ctypes.c_char_p]
 	h.x17h_tensor_device_ptr.argtypes = [P]
 	h.x17h_tensor_device_ptr.restype = P
 	h.x17h_tensor_bytes.argtypes = [P]

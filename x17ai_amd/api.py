@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import ctypes
 import dataclasses
+import os
 from typing import Optional, Sequence, Union
 
 import numpy as np
@@ -70,6 +71,29 @@ class Tensor:
 		t = cls(device, array.shape, dtype)
 		t.upload(array)
 		return t
+
+	@classmethod
+	def from_safetensors_file(cls, path: str, device: Optional[Device]) -> "Tensor":
+		"""Tensor::from_safetensors_file, src/tensor.rs:155-179 (what the reference's block_utils.store_tensor
+		writes for `*_i8 / _f8 / _bf16 / _f32.safetensors`): exactly one tensor, bytes uploaded unchanged."""
+		t = cls.__new__(cls)
+		t.device = device
+		t._h = ctypes.c_void_p()
+		dtype, ndim = ctypes.c_int(), ctypes.c_size_t()
+		shape = (ctypes.c_size_t * 8)()
+		check(_ffi.host().x17h_tensor_from_safetensors_file(device._h if device is not None else None, os.fsencode(path),
+		                                                    ctypes.byref(t._h), ctypes.byref(dtype), shape, ctypes.byref(ndim)))
+		t.dtype = dtype.value
+		t.shape = tuple(int(shape[i]) for i in range(ndim.value))
+		return t
+
+	def save_safetensors_file(self, path: str) -> None:
+		"""Tensor::save_safetensors_file, src/tensor.rs:213-249: CPU tensors only (download first)."""
+		check(_ffi.host().x17h_tensor_save_safetensors_file(self._h, os.fsencode(path)))
+
+	def to_cpu(self) -> "Tensor":
+		"""Tensor::to_cpu + synchronize, src/tensor.rs:98-112."""
+		return Tensor.from_numpy(None, self.download(), self.dtype)
 
 	@property
 	def nbytes(self) -> int:

@@ -3,6 +3,7 @@
 // (include/x17ai_host.h).
 
 #include "x17ai_host.hpp"
+#include <filesystem>
 #include "../../../include/x17ai_host.h"
 
 #include <dlfcn.h>
@@ -226,6 +227,167 @@ Result<std::shared_ptr<Tensor>> Tensor::new_empty(std::vector<size_t> shape, DTy
 	t->bytes = bytes;
 	t->device = std::move(device);
 	return R::ok(std::move(t));
+}
+
+// ---- safetensors: u64 little-endian header length, a JSON header {name: {dtype, shape, data_offsets}, ...,
+// "__metadata__": {...}}, then the tensor bytes.  The header parser below reads just that shape of JSON.
+namespace {
+struct StEntry { std::string name, dtype; std::vector<size_t> shape; size_t begin = 0, end = 0; };
+
+struct StParser {
+	std::string const &s;
+	size_t i = 0;
+	explicit StParser(std::string const &text): s(text) {}
+	void ws() { while (i < s.size() && (s[i] == ' ' || s[i] == '\n' || s[i] == '\t' || s[i] == '\r')) ++i; }
+	bool eat(char c) { ws(); if (i < s.size() && s[i] == c) { ++i; return true; } return false; }
+	bool string(std::string &out) {
+		ws();
+		if (i >= s.size() || s[i] != '"') return false;
+		++i;
+		out.clear();
+		while (i < s.size() && s[i] != '"') {
+			if (s[i] == '\\' && i + 1 < s.size()) { ++i; }
+			out.push_back(s[i++]);
+		}
+		return i < s.size() && s[i++] == '"';
+	}
+	bool number(size_t &out) {
+		ws();
+		if (i >= s.size() || s[i] < '0' || s[i] > '9') return false;
+		out = 0;
+		while (i < s.size() && s[i] >= '0' && s[i] <= '9') out = out * 10 + size_t(s[i++] - '0');
+		return true;
+	}
+	bool numbers(std::vector<size_t> &out) {
+		if (!eat('[')) return false;
+		out.clear();
+		if (eat(']')) return true;
+		do { size_t v; if (!number(v)) return false; out.push_back(v); } while (eat(','));
+		return eat(']');
+	}
+	// skips any JSON value (used for "__metadata__" and unknown keys)
+	bool skip() {
+		ws();
+		if (i >= s.size()) return false;
+		if (s[i] == '"') { std::string t; return string(t); }
+		if (s[i] == '{' || s[i] == '[') {
+			char open = s[i], close = open == '{' ? '}' : ']';
+			++i;
+			if (eat(close)) return true;
+			do {
+				if (open == '{') { std::string k; if (!string(k) || !eat(':')) return false; }
+				if (!skip()) return false;
+			} while (eat(','));
+			return eat(close);
+		}
+		while (i < s.size() && s[i] != ',' && s[i] != '}' && s[i] != ']') ++i;
+		return true;
+	}
+	bool entry(StEntry &e) {
+		if (!eat('{')) return false;
+		do {
+			std::string key;
+			if (!string(key) || !eat(':')) return false;
+			if (key == "dtype") { if (!string(e.dtype)) return false; }
+			else if (key == "shape") { if (!numbers(e.shape)) return false; }
+			else if (key == "data_offsets") {
+				std::vector<size_t> o;
+				if (!numbers(o) || o.size() != 2) return false;
+				e.begin = o[0]; e.end = o[1];
+			} else if (!skip()) return false;
+		} while (eat(','));
+		return eat('}');
+	}
+	bool header(std::vector<StEntry> &out) {
+		if (!eat('{')) return false;
+		if (eat('}')) return true;
+		do {
+			std::string name;
+			if (!string(name) || !eat(':')) return false;
+			if (name == "__metadata__") { if (!skip()) return false; continue; }
+			StEntry e;
+			e.name = name;
+			if (!entry(e)) return false;
+			out.push_back(std::move(e));
+		} while (eat(','));
+		return eat('}');
+	}
+};
+
+char const *st_dtype_name(DType d) {      // src/dtype.rs:26-36
+	switch (d) {
+		case DType::E4m3: return "F8_E4M3";
+		case DType::Int8: return "I8";
+		case DType::Bf16: return "BF16";
+		case DType::F32: return "F32";
+	}
+	return "?";
+}
+} // namespace
+
+Result<std::shared_ptr<Tensor>> Tensor::from_safetensors_file(std::string const &path, std::shared_ptr<Device> device) {
+	using R = Result<std::shared_ptr<Tensor>>;
+	auto bad = [&](std::string const &why) { return R::err(ErrPack{TensorOpError::Io, "invalid safetensors file " + path + ": " + why, nullptr}); };
+	std::ifstream f(path, std::ios::binary);
+	if (!f) return R::err(ErrPack{TensorOpError::Io, "cannot open " + path, nullptr});
+	unsigned char len8[8];
+	if (!f.read(reinterpret_cast<char *>(len8), 8)) return bad("shorter than its length field");
+	uint64_t n = 0;
+	for (int b = 7; b >= 0; --b) n = (n << 8) | len8[b];
+	if (n > (uint64_t(1) << 27)) return bad("header length " + std::to_string(n));
+	std::string header(size_t(n), '\0');
+	if (!f.read(header.data(), std::streamsize(n))) return bad("truncated header");
+	std::vector<StEntry> entries;
+	StParser p(header);
+	if (!p.header(entries)) return bad("header is not the expected JSON");
+	if (entries.size() != 1) return bad("expected exactly one tensor, found " + std::to_string(entries.size()));   // tensor.rs:164-177
+	StEntry const &e = entries[0];
+	DType dtype;
+	if (e.dtype == "F8_E4M3") dtype = DType::E4m3;
+	else if (e.dtype == "I8") dtype = DType::Int8;
+	else if (e.dtype == "BF16") dtype = DType::Bf16;
+	else if (e.dtype == "F32") dtype = DType::F32;
+	else return R::err(ErrPack{TensorOpError::Other, "unsupported dtype " + e.dtype + " in " + path, nullptr});   // dtype.rs:38-50
+	auto t = Tensor::new_empty(e.shape, dtype, std::move(device));
+	if (!t.is_ok()) return t;
+	if (e.end < e.begin || e.end - e.begin != (*t.value)->bytes) return bad("data_offsets do not match dtype and shape");
+	std::vector<char> data((*t.value)->bytes);
+	f.seekg(std::streamoff(8 + n + e.begin));
+	if (!data.empty() && !f.read(data.data(), std::streamsize(data.size()))) return bad("truncated tensor data");
+	Status up = (*t.value)->device->upload_data(reinterpret_cast<uint8_t const *>(data.data()), (*t.value)->ptr, data.size());
+	if (!up.is_ok()) return R::err(*up.error);
+	// the staging buffer dies here: make sure an asynchronous copy has consumed it
+	if (auto *hip = dynamic_cast<HipDevice *>((*t.value)->device.get())) {
+		Status sy = hip->synchronize();
+		if (!sy.is_ok()) return R::err(*sy.error);
+	}
+	return t;
+}
+
+Status Tensor::save_safetensors_file(std::string const &path) const {
+	if (!device || !device->is_cpu()) {
+		return Status::err(TensorOpError::Device, "save_safetensors_file requires a CPU tensor; download it first");   // tensor.rs:230-235
+	}
+	std::error_code ec;
+	std::filesystem::path fp(path);
+	if (fp.has_parent_path()) {
+		std::filesystem::create_directories(fp.parent_path(), ec);
+		if (ec) return Status::err(TensorOpError::Io, "failed to create tensor output directory " + fp.parent_path().string() + ": " + ec.message());
+	}
+	std::string header = "{\"tensor\":{\"dtype\":\"" + std::string(st_dtype_name(dtype)) + "\",\"shape\":[";
+	for (size_t i = 0; i < shape.size(); ++i) header += (i ? "," : "") + std::to_string(shape[i]);
+	header += "],\"data_offsets\":[0," + std::to_string(bytes) + "]}}";
+	while (header.size() % 8 != 0) header.push_back(' ');          // the format pads the header to 8 bytes with spaces
+	std::ofstream f(path, std::ios::binary | std::ios::trunc);
+	if (!f) return Status::err(TensorOpError::Io, "cannot create " + path);
+	uint64_t n = header.size();
+	unsigned char len8[8];
+	for (int b = 0; b < 8; ++b) len8[b] = (unsigned char)(n >> (8 * b));
+	f.write(reinterpret_cast<char const *>(len8), 8);
+	f.write(header.data(), std::streamsize(header.size()));
+	if (bytes != 0) f.write(static_cast<char const *>(ptr), std::streamsize(bytes));
+	if (!f) return Status::err(TensorOpError::Io, "failed to write " + path);
+	return Status::ok();
 }
 
 Tensor::~Tensor() {
@@ -1074,6 +1236,25 @@ int x17h_tensor_upload(X17hTensor *t, void const *src, size_t bytes) {
 int x17h_tensor_download(X17hTensor *t, void *dst, size_t bytes) {
 	if (bytes != t->t->bytes) return fail("download size " + std::to_string(bytes) + " does not match tensor size " + std::to_string(t->t->bytes));
 	return from_status(t->t->device->download_data(t->t->ptr, static_cast<uint8_t *>(dst), bytes));
+}
+int x17h_tensor_from_safetensors_file(X17hDevice *dev, char const *path, X17hTensor **out, int *dtype, size_t *shape, size_t *ndim) {
+	try {
+		std::shared_ptr<Device> device;
+		if (dev != nullptr) device = dev->dev; else device = std::make_shared<CpuDevice>();
+		auto r = Tensor::from_safetensors_file(path, device);
+		if (!r.is_ok()) return fail(*r.error);
+		if ((*r.value)->shape.size() > 8) return fail("tensors of more than 8 dimensions are not supported here");
+		*dtype = int((*r.value)->dtype);
+		*ndim = (*r.value)->shape.size();
+		for (size_t i = 0; i < *ndim; ++i) shape[i] = (*r.value)->shape[i];
+		*out = new X17hTensor{*r.value};
+		return 0;
+	} catch (std::exception const &e) { return fail(e.what()); }
+}
+int x17h_tensor_save_safetensors_file(X17hTensor *t, char const *path) {
+	try {
+		return from_status(t->t->save_safetensors_file(path));
+	} catch (std::exception const &e) { return fail(e.what()); }
 }
 void *x17h_tensor_device_ptr(X17hTensor *t) { return t->t->ptr; }
 size_t x17h_tensor_bytes(X17hTensor *t) { return t->t->bytes; }

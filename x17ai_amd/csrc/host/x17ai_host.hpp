@@ -158,6 +158,11 @@ struct Tensor {
 	std::shared_ptr<Device> device;
 
 	static Result<std::shared_ptr<Tensor>> new_empty(std::vector<size_t> shape, DType dtype, std::shared_ptr<Device> device);
+	// src/tensor.rs:155-179 -- a safetensors file holding exactly one tensor of dtype F8_E4M3 / I8 / BF16 / F32;
+	// the bytes are uploaded as they are (int8 and e4m3 tensors are codes).
+	static Result<std::shared_ptr<Tensor>> from_safetensors_file(std::string const &path, std::shared_ptr<Device> device);
+	// src/tensor.rs:213-249 -- CPU tensors only; written as the single entry "tensor"; parent directories are created.
+	Status save_safetensors_file(std::string const &path) const;
 	~Tensor();
 	size_t elems() const;
 	bool is_on_device(Device const *d) const { return device.get() == d; }   // pointer identity, tensor.rs:87-91
