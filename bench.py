@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] [--only KERNEL] [--copy-probe]
 
-Headline (the JSON line's `value`): BASELINE config 2, the int8 FFN GEMM pair
+Headline (the JSON line's `value`): benchmark config 2, the int8 FFN GEMM pair
   ffn_f_fwd   x[8192, 2048] i8 . W1[16384, 2048]^T  -> GeGLU   -> f[8192, 8192] FixedI8
   ffn_y_fwd   f[8192, 8192] i8 . W2[4096, 8192]^T   -> gated residual with x -> y[8192, 2048] e4m3
 One step = both launches over the 8192-token batch; inputs are resident in HBM before the timed
@@ -13,7 +13,7 @@ region.  value = (2*M*K*N_raw of both GEMMs) * steps / wall time, in TOPS.
 its mean launch duration, measured with HIP events on the launching stream inside the timed
 region, against the MI355X dense int8 MFMA peak.  `cpu_baseline` is the CPU oracle (a port of the
 reference's arithmetic) timed on a bounded row sample of the same workload on the host cores.
-`extras` reports the other BASELINE configurations (fp8 FFN, block forward, attention prefill,
+`extras` reports the other benchmark configurations (fp8 FFN, block forward, attention prefill,
 decode, rms_norm), each as median-of-launches, next to the roofline that bounds it.
 """
 from __future__ import annotations
@@ -289,7 +289,7 @@ def extras(dev, X, recipes):
 
 
 def single(dev, X, recipes, name, iters):
-	"""One kernel of one BASELINE workload, launched `iters` times: what the rocprofv3 summaries under
+	"""One kernel of one benchmark workload, launched `iters` times: what the rocprofv3 summaries under
 	profiles/ are taken from (every code object exports the entry `kernel`, so a profile of several
 	kernels at once cannot tell them apart by name)."""
 	rng = np.random.default_rng(3000)
@@ -388,7 +388,7 @@ def main():
 	value = h["ops_per_step"] * args.steps / h["wall_s"] / 1e12
 	achieved = h["k1_ops"] / h["k1_mean_s"] / 1e12
 	line = {
-		"metric": "int8 FFN GEMM pair throughput (ffn_f_fwd + ffn_y_fwd_i8, BASELINE config 2)",
+		"metric": "int8 TOPS at 1 MI355X (config 2: FFN GEMM pair ffn_f_fwd + ffn_y_fwd_i8); fp8 TOPS, block-fwd tokens/sec and % of MFMA/HBM roofline under extras",
 		"value": value, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
 		"ms_per_step": h["wall_s"] / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
 		"vs_baseline": None, "dtype": "int8", "data": "synthetic",

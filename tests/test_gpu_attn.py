@@ -50,7 +50,7 @@ def _run_attn(dev, kern, q, kv, sink_k, sink_v, temp, window, batch=1, want_l=Tr
 # (T, H, hd, window)
 CASES = [
 	(256, 4, 32, 0), (256, 4, 32, 64), (384, 2, 64, 0), (512, 2, 64, 128), (512, 2, 64, 16),
-	(384, 2, 128, 0), (640, 2, 128, 256), (1024, 8, 64, 256),          # the last one is BASELINE config 1
+	(384, 2, 128, 0), (640, 2, 128, 256), (1024, 8, 64, 256),          # the last one is benchmark config 1
 ]
 
 

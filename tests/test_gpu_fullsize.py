@@ -1,4 +1,4 @@
-"""GPU parity at the full BASELINE sizes.
+"""GPU parity at the full benchmark sizes.
 
 The CPU oracle cannot redo these workloads whole in test time, so each check uses a property that does
 not depend on the size: a GEMM output row depends only on its own token row and the weights, an attention
@@ -37,7 +37,7 @@ def _sample_rows(rng, m, count):
 
 
 def test_config2_ffn_pair_sampled_rows(dev):
-	"""BASELINE config 2: tokens 8192, d_model 2048, d_ff 8192 -- ffn_f (GeGLU -> FixedI8) and the int8
+	"""benchmark config 2: tokens 8192, d_model 2048, d_ff 8192 -- ffn_f (GeGLU -> FixedI8) and the int8
 	ffn_y (gated residual -> e4m3), strict builds, 96 sampled token rows of each against the oracle."""
 	m, d, f = 8192, 2048, 8192
 	rng = rng_for("full-config2")
@@ -61,7 +61,7 @@ def test_config2_ffn_pair_sampled_rows(dev):
 
 
 def test_config2_literal_per_token_per_channel_scales(dev):
-	"""BASELINE config 2 as worded: x ~ N(0,1) per-token int8 (absmax / 127), W1 [2048 x 8192 (x2 gated)] and
+	"""benchmark config 2 as worded: x ~ N(0,1) per-token int8 (absmax / 127), W1 [2048 x 8192 (x2 gated)] and
 	W2 [8192 x 2048] ~ N(0, 1/sqrt(fan_in)) per-output-channel int8, int32 accumulate, fused dequantisation +
 	GeGLU, bf16 out; the bf16 activations are re-quantised per token for the second GEMM.  Sampled rows
 	against the oracle, bit for bit, and the whole against the float64 computation it approximates."""
@@ -137,7 +137,7 @@ def _head_columns(arr, heads, width):
 
 
 def test_config4_attention_sampled_heads(dev):
-	"""BASELINE config 4 attention: 4 sequences x 8192 tokens, 16 heads x 128, window 512.  Heads are
+	"""benchmark config 4 attention: 4 sequences x 8192 tokens, 16 heads x 128, window 512.  Heads are
 	independent, so three heads of two of the sequences are recomputed by the oracle (all 8192 queries)."""
 	t, b, h, hd, w = 8192, 4, 16, 128, 512
 	rng = rng_for("full-config4-attn")
@@ -158,7 +158,7 @@ def test_config4_attention_sampled_heads(dev):
 
 
 def test_config5_prefill_sampled_heads(dev):
-	"""BASELINE config 5 prefill: one sequence of 65536 tokens, 32 heads x 128, window 4096; two heads
+	"""benchmark config 5 prefill: one sequence of 65536 tokens, 32 heads x 128, window 4096; two heads
 	recomputed by the oracle.  Also the speed build against the strict one over the whole output."""
 	t, h, hd, w = 65536, 32, 128, 4096
 	rng = rng_for("full-config5-attn")
@@ -181,7 +181,7 @@ def test_config5_prefill_sampled_heads(dev):
 
 
 def test_config5_decode_sampled_sequences(dev):
-	"""BASELINE config 5 decode: 64 sequences against 4096 cached positions, 32 heads x 128.  Ragged
+	"""benchmark config 5 decode: 64 sequences against 4096 cached positions, 32 heads x 128.  Ragged
 	lengths (0, 1, 15, 16, 17, ..., 4096); four heads of every sequence recomputed by the oracle."""
 	s, cap, h, hd, w = 64, 4096, 32, 128, 4096
 	rng = rng_for("full-config5-decode")

@@ -16,7 +16,7 @@
 //   GemmKernel<Epilogue> & co.     src/device/cuda/gemm.rs:28-918
 //   AttnKernel & co.               src/device/cuda/attn.rs:45-448
 //   RmsNormKernel                  rms_norm.cu:55-113 given the same kernel-object shape
-//   AttnDecodeKernel               no reference counterpart (single-token decode, see DESIGN)
+//   AttnDecodeKernel               no reference counterpart (single-token decode, defined in attn_decode_i8.hip)
 #pragma once
 
 #include <cstddef>

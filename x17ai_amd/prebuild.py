@@ -72,7 +72,7 @@ def _specs():
 		add(("dequant", 1024, 512, INT8, INT8, False, strict))
 		add(("dequant", 1024, 512, INT8, INT8, True, strict))
 	add(("dequant", 512, 256, E4M3, E4M3, False, True))
-	# ---- tests/test_gpu_fullsize.py: BASELINE config 2 in its literal form (per-token / per-channel scales)
+	# ---- tests/test_gpu_fullsize.py: benchmark config 2 in its literal form (per-token / per-channel scales)
 	for strict in (True, False):                             # the speed builds are bench.py's
 		add(("dequant", 2048, 16384, INT8, INT8, True, strict))
 		add(("dequant", 8192, 2048, INT8, INT8, False, strict))
