@@ -137,14 +137,25 @@ void kernel(
 			block_max = __builtin_fmaxf(block_max, mx);
 		}
 	}
-	s_bmax[tid] = block_max;
-	__syncthreads();
-
-	// ---- phase 2b: running max before each thread's tiles (max is exact, so any grouping works),
-	// then running max and rescale factor of every tile (cuda/attn_fwd_i8.cuh:233-256)
+	// ---- phase 2b: running max before each thread's tiles (max is exact, so any grouping works): an
+	// exclusive prefix maximum over the threads -- a shuffle scan inside each wavefront, the wavefront totals
+	// through LDS -- then running max and rescale factor of every tile (cuda/attn_fwd_i8.cuh:233-256)
+	f32 m_before;
 	{
-		f32 m_prev = m0;
-		for (u32 t = 0; t < tid; ++t) m_prev = __builtin_fmaxf(m_prev, s_bmax[t]);
+		u32 const lane = tid % 64;
+		f32 incl = block_max;
+		X17_UNROLL for (int d = 1; d < 64; d <<= 1) {
+			f32 up = __shfl_up(incl, d, 64);
+			if ((int)lane >= d) incl = __builtin_fmaxf(incl, up);
+		}
+		if (lane == 63) s_bmax[tid / 64] = incl;                  // this wavefront's maximum
+		f32 excl = __shfl_up(incl, 1, 64);
+		m_before = lane == 0 ? -__builtin_inff() : excl;
+	}
+	__syncthreads();
+	{
+		f32 m_prev = __builtin_fmaxf(m0, m_before);
+		for (u32 w = 0; w < tid / 64; ++w) m_prev = __builtin_fmaxf(m_prev, s_bmax[w]);
 		X17_UNROLL for (u32 i = 0; i < TPT; ++i) {
 			u32 t = tid * TPT + i;
 			if (t < n_tiles) {
