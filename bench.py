@@ -251,6 +251,17 @@ def extras(dev, X, recipes):
 	p1 = W1 * (W1 - 1) // 2 + (T1 - W1) * W1
 	out["config1_attn"] = {"median_us": med * 1e6, "gops": 4.0 * HD1 * H1 * p1 / 1e9, "tops": 4.0 * HD1 * H1 * p1 / med / 1e12}
 
+	# the same shape as the configuration words it: one absmax / 127 scale per (row, head) of q, k and v, bf16 output
+	def row_scale_tensors(rows, heads):
+		scales = [(0.02 * (0.5 + rng.random((rows, heads)))).astype(np.float32) for _ in range(3)]
+		vw, sw, osc = recipes.attn_row_scale_operands(scales[2], X.BF16)
+		return [X.Tensor.from_numpy(dev, np.ascontiguousarray(a, dtype=np.float32), X.F32) for a in (scales[0], scales[1], vw, sw, osc)]
+	rs1 = row_scale_tensors(T1, H1)
+	ob1 = X.Tensor(dev, (T1, H1 * HD1), X.BF16)
+	k1r = recipes.attn_row_scaled_kernel(dev, H1, HD1, X.BF16, False)
+	med, _ = _median_launch(dev, X, lambda: k1r.launch_row_scaled(q1, kv1, sk1, sv1, tp1, ob1, None, W1, *rs1), 20, 5)
+	out["config1_attn_row_scaled_bf16"] = {"median_us": med * 1e6, "tops": 4.0 * HD1 * H1 * p1 / med / 1e12}
+
 	# ---- config 5: prefill T=65536, H=32, hd=128, W=4096; decode 64 sequences x 4096 cached positions
 	T5, H5, HD5, W5 = 65536, 32, 128, 4096
 	q5 = X.Tensor.from_numpy(dev, _rand_codes(rng, (T5, H5 * HD5)), X.INT8)
@@ -268,7 +279,13 @@ def extras(dev, X, recipes):
 		c5[f"prefill_{tag}_ms"] = med * 1e3
 		c5[f"prefill_{tag}_tops"] = 4.0 * HD5 * H5 * p5 / med / 1e12
 		c5[f"prefill_{tag}_frac_of_int8_peak"] = c5[f"prefill_{tag}_tops"] / PEAK_INT8_TOPS
-	del q5, kv5, o5
+	rs5 = row_scale_tensors(T5, H5)
+	ob5 = X.Tensor(dev, (T5, H5 * HD5), X.BF16)
+	k5r = recipes.attn_row_scaled_kernel(dev, H5, HD5, X.BF16, False)
+	med, _ = _median_launch(dev, X, lambda: k5r.launch_row_scaled(q5, kv5, sk5, sv5, tp5, ob5, None, W5, *rs5), 3, 1)
+	c5["prefill_row_scaled_bf16_ms"] = med * 1e3
+	c5["prefill_row_scaled_bf16_tops"] = 4.0 * HD5 * H5 * p5 / med / 1e12
+	del q5, kv5, o5, ob5, rs5
 	S5, CAP = 64, 4096
 	one = _rand_codes(rng, (1, CAP, 2 * H5 * HD5))
 	cache = X.Tensor.from_numpy(dev, np.ascontiguousarray(np.broadcast_to(one, (S5, CAP, 2 * H5 * HD5))), X.INT8)

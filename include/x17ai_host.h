@@ -109,6 +109,10 @@ int x17h_gemm_kernel_attrs(X17hGemmKernel *k, int32_t out[9]);
 typedef struct X17hAttnConfig {
 	int dtype; size_t n_heads; size_t head_dim; size_t q_stride; size_t kv_stride; size_t o_stride;
 	int strict_math;
+	/* extension, no counterpart in the reference (its codes all share the scale 1/8): row_scales != 0 builds
+	 * the kernel whose q/k/v codes carry one f32 scale per (row, head); out_dtype is then X17H_INT8
+	 * (FixedI8 codes) or X17H_BF16 (real values), otherwise X17H_INT8 */
+	int row_scales; int out_dtype;
 } X17hAttnConfig;
 /* AttnKernel::new, attn.rs:170-232 */
 int x17h_attn_kernel_new(X17hDevice *dev, char const *kernel_name, X17hAttnConfig const *config, X17hAttnKernel **out);
@@ -118,6 +122,15 @@ void x17h_attn_kernel_free(X17hAttnKernel *k);
 int x17h_attn_kernel_launch(X17hAttnKernel *k, X17hTensor *q, X17hTensor *kv, X17hTensor *sink_k,
                             X17hTensor *sink_v, X17hTensor *attn_temperature, X17hTensor *out,
                             X17hTensor *l, size_t window_size, size_t batch);
+/* The same launch for a kernel built with row_scales (no counterpart in the reference; the closest
+ * precedent is the per-head temperature vector of attn.rs:421-437).  q_scale, k_scale, v_weight: f32
+ * [rows, n_heads]; sink_v_weight, out_scale: f32 [n_heads].  Real q = code * q_scale, real k = code * k_scale,
+ * real v = code * v_weight * v_ref[h]; sink_v_weight = (1/8) / v_ref, out_scale = v_ref (bf16 out) or 8 * v_ref. */
+int x17h_attn_kernel_launch_row_scaled(X17hAttnKernel *k, X17hTensor *q, X17hTensor *kv, X17hTensor *sink_k,
+                                       X17hTensor *sink_v, X17hTensor *attn_temperature, X17hTensor *out,
+                                       X17hTensor *l, size_t window_size, size_t batch,
+                                       X17hTensor *q_scale, X17hTensor *k_scale, X17hTensor *v_weight,
+                                       X17hTensor *sink_v_weight, X17hTensor *out_scale);
 /* AttnKernelConfig::n_ops, attn.rs:72-84 */
 double x17h_attn_kernel_n_ops(X17hAttnKernel *k, size_t seq_len, size_t window_size);
 int x17h_attn_kernel_metadata(X17hAttnKernel *k, size_t out[3]);

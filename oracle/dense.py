@@ -144,6 +144,49 @@ def attn_one_head(q, k, v, sink_k, sink_v, temperature_scale: float, window: int
 	return o, l
 
 
+def quantize_rows(a: np.ndarray):
+	"""Symmetric int8 quantisation of the last axis: scale = absmax / 127 (1 for an all-zero row),
+	codes = rint(a / scale).  Returns (codes int8, scale float32 without the last axis)."""
+	absmax = np.abs(a).max(axis=-1)
+	scale = np.where(absmax > 0, absmax / 127.0, 1.0).astype(np.float32)
+	codes = np.clip(np.rint(a / scale[..., None].astype(np.float64)), -127, 127).astype(np.int8)
+	return codes, scale
+
+
+def attn_one_head_row_scaled(q_codes, k_codes, v_codes, q_scale, k_scale, v_scale, sink_k, sink_v,
+                             temperature_scale: float, window: int, quantize_p: bool = True):
+	"""The dense softmax of attn_one_head over operands given as int8 codes with one scale per row
+	(real value = code * scale); sink_k, sink_v are real values.  With quantize_p the probability of
+	key j enters the numerator as rint(255 p_j w_j) / (255 w_j), w_j = v_scale[j] / max(v_scale), which
+	models u8 probabilities that carry the value row's relative scale; without it the softmax is exact.
+	Returns o [T, hd] (real values)."""
+	t, hd = q_codes.shape
+	q = q_codes.astype(np.float64) * np.asarray(q_scale, dtype=np.float64)[:, None]
+	k = k_codes.astype(np.float64) * np.asarray(k_scale, dtype=np.float64)[:, None]
+	v_scale = np.asarray(v_scale, dtype=np.float32)
+	v_ref = np.float32(v_scale.max())
+	w = (v_scale / v_ref).astype(np.float64)                        # float32 quotient, as a caller would form it
+	k = np.concatenate((sink_k[None, :], k), axis=0)
+	temperature = math.sqrt(1.0 / hd) * np.log(ssmax_n(t, window)) * temperature_scale
+	s = q @ k.T
+	rows = np.arange(t)[:, None]
+	cols = np.arange(t)[None, :]
+	real_mask = cols >= rows
+	if window > 0:
+		real_mask |= cols < rows - window
+	mask = np.zeros((t, t + 1), dtype=bool)
+	mask[:, 1:] = real_mask
+	s = np.where(mask, -np.inf, s) * temperature
+	p = np.exp(s - s.max(axis=1, keepdims=True))
+	total = p.sum(axis=1, keepdims=True)
+	if quantize_p:
+		pk = np.rint(p[:, 1:] * 255.0 * w[None, :]) * (float(v_ref) / 255.0)
+		num = pk @ v_codes.astype(np.float64)
+	else:
+		num = p[:, 1:] @ (v_codes.astype(np.float64) * v_scale.astype(np.float64)[:, None])
+	return (p[:, :1] * sink_v[None, :] + num) / total
+
+
 def attn(q, k, v, sinks_k, sinks_v, attn_temperature, window: int, prob_steps: float = 8.0):
 	"""new_block.py:234-258.  q, k, v: [T, H, hd]; sinks [H, hd]; attn_temperature [H]."""
 	outs, ls = [], []

@@ -224,6 +224,32 @@ def attn_fwd_i8(q, kv, sink_k, sink_v, head_temp, n_heads: int, head_dim: int, w
 	return out, l
 
 
+def attn_fwd_i8_row_scaled(q, kv, sink_k, sink_v, head_temp, n_heads: int, head_dim: int, window: int,
+                           q_scale, k_scale, v_weight, sink_v_weight, out_scale, out_bf16: bool = False,
+                           want_l: bool = True, fast_exp: bool = False):
+	"""attn_fwd_i8 over row-scaled operands: q_scale, k_scale, v_weight float32 [T, H]; sink_v_weight,
+	out_scale float32 [H].  Returns (out, L): out int8 codes, or bf16 bit patterns (uint16) with out_bf16."""
+	q = np.ascontiguousarray(q, dtype=np.int8)
+	kv = np.ascontiguousarray(kv, dtype=np.int8)
+	sink_k = np.ascontiguousarray(sink_k, dtype=np.int8)
+	sink_v = np.ascontiguousarray(sink_v, dtype=np.int8)
+	head_temp = np.ascontiguousarray(head_temp, dtype=np.float32).reshape(-1)
+	t = q.shape[0]
+	assert q.shape == (t, n_heads * head_dim) and kv.shape == (t, 2 * n_heads * head_dim)
+	assert sink_k.shape == (n_heads, head_dim) and sink_v.shape == (n_heads, head_dim)
+	rows = [np.ascontiguousarray(a, dtype=np.float32) for a in (q_scale, k_scale, v_weight)]
+	heads = [np.ascontiguousarray(a, dtype=np.float32).reshape(-1) for a in (sink_v_weight, out_scale)]
+	assert all(a.shape == (t, n_heads) for a in rows) and all(a.shape == (n_heads,) for a in heads)
+	out = np.empty(q.shape, dtype=np.uint16 if out_bf16 else np.int8)
+	l = np.empty((n_heads, t), dtype=np.float32) if want_l else None
+	rc = lib().x17o_attn_fwd_i8_row_scaled(_sz(t), _sz(n_heads), _sz(head_dim), _p(q), _p(kv), _p(sink_k), _p(sink_v),
+	                                       _p(head_temp), _p(out), _p(l) if want_l else None, _sz(window),
+	                                       ctypes.c_int(int(fast_exp)), _p(rows[0]), _p(rows[1]), _p(rows[2]),
+	                                       _p(heads[0]), _p(heads[1]), ctypes.c_int(int(out_bf16)))
+	assert rc == 0
+	return out, l
+
+
 def attn_decode_i8(q, cache, cache_len, sink_k, sink_v, head_temp, n_heads: int, head_dim: int,
                    window: int, want_l: bool = True, fast_exp: bool = False):
 	"""q [S, H*hd], cache [S, cap, H*2*hd], cache_len uint32 [S] -> (out [S, H*hd], L [S, H])."""

@@ -26,6 +26,8 @@
  *   gemm_i32         numpy int64 matmul
  *   epilogues        closed-form float64 formulas of the reference's torch oracle
  *   attention/decode dense float64 softmax restatement, closed-form special cases
+ *   row-scaled attention  bit-identity with the reference mode at scales 1/8, dense float64 softmax
+ *                    over the dequantised operands, invariance under power-of-two rescalings
  *   rms_norm         textbook float64 RMS norm + the reference's legacy known-answer
  * The float32 GEMM (gemm_f32_seq) is pinned against float64 matmul to a stated
  * tolerance only: its summation order is a definition of this file, the
@@ -427,15 +429,36 @@ X17_EXPORT void x17o_epilogue_l2norm(const int32_t *acc, int8_t *C, float *rrms,
  * out [T, H*hd], L [H, T] (may be NULL).  `pos0` is the absolute position of row 0 of
  * q relative to row 0 of kv (0 for prefill; used by the decode entry below).
  * `fast_exp` != 0 replaces sfu_ex2 by exp2f so that the tests can bound how far a
- * hardware-exponent build may drift from the strict definition. */
+ * hardware-exponent build may drift from the strict definition.
+ *
+ * Row-scaled operands (`rs` != NULL; no counterpart in the reference, whose q/k/v are FixedI8 codes
+ * with the one constant scale 1/8).  Real values are q_code * q_scale[row, h], k_code * k_scale[row, h],
+ * v_code * v_scale[row, h]; the caller passes v_weight = v_scale / v_ref[h] (<= 1),
+ * sink_v_weight[h] = (1/8) / v_ref[h] and out_scale[h] = v_ref[h] * (8 for a FixedI8 output, 1 for bf16).
+ * The recurrence is the one above with
+ *   tq  = ((f32(hd^-1/2) * lg2(n)) * head_temp[h]) * q_scale[i, h]
+ *   s_j = (f32(q_i . k_j) * k_scale[j, h]) * tq,   sink score = f32(q_i . sink_k) * (tq * 0.125)
+ *   P_j = rne(p_j * v_weight[j, h]) (the partial sums still add the unweighted p_j)
+ *   O starts at f32(255 * sink_v) * sink_v_weight[h];   out = store((O * rcp(sum)) * out_scale[h])
+ * so that with every scale 1/8 and every weight and out_scale 1 each step produces the bits of the
+ * reference mode (multiplications by powers of two commute with rounding). */
+typedef struct {
+	const float *q_scale;        /* [n_q, H] */
+	const float *k_scale;        /* [kv rows, H] */
+	const float *v_weight;       /* [kv rows, H] */
+	const float *sink_v_weight;  /* [H] */
+	const float *out_scale;      /* [H] */
+	int out_bf16;                /* 0: FixedI8 bytes, 1: bf16 (out is then uint16_t*, o_stride in elements) */
+} RowScales;
+
 static void attn_rows(size_t n_q, size_t pos0, size_t H, size_t hd,
                       const int8_t *q, size_t q_stride,
                       const int8_t *kv, size_t kv_stride,
                       const int8_t *sink_k, const int8_t *sink_v, const float *head_temp,
                       int8_t *out, size_t o_stride, float *L, size_t l_stride,
-                      size_t window, int fast_exp) {
+                      size_t window, int fast_exp, const RowScales *rs) {
 	size_t Wr = window == 0 ? (size_t)-1 : ((window - 1) / 16 + 1) * 16;
-	float base = (float)(constexpr_inv_sqrt((double)hd) / 64.0);
+	float base = rs ? (float)constexpr_inv_sqrt((double)hd) : (float)(constexpr_inv_sqrt((double)hd) / 64.0);
 	#pragma omp parallel for collapse(2) schedule(dynamic, 8)
 	for (size_t h = 0; h < H; ++h) {
 		for (size_t r = 0; r < n_q; ++r) {
@@ -447,12 +470,16 @@ static void attn_rows(size_t n_q, size_t pos0, size_t H, size_t hd,
 			uint32_t n = (uint32_t)visible + 4u;
 			float temp = base * sfu_lg2((float)n);
 			temp = temp * head_temp[h];
+			if (rs) temp = temp * rs->q_scale[r * H + h];
 			int32_t sdot = 0;
 			for (size_t d = 0; d < hd; ++d) sdot += (int32_t)qi[d] * (int32_t)sk[d];
-			float m = (float)sdot * temp;
+			float m = rs ? (float)sdot * (temp * 0.125f) : (float)sdot * temp;
 			float sum[4] = {63.75f, 63.75f, 63.75f, 63.75f};
 			float O[512];
 			for (size_t d = 0; d < hd; ++d) O[d] = (float)((int32_t)sv[d] * 255);
+			if (rs) {
+				for (size_t d = 0; d < hd; ++d) O[d] = O[d] * rs->sink_v_weight[h];
+			}
 			size_t j_lo = i - visible;
 			for (size_t t = j_lo / 16; t * 16 < i; ++t) {
 				float s[16];
@@ -463,7 +490,7 @@ static void attn_rows(size_t n_q, size_t pos0, size_t H, size_t hd,
 					const int8_t *kj = kv + j * kv_stride + h * 2 * hd;
 					int32_t dot = 0;
 					for (size_t d = 0; d < hd; ++d) dot += (int32_t)qi[d] * (int32_t)kj[d];
-					s[k] = (float)dot * temp;
+					s[k] = rs ? ((float)dot * rs->k_scale[j * H + h]) * temp : (float)dot * temp;
 					tmax = fmaxf(tmax, s[k]);
 				}
 				float resc = 1.0f;
@@ -477,7 +504,8 @@ static void attn_rows(size_t n_q, size_t pos0, size_t H, size_t hd,
 				for (size_t k = 0; k < 16; ++k) {
 					float e = fast_exp ? exp2f(s[k] - m) : sfu_ex2(s[k] - m);
 					p[k] = e * 255.0f;
-					P[k] = (int32_t)rintf(p[k]);
+					P[k] = rs && s[k] != -INFINITY ? (int32_t)rintf(p[k] * rs->v_weight[(t * 16 + k) * H + h])
+					                               : (int32_t)rintf(p[k]);
 				}
 				for (size_t qq = 0; qq < 4; ++qq) {
 					float add = (p[4 * qq] + p[4 * qq + 1]) + (p[4 * qq + 2] + p[4 * qq + 3]);
@@ -496,6 +524,17 @@ static void attn_rows(size_t n_q, size_t pos0, size_t H, size_t hd,
 			float S = (sum[0] + sum[1]) + (sum[2] + sum[3]);
 			if (L) L[h * l_stride + r] = sfu_lg2(S) + m;
 			float inv = sfu_rcp(S);
+			if (rs) {
+				float os = rs->out_scale[h];
+				if (rs->out_bf16) {
+					uint16_t *o = (uint16_t *)out + r * o_stride + h * hd;
+					for (size_t d = 0; d < hd; ++d) o[d] = bf16_rne((O[d] * inv) * os);
+				} else {
+					int8_t *o = out + r * o_stride + h * hd;
+					for (size_t d = 0; d < hd; ++d) o[d] = fixedi8((O[d] * inv) * os);
+				}
+				continue;
+			}
 			int8_t *o = out + r * o_stride + h * hd;
 			for (size_t d = 0; d < hd; ++d) o[d] = fixedi8(O[d] * inv);
 		}
@@ -509,7 +548,23 @@ X17_EXPORT int x17o_attn_fwd_i8(size_t T, size_t H, size_t hd,
                                 size_t window, int fast_exp) {
 	if (hd > 512) return -1;
 	attn_rows(T, 0, H, hd, q, H * hd, kv, 2 * H * hd, sink_k, sink_v, head_temp,
-	          out, H * hd, L, T, window, fast_exp);
+	          out, H * hd, L, T, window, fast_exp, NULL);
+	return 0;
+}
+
+/* attn_fwd_i8 with row-scaled operands (see RowScales above).  out is int8 [T, H*hd] or, with
+ * out_bf16 != 0, bf16 bits [T, H*hd]. */
+X17_EXPORT int x17o_attn_fwd_i8_row_scaled(size_t T, size_t H, size_t hd,
+                                           const int8_t *q, const int8_t *kv,
+                                           const int8_t *sink_k, const int8_t *sink_v,
+                                           const float *head_temp, void *out, float *L,
+                                           size_t window, int fast_exp,
+                                           const float *q_scale, const float *k_scale, const float *v_weight,
+                                           const float *sink_v_weight, const float *out_scale, int out_bf16) {
+	if (hd > 512) return -1;
+	RowScales rs = {q_scale, k_scale, v_weight, sink_v_weight, out_scale, out_bf16};
+	attn_rows(T, 0, H, hd, q, H * hd, kv, 2 * H * hd, sink_k, sink_v, head_temp,
+	          (int8_t *)out, H * hd, L, T, window, fast_exp, &rs);
 	return 0;
 }
 
@@ -530,7 +585,7 @@ X17_EXPORT int x17o_attn_decode_i8(size_t S, size_t cap, const uint32_t *cache_l
 		attn_rows(1, cache_len[s], H, hd, q + s * H * hd, H * hd,
 		          cache + s * cap * 2 * H * hd, 2 * H * hd,
 		          sink_k, sink_v, head_temp,
-		          out + s * H * hd, H * hd, L ? L + s * H : NULL, 1, window, fast_exp);
+		          out + s * H * hd, H * hd, L ? L + s * H : NULL, 1, window, fast_exp, NULL);
 	}
 	return 0;
 }

@@ -178,3 +178,94 @@ def test_rms_norm_bit_exact(dev, rows, d):
 	assert np.array_equal(out.download(), S.rms_norm(xb, recipes.L2_NORM_EPS, "bf16"))
 	with pytest.raises(X.X17Error, match="rows must be divisible by 8"):
 		kern.launch(X.Tensor(dev, (4, d), X.E4M3), X.Tensor(dev, (4, d), X.INT8))
+
+
+# ---------------------------------------------------------------- row-scaled operands (own definition)
+
+def _row_scaled_inputs(rng, rows, h, hd):
+	"""q, k, v ~ N(0, 1) times a per-(row, head) magnitude, quantised per row to int8 at absmax / 127."""
+	from oracle import dense as D
+	spread = np.exp(rng.normal(0.0, 0.5, (3, rows, h, 1)))
+	qc, qs = D.quantize_rows(rng.standard_normal((rows, h, hd)) * spread[0])
+	kc, ks = D.quantize_rows(rng.standard_normal((rows, h, hd)) * spread[1])
+	vc, vs = D.quantize_rows(rng.standard_normal((rows, h, hd)) * spread[2])
+	kv = np.concatenate((kc, vc), axis=2).reshape(rows, 2 * h * hd)
+	sink_k = i8_codes(rng, (h, hd))
+	sink_v = i8_codes(rng, (h, hd), 1.3)
+	temp = (0.5 + rng.random(h)).astype(np.float32)
+	return qc.reshape(rows, h * hd), kv, qs, ks, vs, sink_k, sink_v, temp
+
+
+def _run_row_scaled(dev, kern, q, kv, sink_k, sink_v, temp, window, qs, ks, vw, sw, osc, batch=1):
+	h = sink_k.shape[0]
+	out = X.Tensor(dev, q.shape, kern.config.out_dtype)
+	l = X.Tensor(dev, (h, q.shape[0]), X.F32)
+	f32 = lambda a: X.Tensor.from_numpy(dev, np.ascontiguousarray(a, dtype=np.float32), X.F32)
+	kern.launch_row_scaled(X.Tensor.from_numpy(dev, q, X.INT8), X.Tensor.from_numpy(dev, kv, X.INT8),
+	                       X.Tensor.from_numpy(dev, sink_k, X.INT8), X.Tensor.from_numpy(dev, sink_v, X.INT8),
+	                       f32(temp), out, l, window, f32(qs), f32(ks), f32(vw), f32(sw), f32(osc), batch)
+	return out.download(), l.download()
+
+
+# the first case is benchmark config 1 as written: per-row absmax / 127 scales, bf16 output
+@pytest.mark.parametrize("t,h,hd,w,out_dtype", [
+	(1024, 8, 64, 256, X.BF16), (384, 4, 32, 0, X.BF16), (640, 2, 128, 256, X.BF16), (512, 2, 64, 48, X.INT8),
+])
+def test_attn_row_scaled_strict_bit_exact(dev, t, h, hd, w, out_dtype):
+	rng = rng_for("attn-rows", t, h, hd, w)
+	q, kv, qs, ks, vs, sk, sv, temp = _row_scaled_inputs(rng, t, h, hd)
+	vw, sw, osc = recipes.attn_row_scale_operands(vs, out_dtype)
+	kern = recipes.attn_row_scaled_kernel(dev, h, hd, out_dtype, True)
+	got, got_l = _run_row_scaled(dev, kern, q, kv, sk, sv, temp, w, qs, ks, vw, sw, osc)
+	want, want_l = S.attn_fwd_i8_row_scaled(q, kv, sk, sv, temp, h, hd, w, qs, ks, vw, sw, osc, out_bf16=out_dtype == X.BF16)
+	assert np.array_equal(got, want)
+	assert np.array_equal(got_l.view(np.uint32), want_l.view(np.uint32))
+
+
+def test_attn_row_scaled_equals_plain_kernel_at_scale_one_eighth(dev):
+	"""With every scale 1/8 and every weight 1 the row-scaled kernel IS the reference's arithmetic."""
+	t, h, hd, w, b = 256, 2, 64, 64, 2
+	rng = rng_for("attn-rows-eighth")
+	q, kv, sk, sv, temp = _attn_inputs(rng, b * t, h, hd)
+	plain, plain_l = _run_attn(dev, recipes.attn_kernel(dev, h, hd, True), q, kv, sk, sv, temp, w, batch=b)
+	eighth = np.full((b * t, h), 0.125, np.float32)
+	kern = recipes.attn_row_scaled_kernel(dev, h, hd, X.INT8, True)
+	got, got_l = _run_row_scaled(dev, kern, q, kv, sk, sv, temp, w, eighth, eighth, np.ones((b * t, h)), np.ones(h), np.ones(h),
+	                             batch=b)
+	assert np.array_equal(got, plain)
+	assert np.array_equal(got_l.view(np.uint32), plain_l.view(np.uint32))
+
+
+@pytest.mark.parametrize("t,h,hd,w", [(1024, 8, 64, 256), (640, 2, 128, 256)])
+def test_attn_row_scaled_fast_within_tolerance(dev, t, h, hd, w):
+	"""Hardware-exponent build, bf16 output: relative L2 error against the strict definition below 2^-8
+	and no element further off than 3 % of the largest output (a probability that rounds the other way
+	moves one value row by one step)."""
+	rng = rng_for("attn-rows", t, h, hd, w)
+	q, kv, qs, ks, vs, sk, sv, temp = _row_scaled_inputs(rng, t, h, hd)
+	vw, sw, osc = recipes.attn_row_scale_operands(vs, X.BF16)
+	kern = recipes.attn_row_scaled_kernel(dev, h, hd, X.BF16, False)
+	got, got_l = _run_row_scaled(dev, kern, q, kv, sk, sv, temp, w, qs, ks, vw, sw, osc)
+	want, want_l = S.attn_fwd_i8_row_scaled(q, kv, sk, sv, temp, h, hd, w, qs, ks, vw, sw, osc, out_bf16=True)
+	g = (got.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+	e = (want.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+	rel_l2 = np.sqrt(np.sum((g - e) ** 2) / np.sum(e ** 2))
+	max_abs = np.abs(g - e).max() / np.abs(e).max()
+	assert rel_l2 < 2.0 ** -8 and max_abs < 0.03, (rel_l2, max_abs)
+	assert np.max(np.abs(got_l - want_l)) < 1e-4
+
+
+def test_attn_row_scaled_launch_checks(dev):
+	t, h, hd = 128, 2, 64
+	rng = rng_for("attn-rows-checks")
+	q, kv, qs, ks, vs, sk, sv, temp = _row_scaled_inputs(rng, t, h, hd)
+	vw, sw, osc = recipes.attn_row_scale_operands(vs, X.BF16)
+	kern = recipes.attn_row_scaled_kernel(dev, h, hd, X.BF16, True)
+	with pytest.raises(X.X17Error):          # scale matrix of the wrong shape
+		_run_row_scaled(dev, kern, q, kv, sk, sv, temp, 0, qs[:64], ks, vw, sw, osc)
+	with pytest.raises(X.X17Error):          # a plain launch of a row-scaled kernel
+		_run_attn(dev, kern, q, kv, sk, sv, temp, 0)
+	with pytest.raises(X.X17Error):          # and scales handed to a plain kernel
+		_run_row_scaled(dev, recipes.attn_kernel(dev, h, hd, True), q, kv, sk, sv, temp, 0, qs, ks, vw, sw, osc)
+	with pytest.raises(X.X17Error):          # bf16 output exists only with row scales
+		X.AttnKernel(None, "attn-bad-out", X.AttnKernelConfig(X.INT8, h, hd, h * hd, 2 * h * hd, h * hd, False, X.BF16))

@@ -290,3 +290,66 @@ def test_rms_norm_against_float64_and_legacy_known_answer():
 	exp = np.array([[-1.0451, -0.5656, -0.5322, -1.0963, -1.4501], [-1.1974, 0.6153, 1.7407, -0.2158, -0.3330],
 	                [0.1495, -0.9000, -0.6040, 1.8255, 0.6856], [0.1059, 1.8422, 0.0118, -1.0116, -0.7559]])
 	assert np.allclose(D.rms_norm(inp, 1e-5)[0], exp, atol=1e-4)
+
+
+# ---------------------------------------------------------------- row-scaled attention (own definition)
+
+def bf16_bits_to_f64(bits: np.ndarray) -> np.ndarray:
+	return (bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+
+
+def _row_scaled_inputs(r, t, h, hd):
+	"""q, k, v ~ N(0, 1) with a per-(row, head) spread of magnitudes, int8 codes at scale absmax / 127."""
+	spread = np.exp(r.normal(0.0, 0.7, (3, t, h, 1)))
+	qc, qs = D.quantize_rows(r.standard_normal((t, h, hd)) * spread[0])
+	kc, ks = D.quantize_rows(r.standard_normal((t, h, hd)) * spread[1])
+	vc, vs = D.quantize_rows(r.standard_normal((t, h, hd)) * spread[2])
+	sk = S.f32_to_fixedi8((r.standard_normal((h, hd)) * 8).astype(np.float32))
+	sv = S.f32_to_fixedi8((r.standard_normal((h, hd)) * 8).astype(np.float32))
+	temp = (0.5 + r.random(h)).astype(np.float32)
+	kv = np.concatenate((kc, vc), axis=2).reshape(t, -1)
+	return qc.reshape(t, -1), kv, qs, ks, vs, sk, sv, temp
+
+
+def test_row_scaled_attention_reduces_to_the_reference_mode_at_scale_one_eighth():
+	t, h, hd, w = 192, 2, 64, 48
+	q, kv, sk, sv, temp = _attn_inputs(_rng(31), t, h, hd)
+	ref_out, ref_l = S.attn_fwd_i8(q, kv, sk, sv, temp, h, hd, w)
+	eighth = np.full((t, h), 0.125, np.float32)
+	ones = np.ones((t, h), np.float32)
+	out, l = S.attn_fwd_i8_row_scaled(q, kv, sk, sv, temp, h, hd, w, eighth, eighth, ones, np.ones(h), np.ones(h))
+	assert np.array_equal(out, ref_out) and np.array_equal(l, ref_l)
+	# a power of two moves freely between the query scale and the head temperature (the key scale has no
+	# such partner: the sink key keeps its fixed scale of 1/8)
+	out2, l2 = S.attn_fwd_i8_row_scaled(q, kv, sk, sv, temp * 4, h, hd, w, eighth / 4, eighth, ones, np.ones(h), np.ones(h))
+	assert np.array_equal(out2, ref_out) and np.array_equal(l2, ref_l)
+	# the bf16 store holds the same values before their rounding to codes
+	outb, _ = S.attn_fwd_i8_row_scaled(q, kv, sk, sv, temp, h, hd, w, eighth, eighth, ones, np.ones(h), np.full(h, 0.125),
+	                                   out_bf16=True)
+	unclamped = np.abs(ref_out) < 127
+	assert np.all(np.abs(bf16_bits_to_f64(outb) * 8.0 - ref_out)[unclamped] <= 0.5 + 127 * 2.0 ** -8)
+
+
+@pytest.mark.parametrize("t,h,hd,w", [(256, 2, 64, 64), (192, 3, 32, 0), (128, 1, 128, 32)])
+def test_row_scaled_attention_against_dense_float64(t, h, hd, w):
+	from x17ai_amd.recipes import attn_row_scale_operands
+	from x17ai_amd.api import BF16
+	q, kv, qs, ks, vs, sk, sv, temp = _row_scaled_inputs(_rng(32), t, h, hd)
+	v_weight, sink_w, out_scale = attn_row_scale_operands(vs, BF16)
+	assert v_weight.max() == 1.0 and v_weight.min() > 0
+	out, _ = S.attn_fwd_i8_row_scaled(q, kv, sk, sv, temp, h, hd, w, qs, ks, v_weight, sink_w, out_scale, out_bf16=True)
+	got = bf16_bits_to_f64(out).reshape(t, h, hd)
+	kvr = kv.reshape(t, h, 2, hd)
+	for hh in range(h):
+		args = (q.reshape(t, h, hd)[:, hh], kvr[:, hh, 0], kvr[:, hh, 1], qs[:, hh], ks[:, hh], vs[:, hh],
+		        sk[hh] / 8.0, sv[hh] / 8.0, float(temp[hh]), w)
+		same_grid = D.attn_one_head_row_scaled(*args, quantize_p=True)
+		exact = D.attn_one_head_row_scaled(*args, quantize_p=False)
+		scale = np.abs(exact).max()
+		# same probability grid: bf16 rounding of the output (2^-9 relative) everywhere, except where a
+		# probability sits on a rounding boundary and goes the other way (one step of one value row)
+		err = np.abs(got[:, hh] - same_grid) / scale
+		assert np.mean(err > 2.0 ** -8) < 0.03 and err.max() < 0.03, (np.mean(err > 2.0 ** -8), err.max())
+		# exact softmax: what 8-bit probabilities cost
+		err = np.abs(got[:, hh] - exact) / scale
+		assert np.sqrt(np.mean(err ** 2)) < 0.01 and err.max() < 0.06, (np.sqrt(np.mean(err ** 2)), err.max())

@@ -305,6 +305,9 @@ class AttnKernelConfig:         # attn.rs:45-84
 	q_stride: int
 	kv_stride: int
 	o_stride: int
+	# extension: q/k/v codes with one f32 scale per (row, head); out_dtype INT8 (FixedI8) or, with row scales, BF16
+	row_scales: bool = False
+	out_dtype: int = INT8
 
 	def heads_per_kernel(self) -> int:
 		return 1 if self.head_dim == 0 else max(128 // self.head_dim, 1)
@@ -318,7 +321,7 @@ class AttnKernel:
 
 	def __init__(self, device: Optional[Device], kernel_name: str, config: AttnKernelConfig, strict_math: bool = True):
 		c = _ffi.AttnConfigC(config.dtype, config.n_heads, config.head_dim, config.q_stride, config.kv_stride,
-		                     config.o_stride, int(strict_math))
+		                     config.o_stride, int(strict_math), int(config.row_scales), config.out_dtype)
 		self.device = device
 		self.name = kernel_name
 		self.config = config
@@ -331,6 +334,14 @@ class AttnKernel:
 	           l: Optional[Tensor], window_size: int, batch: int = 1) -> None:
 		check(_ffi.host().x17h_attn_kernel_launch(self._h, q._h, kv._h, sink_k._h, sink_v._h, attn_temperature._h, out._h,
 		                                          l._h if l is not None else None, window_size, batch))
+
+	def launch_row_scaled(self, q: Tensor, kv: Tensor, sink_k: Tensor, sink_v: Tensor, attn_temperature: Tensor,
+	                      out: Tensor, l: Optional[Tensor], window_size: int, q_scale: Tensor, k_scale: Tensor,
+	                      v_weight: Tensor, sink_v_weight: Tensor, out_scale: Tensor, batch: int = 1) -> None:
+		"""Launch of a kernel built with config.row_scales (see recipes.attn_row_scale_operands)."""
+		check(_ffi.host().x17h_attn_kernel_launch_row_scaled(
+			self._h, q._h, kv._h, sink_k._h, sink_v._h, attn_temperature._h, out._h, l._h if l is not None else None,
+			window_size, batch, q_scale._h, k_scale._h, v_weight._h, sink_v_weight._h, out_scale._h))
 
 	def n_ops(self, seq_len: int, window_size: int) -> float:
 		return float(_ffi.host().x17h_attn_kernel_n_ops(self._h, seq_len, window_size))

@@ -905,6 +905,10 @@ double AttnKernelConfig::n_ops(size_t seq_len, size_t window_size) const {
 
 bool AttnKernelConfig::validate(Diagnostics &diag) const {
 	if (dtype != DType::Int8) { diag.add_error(std::string("attention kernel config currently requires dtype i8, got ") + dtype_name(dtype)); return false; }
+	if (out_dtype != DType::Int8 && !(row_scales && out_dtype == DType::Bf16)) {
+		diag.add_error(std::string("attention kernel config writes i8, or bf16 with row scales, got ") + dtype_name(out_dtype));
+		return false;
+	}
 	if (n_heads == 0) { diag.add_error("attention kernel config requires n_heads > 0"); return false; }
 	if (head_dim == 0 || head_dim % 32 != 0) {
 		diag.add_error("attention kernel config requires head_dim to be a non-zero multiple of 32, got " + std::to_string(head_dim));
@@ -939,6 +943,9 @@ std::unique_ptr<AttnKernel> AttnKernel::create(std::shared_ptr<HipDevice> device
 	common << "#define X17_N_HEADS " << config.n_heads << "\n#define X17_HEAD_DIM " << config.head_dim << "\n";
 	common << "#define X17_Q_STRIDE " << config.q_stride << "\n#define X17_KV_STRIDE " << config.kv_stride << "\n#define X17_O_STRIDE " << config.o_stride << "\n";
 	common << "#define X17_STRICT_MATH " << (strict_math ? 1 : 0) << "\n";
+	if (config.row_scales) {
+		common << "#define X17_ATTN_ROW_SCALES 1\n#define X17_ATTN_OUT_BF16 " << (config.out_dtype == DType::Bf16 ? 1 : 0) << "\n";
+	}
 	auto built = kernel_build::build(kernel_name, common.str(), "attn_fwd_i8.hip", "attn_meta.cpp", diag);
 	if (!built) return nullptr;
 	auto meta = kernel_build::read_metadata_json(built->meta_json_path, diag);
@@ -977,8 +984,26 @@ Status AttnKernel::launch(AttnKernelArgs const &a) {
 	if (!s.is_ok()) return s;
 	s = tensor_check::vector_shape("attention", "attn_temperature", *a.attn_temperature, config.n_heads, *device, DType::F32);
 	if (!s.is_ok()) return s;
-	s = tensor_check::matrix_shape("attention", "out", *a.out, rows, config.o_stride, *device, config.dtype, tmp);
+	s = tensor_check::matrix_shape("attention", "out", *a.out, rows, config.o_stride, *device, config.out_dtype, tmp);
 	if (!s.is_ok()) return s;
+	bool const any_scale = a.q_scale || a.k_scale || a.v_weight || a.sink_v_weight || a.out_scale;
+	if (config.row_scales) {
+		if (!a.q_scale || !a.k_scale || !a.v_weight || !a.sink_v_weight || !a.out_scale) {
+			return Status::err(TensorOpError::Other, "attention kernel " + name + " needs q_scale, k_scale, v_weight, sink_v_weight and out_scale");
+		}
+		s = tensor_check::matrix_shape("attention", "q_scale", *a.q_scale, rows, config.n_heads, *device, DType::F32, tmp);
+		if (!s.is_ok()) return s;
+		s = tensor_check::matrix_shape("attention", "k_scale", *a.k_scale, rows, config.n_heads, *device, DType::F32, tmp);
+		if (!s.is_ok()) return s;
+		s = tensor_check::matrix_shape("attention", "v_weight", *a.v_weight, rows, config.n_heads, *device, DType::F32, tmp);
+		if (!s.is_ok()) return s;
+		s = tensor_check::vector_shape("attention", "sink_v_weight", *a.sink_v_weight, config.n_heads, *device, DType::F32);
+		if (!s.is_ok()) return s;
+		s = tensor_check::vector_shape("attention", "out_scale", *a.out_scale, config.n_heads, *device, DType::F32);
+		if (!s.is_ok()) return s;
+	} else if (any_scale) {
+		return Status::err(TensorOpError::Other, "attention kernel " + name + " was built without row scales");
+	}
 	if (a.l != nullptr) {
 		s = tensor_check::matrix_shape("attention", "l", *a.l, config.n_heads, rows, *device, DType::F32, tmp);
 		if (!s.is_ok()) return s;
@@ -1002,7 +1027,14 @@ Status AttnKernel::launch(AttnKernelArgs const &a) {
 	void *out_ptr = a.out->ptr;
 	void *l_ptr = a.l != nullptr ? a.l->ptr : nullptr;
 	size_t window_arg = a.window_size;
-	void *raw_args[9] = {&seq_len_arg, &q_ptr, &kv_ptr, &sk, &sv, &tp, &out_ptr, &l_ptr, &window_arg};
+	void *scale_ptrs[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+	if (config.row_scales) {
+		Tensor const *t[5] = {a.q_scale, a.k_scale, a.v_weight, a.sink_v_weight, a.out_scale};
+		for (int i = 0; i < 5; ++i) scale_ptrs[i] = t[i]->ptr;
+	}
+	// the plain kernel takes the first nine arguments only
+	void *raw_args[14] = {&seq_len_arg, &q_ptr, &kv_ptr, &sk, &sv, &tp, &out_ptr, &l_ptr, &window_arg,
+	                      &scale_ptrs[0], &scale_ptrs[1], &scale_ptrs[2], &scale_ptrs[3], &scale_ptrs[4]};
 	size_t grid[3] = {seq_len / metadata.Q_PER_BLOCK, config.head_group_cnt(), a.batch};
 	size_t block[3] = {metadata.THREADS_PER_BLOCK, 1, 1};
 	return kernel->launch(*device->stream, grid, block, metadata.SMEM_BYTES, raw_args);
@@ -1339,7 +1371,9 @@ int x17h_gemm_kernel_attrs(X17hGemmKernel *k, int32_t out[9]) { return attrs_out
 int x17h_attn_kernel_new(X17hDevice *dev, char const *kernel_name, X17hAttnConfig const *c, X17hAttnKernel **out) {
 	try {
 		if (!valid_dtype(c->dtype)) return fail("unknown dtype");
-		AttnKernelConfig cfg{DType(c->dtype), c->n_heads, c->head_dim, c->q_stride, c->kv_stride, c->o_stride};
+		if (!valid_dtype(c->out_dtype)) return fail("unknown out_dtype");
+		AttnKernelConfig cfg{DType(c->dtype), c->n_heads, c->head_dim, c->q_stride, c->kv_stride, c->o_stride,
+		                     c->row_scales != 0, DType(c->out_dtype)};
 		Diagnostics diag;
 		auto k = AttnKernel::create(dev != nullptr ? dev->dev : nullptr, kernel_name, cfg, c->strict_math != 0, diag);
 		if (!k) return fail_diag("attention", diag);
@@ -1354,6 +1388,17 @@ int x17h_attn_kernel_launch(X17hAttnKernel *k, X17hTensor *q, X17hTensor *kv, X1
 	if (!q || !kv || !sink_k || !sink_v || !temp || !out) return fail("attention launch needs q, kv, sinks, temperature and out");
 	AttnKernelArgs a{q->t.get(), kv->t.get(), sink_k->t.get(), sink_v->t.get(), temp->t.get(), out->t.get(),
 	                 l != nullptr ? l->t.get() : nullptr, window_size, batch};
+	return from_status(k->k->launch(a));
+}
+int x17h_attn_kernel_launch_row_scaled(X17hAttnKernel *k, X17hTensor *q, X17hTensor *kv, X17hTensor *sink_k, X17hTensor *sink_v,
+                                       X17hTensor *temp, X17hTensor *out, X17hTensor *l, size_t window_size, size_t batch,
+                                       X17hTensor *q_scale, X17hTensor *k_scale, X17hTensor *v_weight,
+                                       X17hTensor *sink_v_weight, X17hTensor *out_scale) {
+	if (!q || !kv || !sink_k || !sink_v || !temp || !out) return fail("attention launch needs q, kv, sinks, temperature and out");
+	if (!q_scale || !k_scale || !v_weight || !sink_v_weight || !out_scale) return fail("row-scaled attention launch needs all five scale tensors");
+	AttnKernelArgs a{q->t.get(), kv->t.get(), sink_k->t.get(), sink_v->t.get(), temp->t.get(), out->t.get(),
+	                 l != nullptr ? l->t.get() : nullptr, window_size, batch,
+	                 q_scale->t.get(), k_scale->t.get(), v_weight->t.get(), sink_v_weight->t.get(), out_scale->t.get()};
 	return from_status(k->k->launch(a));
 }
 double x17h_attn_kernel_n_ops(X17hAttnKernel *k, size_t seq_len, size_t window_size) { return k->k->config.n_ops(seq_len, window_size); }

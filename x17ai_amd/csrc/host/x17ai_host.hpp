@@ -234,6 +234,10 @@ struct GemmKernel {
 
 struct AttnKernelConfig {
 	DType dtype; size_t n_heads, head_dim, q_stride, kv_stride, o_stride;
+	// Extension (the reference's codes all share the scale 1/8): one f32 scale per (row, head) for q, k and v.
+	// out_dtype is Int8 (FixedI8 codes) or, in the row-scaled build only, Bf16 (real values).
+	bool row_scales = false;
+	DType out_dtype = DType::Int8;
 	size_t heads_per_kernel() const;
 	size_t head_group_cnt() const;
 	size_t head_group_dim() const;
@@ -245,6 +249,9 @@ struct AttnKernelArgs {
 	Tensor const *q, *kv, *sink_k, *sink_v, *attn_temperature, *out, *l;   // l may be null
 	size_t window_size;
 	size_t batch = 1;       // extension: `batch` sequences of seq_len/batch rows, each with its own causal origin
+	// row-scaled kernels only: f32 [rows, n_heads] scales of q and k, weights (<= 1) of the value rows, and per head
+	// the weight of the sink value and the output scale
+	Tensor const *q_scale = nullptr, *k_scale = nullptr, *v_weight = nullptr, *sink_v_weight = nullptr, *out_scale = nullptr;
 };
 
 struct AttnLauncherMetadata { size_t THREADS_PER_BLOCK, SMEM_BYTES, Q_PER_BLOCK; };

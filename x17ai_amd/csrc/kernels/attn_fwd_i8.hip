@@ -39,6 +39,15 @@
 //
 // Extension over the reference ABI: gridDim.z = number of independent sequences stacked along
 // the rows of q / kv / out (each `seq_len` rows, own causal origin); L is [H, gridDim.z * seq_len].
+//
+// X17_ATTN_ROW_SCALES = 1 (no counterpart in the reference, whose codes share the constant scale 1/8):
+// five more parameters give one f32 scale per (row, head) for q and k, a weight <= 1 per (row, head)
+// for v, and per head the weight of the sink value and the output scale.  The recurrence becomes
+//   tq = ((f32(hd^-1/2) * lg2(n)) * head_temp[h]) * q_scale[i, h],  s_j = (f32(q_i . k_j) * k_scale[j, h]) * tq,
+//   sink score = f32(q_i . sink_k) * (tq * 0.125),  P_j = rne(p_j * v_weight[j, h]),
+//   O starts at f32(255 * sink_v) * sink_v_weight[h],  out = store((O * rcp(sum)) * out_scale[h])
+// and produces the bits of the plain kernel when every scale is 1/8 and every weight and out_scale is 1.
+// X17_ATTN_OUT_BF16 = 1 stores bf16 real values (round to nearest even) instead of FixedI8 codes.
 
 #include "common.h"
 #include "x17_device.h"
@@ -59,6 +68,9 @@ constexpr u32 K_SLICES = HD / 32;      // 32 bytes of head_dim per QK MFMA
 constexpr u32 D_BLOCKS = HD / 32;      // 32 output dims per PV MFMA
 constexpr u32 CPR = HD / 16;           // 16-byte chunks per key row
 constexpr bool STRICT = X17_STRICT_MATH != 0;
+constexpr bool ROW_SCALES = at::ROW_SCALES;
+constexpr bool OUT_BF16 = X17_ATTN_OUT_BF16 != 0;
+static_assert(ROW_SCALES || !OUT_BF16, "the bf16 output needs the row-scaled build (it supplies out_scale)");
 
 static_assert(HD == 32 || HD == 64 || HD == 128, "head_dim must be 32, 64 or 128");
 static_assert(N_HEADS % HPK == 0, "n_heads must be divisible by heads_per_kernel");
@@ -66,7 +78,8 @@ static_assert(N_HEADS % HPK == 0, "n_heads must be divisible by heads_per_kernel
 constexpr f32 PROB_SCALE = 255.0f;                                  // cuda/attn_fwd_i8.cuh:206
 constexpr f32 LOG2_PROB_SCALE = 7.9943534368588578f;                // lg2(255)
 constexpr f32 MAX_LIFT = 64.0f;                                     // 255 * 64 stays far inside f16
-constexpr f32 BASE_TEMPERATURE = f32(constexpr_inv_sqrt(f64(HD)) / 64.0);   // :47, :447-449
+constexpr f32 BASE_TEMPERATURE = ROW_SCALES ? f32(constexpr_inv_sqrt(f64(HD)))
+                                            : f32(constexpr_inv_sqrt(f64(HD)) / 64.0);   // :47, :447-449
 
 typedef short v4s __attribute__((ext_vector_type(4)));
 
@@ -119,6 +132,14 @@ void kernel(
 	i8 *out,
 	f32 *l_out,
 	u32 window_size
+#if X17_ATTN_ROW_SCALES
+	,
+	f32 const *q_scale,          // [rows, n_heads]
+	f32 const *k_scale,          // [rows, n_heads]
+	f32 const *v_weight,         // [rows, n_heads]
+	f32 const *sink_v_weight,    // [n_heads]
+	f32 const *out_scale         // [n_heads]
+#endif
 ) {
 	extern __shared__ __attribute__((aligned(1024))) u8 smem[];
 
@@ -177,6 +198,15 @@ void kernel(
 				__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(src + stage_k_src), X17_LDS_PTR(k_dst), 16, 0, 0);
 				__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(src + stage_v_src), X17_LDS_PTR(v_dst), 16, 0, 0);
 			}
+#if X17_ATTN_ROW_SCALES
+			if (wave == 0) {
+				// lanes 0..31 fetch the keys' scales, lanes 32..63 the value rows' weights: 4 bytes per lane
+				f32 const *base = half == 0 ? k_scale : v_weight;
+				f32 const *src = base + (row_base + (size_t)kb * at::KV_PER_STEP + qlane) * N_HEADS + head;
+				u8 *dst = smem + at::SCALE_RING_OFFSET + slot * at::SCALE_TILE_BYTES;
+				__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(src), X17_LDS_PTR(dst), 4, 0, 0);
+			}
+#endif
 		};
 		auto widen_v = [&](u32 slot, u32 tile) {
 			if (stager) {
@@ -196,9 +226,18 @@ void kernel(
 				*reinterpret_cast<v4u *>(dst + 16) = v4u{w[4], w[5], w[6], w[7]};
 			}
 		};
-		// each staging thread has two loads in flight per prefetched step; they complete in issue order
+		// each staging thread has two loads in flight per prefetched step (three in the first wavefront of
+		// the row-scaled build); they complete in issue order
 		auto wait_steps_in_flight = [&](u32 steps) {
-			if (steps >= 2) {
+			if (ROW_SCALES && wave == 0) {
+				if (steps >= 2) {
+					__builtin_amdgcn_s_waitcnt(0x0F76);          // vmcnt(6)
+				} else if (steps == 1) {
+					__builtin_amdgcn_s_waitcnt(0x0F73);          // vmcnt(3)
+				} else {
+					__builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0)
+				}
+			} else if (steps >= 2) {
 				__builtin_amdgcn_s_waitcnt(0x0F74);          // vmcnt(4)
 			} else if (steps == 1) {
 				__builtin_amdgcn_s_waitcnt(0x0F72);          // vmcnt(2)
@@ -216,6 +255,9 @@ void kernel(
 		u32 const visible = qi < wr ? qi : wr;
 		f32 temperature = BASE_TEMPERATURE * strict::lg2(f32(visible + 4u));
 		temperature = temperature * attn_temperature[head];
+#if X17_ATTN_ROW_SCALES
+		temperature = temperature * q_scale[(row_base + qi) * N_HEADS + head];
+#endif
 		// (the sign is the head's: lg2(visible + 4) >= 2)
 		bool const positive_temperature = __builtin_amdgcn_readfirstlane(f2u(attn_temperature[head])) - 1u < 0x7F7FFFFFu;
 
@@ -226,7 +268,7 @@ void kernel(
 		}
 		sink_dot += partner_i32(sink_dot, half);
 
-		f32 m = f32(sink_dot) * temperature;
+		f32 m = ROW_SCALES ? f32(sink_dot) * (temperature * 0.125f) : f32(sink_dot) * temperature;
 		f32 m_ref = m;                       // speed build: the maximum O's scale refers to, and 2^(m - m_ref)
 		f32 lift = 1.0f;
 		v2h lift2 = {(_Float16)1.0f, (_Float16)1.0f};
@@ -242,6 +284,14 @@ void kernel(
 				}
 			}
 		}
+#if X17_ATTN_ROW_SCALES
+		{
+			f32 const sink_weight = sink_v_weight[head];
+			X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
+				X17_UNROLL for (int r = 0; r < 16; ++r) o_acc[db][r] = o_acc[db][r] * sink_weight;
+			}
+		}
+#endif
 
 		// ---- pipeline prologue
 		u32 const n_steps = kb_end - kb_begin;
@@ -285,9 +335,22 @@ void kernel(
 					// Speed build, tile fully visible, positive temperature: the row maximum is taken over the
 					// integer dots (the scaling is monotone, so f32(max) * temperature IS the maximum score) and
 					// the scaling is fused into the exponent's subtraction further down.
-					bool const int_path = !STRICT && !need_mask && positive_temperature;
+					bool const int_path = !STRICT && !ROW_SCALES && !need_mask && positive_temperature;
 					f32 s[8];
 					f32 tmax;
+					// row-scaled build: this lane's 8 keys of the tile are 4 * half + {0..3} and 8 + 4 * half + {0..3}
+					[[maybe_unused]] f32 key_scale[8];
+					[[maybe_unused]] f32 value_weight[8];
+					if constexpr (ROW_SCALES) {
+						f32 const *sc = reinterpret_cast<f32 const *>(smem + at::SCALE_RING_OFFSET + slot * at::SCALE_TILE_BYTES)
+						                + 16 * tile + 4 * half;
+						v4f k0 = *reinterpret_cast<v4f const *>(sc), k1 = *reinterpret_cast<v4f const *>(sc + 8);
+						v4f w0 = *reinterpret_cast<v4f const *>(sc + 32), w1 = *reinterpret_cast<v4f const *>(sc + 40);
+						X17_UNROLL for (int r = 0; r < 4; ++r) {
+							key_scale[r] = k0[r]; key_scale[4 + r] = k1[r];
+							value_weight[r] = w0[r]; value_weight[4 + r] = w1[r];
+						}
+					}
 					if (int_path) {
 						i32 const *a = reinterpret_cast<i32 const *>(&s_acc) + 8 * tile;
 						auto mx = [](i32 x, i32 y) { return x > y ? x : y; };     // pairs of these become v_max3_i32
@@ -296,7 +359,11 @@ void kernel(
 						imax = imax > other ? imax : other;
 						tmax = f32(imax) * temperature;
 					} else {
-						X17_UNROLL for (u32 r = 0; r < 8; ++r) s[r] = f32(s_acc[8 * tile + r]) * temperature;
+						if constexpr (ROW_SCALES) {
+							X17_UNROLL for (u32 r = 0; r < 8; ++r) s[r] = (f32(s_acc[8 * tile + r]) * key_scale[r]) * temperature;
+						} else {
+							X17_UNROLL for (u32 r = 0; r < 8; ++r) s[r] = f32(s_acc[8 * tile + r]) * temperature;
+						}
 						if (need_mask) {
 							X17_UNROLL for (u32 r = 0; r < 8; ++r) {
 								u32 j = key0 + 16 * tile + 8 * (r / 4) + 4 * half + (r % 4);
@@ -355,6 +422,10 @@ void kernel(
 					sum_lo = fmaf32(sum_lo, resc, add_lo);
 					sum_hi = fmaf32(sum_hi, resc, add_hi);
 
+					if constexpr (ROW_SCALES) {
+						// the numerator takes the probabilities at the value rows' relative scales
+						X17_UNROLL for (u32 r = 0; r < 8; ++r) p[r] = p[r] * value_weight[r];
+					}
 					v4u pp;
 					X17_UNROLL for (int w = 0; w < 4; ++w) {
 						u32 word = pack_f16(__builtin_rintf(p[2 * w]), __builtin_rintf(p[2 * w + 1]));
@@ -411,6 +482,25 @@ void kernel(
 		if constexpr (!STRICT) {
 			inv = inv * sfu::rcp(lift);
 		}
+#if X17_ATTN_ROW_SCALES
+		f32 const head_out_scale = out_scale[head];
+		if constexpr (OUT_BF16) {
+			u16 *o_row = reinterpret_cast<u16 *>(out) + (row_base + qi) * O_STRIDE + (size_t)head * HD;
+			X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
+				X17_UNROLL for (int g = 0; g < 4; ++g) {
+					u32 b[4];
+					X17_UNROLL for (int e = 0; e < 4; ++e) b[e] = f32_to_bf16_rne((o_acc[db][4 * g + e] * inv) * head_out_scale);
+					v2u pair = {b[0] | (b[1] << 16), b[2] | (b[3] << 16)};
+					*reinterpret_cast<v2u *>(o_row + 32 * db + 8 * g + 4 * half) = pair;
+				}
+			}
+			continue;
+		}
+		X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
+			X17_UNROLL for (int r = 0; r < 16; ++r) o_acc[db][r] = (o_acc[db][r] * inv) * head_out_scale;
+		}
+		inv = 1.0f;          // exact: the stores below multiply by it once more
+#endif
 		i8 *o_row = out + (row_base + qi) * O_STRIDE + (size_t)head * HD;
 		X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
 			// word g of this lane = dims 32*db + 8*g + 4*half .. +3

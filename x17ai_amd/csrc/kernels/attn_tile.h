@@ -3,6 +3,13 @@
 // (reference: templates/attn/meta.cu:10-16).  Needs X17_HEAD_DIM from common.h.
 #pragma once
 
+#ifndef X17_ATTN_ROW_SCALES
+#define X17_ATTN_ROW_SCALES 0      // 1: q/k/v codes carry one f32 scale per (row, head)
+#endif
+#ifndef X17_ATTN_OUT_BF16
+#define X17_ATTN_OUT_BF16 0        // 1: the output is written as bf16 real values instead of FixedI8 codes
+#endif
+
 namespace x17 { namespace attn_tile {
 
 constexpr unsigned HEAD_DIM = X17_HEAD_DIM;
@@ -28,10 +35,14 @@ constexpr unsigned WAVES_PER_SIMD = X17_ATTN_WAVES_PER_SIMD;
 constexpr unsigned K_TILE_BYTES = KV_PER_STEP * HEAD_DIM;        // int8 keys, row = one key
 constexpr unsigned RAW_V_TILE_BYTES = KV_PER_STEP * HEAD_DIM;    // int8 values as they arrive
 constexpr unsigned V_TILE_BYTES = KV_PER_STEP * HEAD_DIM * 2;    // values widened to f16
-// LDS map: K ring | raw V ring | two f16 V tiles (the tile in use and the one being widened)
+// row-scaled operands: per step the 32 keys' scales followed by the 32 value rows' weights (f32)
+constexpr bool ROW_SCALES = X17_ATTN_ROW_SCALES != 0;
+constexpr unsigned SCALE_TILE_BYTES = 2 * KV_PER_STEP * 4;
+// LDS map: K ring | raw V ring | two f16 V tiles (the tile in use and the one being widened) | scale ring
 constexpr unsigned K_RING_OFFSET = 0;
 constexpr unsigned RAW_V_RING_OFFSET = RING * K_TILE_BYTES;
 constexpr unsigned V_TILES_OFFSET = RAW_V_RING_OFFSET + RING * RAW_V_TILE_BYTES;
-constexpr unsigned SMEM_BYTES = V_TILES_OFFSET + 2 * V_TILE_BYTES;
+constexpr unsigned SCALE_RING_OFFSET = V_TILES_OFFSET + 2 * V_TILE_BYTES;
+constexpr unsigned SMEM_BYTES = SCALE_RING_OFFSET + (ROW_SCALES ? RING * SCALE_TILE_BYTES : 0);
 
 }} // namespace x17::attn_tile

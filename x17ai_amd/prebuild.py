@@ -40,6 +40,10 @@ def _specs():
 		add(("attn", h, hd, True))
 	for h, hd in ((2, 64), (2, 128), (8, 64)):
 		add(("attn", h, hd, False))
+	for h, hd, out in ((8, 64, BF16), (4, 32, BF16), (2, 128, BF16), (2, 64, INT8), (2, 64, BF16)):
+		add(("attn_rows", h, hd, out, True))
+	for h, hd in ((8, 64), (2, 128)):
+		add(("attn_rows", h, hd, BF16, False))
 	for h, hd, cap in ((4, 32, 256), (4, 64, 256), (2, 128, 512)):
 		add(("decode", h, hd, cap, True))
 	for d in (512, 2048, 4096):
@@ -63,6 +67,7 @@ def _specs():
 	add(("ffn_f", 2048, 16384, False, E4M3))
 	add(("ffn_y", 2048, 8192, False, E4M3, INT8))
 	add(("attn", 8, 64, False))
+	add(("attn_rows", 32, 128, BF16, False))
 	add(("copy_probe",))
 	# ---- tests/test_gpu_fullsize.py (the strict ffn pair, attention and decode kernels are listed above)
 	add(("attn", 16, 128, True))
@@ -95,6 +100,8 @@ def _build_one(spec) -> str:
 		return recipes.ffn_f_f8_kernel(None, spec[1], spec[2], spec[3]).name
 	if kind == "attn":
 		return recipes.attn_kernel(None, spec[1], spec[2], spec[3]).name
+	if kind == "attn_rows":
+		return recipes.attn_row_scaled_kernel(None, spec[1], spec[2], spec[3], spec[4]).name
 	if kind == "decode":
 		return recipes.attn_decode_kernel(None, spec[1], spec[2], spec[3], spec[4]).name
 	if kind == "rms_norm":

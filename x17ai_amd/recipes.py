@@ -56,6 +56,16 @@ def attn_kernel(device: Optional[Device], n_heads: int, head_dim: int, strict: b
 	return AttnKernel(device, f"attn_fwd_i8-h{n_heads}-hd{head_dim}-{_mode(strict)}", cfg, strict)
 
 
+def attn_row_scaled_kernel(device: Optional[Device], n_heads: int, head_dim: int, out_dtype: int = BF16,
+                           strict: bool = True) -> AttnKernel:
+	"""The attention kernel over int8 codes with one scale per (row, head) -- symmetric absmax / 127
+	quantisation of q, k and v -- writing bf16 real values or FixedI8 codes."""
+	width = n_heads * head_dim
+	cfg = AttnKernelConfig(INT8, n_heads, head_dim, width, 2 * width, width, True, out_dtype)
+	tag = "bf16" if out_dtype == BF16 else "i8"
+	return AttnKernel(device, f"attn_fwd_i8_rows-h{n_heads}-hd{head_dim}-o{tag}-{_mode(strict)}", cfg, strict)
+
+
 def attn_y_kernel(device: Optional[Device], model_dim: int, attn_width: int, strict: bool = True,
                   c_dtype: int = E4M3) -> GemmKernel:
 	"""src/main.rs:525-576 -- attn_out[i8] . Wy[i8]^T with the gated-residual epilogue -> e4m3."""
@@ -116,3 +126,27 @@ def attn_decode_kernel(device: Optional[Device], n_heads: int, head_dim: int, ca
                        strict: bool = True) -> AttnDecodeKernel:
 	return AttnDecodeKernel(device, f"attn_decode_i8-h{n_heads}-hd{head_dim}-cap{cache_capacity}-{_mode(strict)}",
 	                        n_heads, head_dim, cache_capacity, strict)
+
+
+def attn_row_scale_operands(v_scale, out_dtype: int):
+	"""Per-head operands of the row-scaled attention kernel from the value rows' scales.
+
+	v_scale: float32 [rows, n_heads], real v = code * v_scale.  Returns float32 arrays
+	(v_weight [rows, n_heads], sink_v_weight [n_heads], out_scale [n_heads]): each head's largest value
+	scale becomes its reference scale v_ref, a row's 8-bit probabilities are weighted by
+	v_scale / v_ref <= 1, the sink value (a FixedI8 code, real = code / 8) enters at (1 / 8) / v_ref, and
+	the result is brought back by v_ref (bf16 output, real values) or 8 * v_ref (FixedI8 output)."""
+	import numpy as np
+	v_scale = np.asarray(v_scale, dtype=np.float32)
+	if v_scale.ndim != 2 or not np.all(np.isfinite(v_scale)) or not np.all(v_scale > 0):
+		raise ValueError("v_scale must be a [rows, n_heads] array of finite positive scales")
+	v_ref = v_scale.max(axis=0)
+	v_weight = (v_scale / v_ref[None, :]).astype(np.float32)
+	sink_v_weight = (np.float32(1.0 / FIXED_I8_SCALE) / v_ref).astype(np.float32)
+	if out_dtype == BF16:
+		out_scale = v_ref
+	elif out_dtype == INT8:
+		out_scale = (np.float32(FIXED_I8_SCALE) * v_ref).astype(np.float32)
+	else:
+		raise ValueError("row-scaled attention writes int8 or bf16")
+	return v_weight, sink_v_weight, out_scale
