@@ -251,9 +251,10 @@ def extras(dev, X, recipes):
 	p1 = W1 * (W1 - 1) // 2 + (T1 - W1) * W1
 	out["config1_attn"] = {"median_us": med * 1e6, "gops": 4.0 * HD1 * H1 * p1 / 1e9, "tops": 4.0 * HD1 * H1 * p1 / med / 1e12}
 
-	# the same shape as the configuration words it: one absmax / 127 scale per (row, head) of q, k and v, bf16 output
+	# the same shape as the configuration words it: one scale per (row, head) of q, k and v, bf16 output; the scales
+	# vary around 1/8 so that the scores keep the spread they have in the fixed-scale runs
 	def row_scale_tensors(rows, heads):
-		scales = [(0.02 * (0.5 + rng.random((rows, heads)))).astype(np.float32) for _ in range(3)]
+		scales = [(0.125 * (0.75 + 0.5 * rng.random((heads, rows)))).astype(np.float32) for _ in range(3)]
 		vw, sw, osc = recipes.attn_row_scale_operands(scales[2], X.BF16)
 		return [X.Tensor.from_numpy(dev, np.ascontiguousarray(a, dtype=np.float32), X.F32) for a in (scales[0], scales[1], vw, sw, osc)]
 	rs1 = row_scale_tensors(T1, H1)
@@ -301,6 +302,15 @@ def extras(dev, X, recipes):
 		c5[f"decode_{tag}_cache_gbs"] = nbytes / med / 1e9            # whole cache / time: counts the V rows skipped
 		c5[f"decode_{tag}_hbm_gbs"] = DECODE_TRAFFIC_BYTES / med / 1e9  # bytes actually fetched (rocprofv3) / time
 		c5[f"decode_{tag}_frac_of_hbm"] = DECODE_TRAFFIC_BYTES / med / 1e9 / PEAK_HBM_GBS
+	# the cache as a row-scaled prefill leaves it: one scale per (row, head) of k and v, bf16 output
+	kd_rows = recipes.attn_decode_row_scaled_kernel(dev, H5, HD5, CAP, X.BF16, False)
+	scale_one = [(0.125 * (0.75 + 0.5 * rng.random((1, H5, CAP)))).astype(np.float32) for _ in range(2)]
+	vw5, sw5, os5 = recipes.attn_row_scale_operands(np.broadcast_to(scale_one[1], (S5, H5, CAP)), X.BF16)
+	f32t = lambda a: X.Tensor.from_numpy(dev, np.ascontiguousarray(a, dtype=np.float32), X.F32)
+	rsd = [f32t(0.125 * (0.75 + 0.5 * rng.random((S5, H5)))), f32t(np.broadcast_to(scale_one[0], (S5, H5, CAP))), f32t(vw5), f32t(sw5), f32t(os5)]
+	odb = X.Tensor(dev, (S5, H5 * HD5), X.BF16)
+	med, _ = _median_launch(dev, X, lambda: kd_rows.launch_row_scaled(qd, cache, lens, sk5, sv5, tp5, odb, None, W5, *rsd), 10, 3)
+	c5["decode_row_scaled_bf16_us"] = med * 1e6
 	out["config5_long_context"] = c5
 	return out
 

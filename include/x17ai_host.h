@@ -124,7 +124,7 @@ int x17h_attn_kernel_launch(X17hAttnKernel *k, X17hTensor *q, X17hTensor *kv, X1
                             X17hTensor *l, size_t window_size, size_t batch);
 /* The same launch for a kernel built with row_scales (no counterpart in the reference; the closest
  * precedent is the per-head temperature vector of attn.rs:421-437).  q_scale, k_scale, v_weight: f32
- * [rows, n_heads]; sink_v_weight, out_scale: f32 [n_heads].  Real q = code * q_scale, real k = code * k_scale,
+ * [n_heads, rows] (head-major, like l); sink_v_weight, out_scale: f32 [n_heads].  Real q = code * q_scale, real k = code * k_scale,
  * real v = code * v_weight * v_ref[h]; sink_v_weight = (1/8) / v_ref, out_scale = v_ref (bf16 out) or 8 * v_ref. */
 int x17h_attn_kernel_launch_row_scaled(X17hAttnKernel *k, X17hTensor *q, X17hTensor *kv, X17hTensor *sink_k,
                                        X17hTensor *sink_v, X17hTensor *attn_temperature, X17hTensor *out,
@@ -150,6 +150,16 @@ void x17h_decode_kernel_free(X17hDecodeKernel *k);
 int x17h_decode_kernel_launch(X17hDecodeKernel *k, X17hTensor *q, X17hTensor *cache, X17hTensor *cache_len,
                               X17hTensor *sink_k, X17hTensor *sink_v, X17hTensor *attn_temperature,
                               X17hTensor *out, X17hTensor *l, size_t window_size);
+/* The decode kernel over a row-scaled cache (as X17hAttnConfig.row_scales; no reference counterpart):
+ * q_scale f32 [S, H]; k_scale, v_weight f32 [S, H, capacity]; sink_v_weight, out_scale f32 [H];
+ * out_dtype X17H_INT8 or X17H_BF16.  Only the scales of visible rows are read. */
+int x17h_decode_kernel_new_row_scaled(X17hDevice *dev, char const *kernel_name, size_t n_heads, size_t head_dim,
+                                      size_t cache_capacity, int strict_math, int out_dtype, X17hDecodeKernel **out);
+int x17h_decode_kernel_launch_row_scaled(X17hDecodeKernel *k, X17hTensor *q, X17hTensor *cache, X17hTensor *cache_len,
+                                         X17hTensor *sink_k, X17hTensor *sink_v, X17hTensor *attn_temperature,
+                                         X17hTensor *out, X17hTensor *l, size_t window_size,
+                                         X17hTensor *q_scale, X17hTensor *k_scale, X17hTensor *v_weight,
+                                         X17hTensor *sink_v_weight, X17hTensor *out_scale);
 
 /* Measurement aid with no reference counterpart: a plain device-to-device copy kernel of known
  * size, against which HBM-traffic counters are calibrated (src and dst: equal sizes, multiple of 16). */

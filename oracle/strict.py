@@ -227,7 +227,7 @@ def attn_fwd_i8(q, kv, sink_k, sink_v, head_temp, n_heads: int, head_dim: int, w
 def attn_fwd_i8_row_scaled(q, kv, sink_k, sink_v, head_temp, n_heads: int, head_dim: int, window: int,
                            q_scale, k_scale, v_weight, sink_v_weight, out_scale, out_bf16: bool = False,
                            want_l: bool = True, fast_exp: bool = False):
-	"""attn_fwd_i8 over row-scaled operands: q_scale, k_scale, v_weight float32 [T, H]; sink_v_weight,
+	"""attn_fwd_i8 over row-scaled operands: q_scale, k_scale, v_weight float32 [H, T]; sink_v_weight,
 	out_scale float32 [H].  Returns (out, L): out int8 codes, or bf16 bit patterns (uint16) with out_bf16."""
 	q = np.ascontiguousarray(q, dtype=np.int8)
 	kv = np.ascontiguousarray(kv, dtype=np.int8)
@@ -239,7 +239,7 @@ def attn_fwd_i8_row_scaled(q, kv, sink_k, sink_v, head_temp, n_heads: int, head_
 	assert sink_k.shape == (n_heads, head_dim) and sink_v.shape == (n_heads, head_dim)
 	rows = [np.ascontiguousarray(a, dtype=np.float32) for a in (q_scale, k_scale, v_weight)]
 	heads = [np.ascontiguousarray(a, dtype=np.float32).reshape(-1) for a in (sink_v_weight, out_scale)]
-	assert all(a.shape == (t, n_heads) for a in rows) and all(a.shape == (n_heads,) for a in heads)
+	assert all(a.shape == (n_heads, t) for a in rows) and all(a.shape == (n_heads,) for a in heads)
 	out = np.empty(q.shape, dtype=np.uint16 if out_bf16 else np.int8)
 	l = np.empty((n_heads, t), dtype=np.float32) if want_l else None
 	rc = lib().x17o_attn_fwd_i8_row_scaled(_sz(t), _sz(n_heads), _sz(head_dim), _p(q), _p(kv), _p(sink_k), _p(sink_v),
@@ -267,6 +267,36 @@ def attn_decode_i8(q, cache, cache_len, sink_k, sink_v, head_temp, n_heads: int,
 	                               _p(q), _p(cache), _p(sink_k), _p(sink_v), _p(head_temp),
 	                               _p(out), _p(l) if want_l else None, _sz(window),
 	                               ctypes.c_int(int(fast_exp)))
+	assert rc == 0
+	return out, l
+
+
+def attn_decode_i8_row_scaled(q, cache, cache_len, sink_k, sink_v, head_temp, n_heads: int, head_dim: int, window: int,
+                              q_scale, k_scale, v_weight, sink_v_weight, out_scale, out_bf16: bool = False,
+                              want_l: bool = True, fast_exp: bool = False):
+	"""attn_decode_i8 over row-scaled operands: q_scale float32 [S, H]; k_scale, v_weight [S, H, cap];
+	sink_v_weight, out_scale [H].  out: int8 codes or (out_bf16) bf16 bit patterns."""
+	q = np.ascontiguousarray(q, dtype=np.int8)
+	cache = np.ascontiguousarray(cache, dtype=np.int8)
+	cache_len = np.ascontiguousarray(cache_len, dtype=np.uint32)
+	sink_k = np.ascontiguousarray(sink_k, dtype=np.int8)
+	sink_v = np.ascontiguousarray(sink_v, dtype=np.int8)
+	head_temp = np.ascontiguousarray(head_temp, dtype=np.float32).reshape(-1)
+	s, cap, w = cache.shape
+	assert w == 2 * n_heads * head_dim and q.shape == (s, n_heads * head_dim)
+	q_scale = np.ascontiguousarray(q_scale, dtype=np.float32)
+	k_scale = np.ascontiguousarray(k_scale, dtype=np.float32)
+	v_weight = np.ascontiguousarray(v_weight, dtype=np.float32)
+	heads = [np.ascontiguousarray(a, dtype=np.float32).reshape(-1) for a in (sink_v_weight, out_scale)]
+	assert q_scale.shape == (s, n_heads) and k_scale.shape == (s, n_heads, cap) and v_weight.shape == (s, n_heads, cap)
+	assert all(a.shape == (n_heads,) for a in heads)
+	out = np.empty(q.shape, dtype=np.uint16 if out_bf16 else np.int8)
+	l = np.empty((s, n_heads), dtype=np.float32) if want_l else None
+	rc = lib().x17o_attn_decode_i8_row_scaled(_sz(s), _sz(cap), _p(cache_len), _sz(n_heads), _sz(head_dim),
+	                                          _p(q), _p(cache), _p(sink_k), _p(sink_v), _p(head_temp),
+	                                          _p(out), _p(l) if want_l else None, _sz(window), ctypes.c_int(int(fast_exp)),
+	                                          _p(q_scale), _p(k_scale), _p(v_weight), _p(heads[0]), _p(heads[1]),
+	                                          ctypes.c_int(int(out_bf16)))
 	assert rc == 0
 	return out, l
 

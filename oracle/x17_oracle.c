@@ -432,20 +432,21 @@ X17_EXPORT void x17o_epilogue_l2norm(const int32_t *acc, int8_t *C, float *rrms,
  * hardware-exponent build may drift from the strict definition.
  *
  * Row-scaled operands (`rs` != NULL; no counterpart in the reference, whose q/k/v are FixedI8 codes
- * with the one constant scale 1/8).  Real values are q_code * q_scale[row, h], k_code * k_scale[row, h],
- * v_code * v_scale[row, h]; the caller passes v_weight = v_scale / v_ref[h] (<= 1),
+ * with the one constant scale 1/8).  Real values are q_code * q_scale[h, row], k_code * k_scale[h, row],
+ * v_code * v_scale[h, row] (head-major, like L); the caller passes v_weight = v_scale / v_ref[h] (<= 1),
  * sink_v_weight[h] = (1/8) / v_ref[h] and out_scale[h] = v_ref[h] * (8 for a FixedI8 output, 1 for bf16).
  * The recurrence is the one above with
- *   tq  = ((f32(hd^-1/2) * lg2(n)) * head_temp[h]) * q_scale[i, h]
- *   s_j = (f32(q_i . k_j) * k_scale[j, h]) * tq,   sink score = f32(q_i . sink_k) * (tq * 0.125)
- *   P_j = rne(p_j * v_weight[j, h]) (the partial sums still add the unweighted p_j)
+ *   tq  = ((f32(hd^-1/2) * lg2(n)) * head_temp[h]) * q_scale[h, i]
+ *   s_j = (f32(q_i . k_j) * k_scale[h, j]) * tq,   sink score = f32(q_i . sink_k) * (tq * 0.125)
+ *   P_j = rne(p_j * v_weight[h, j]) (the partial sums still add the unweighted p_j)
  *   O starts at f32(255 * sink_v) * sink_v_weight[h];   out = store((O * rcp(sum)) * out_scale[h])
  * so that with every scale 1/8 and every weight and out_scale 1 each step produces the bits of the
  * reference mode (multiplications by powers of two commute with rounding). */
 typedef struct {
-	const float *q_scale;        /* [n_q, H] */
-	const float *k_scale;        /* [kv rows, H] */
-	const float *v_weight;       /* [kv rows, H] */
+	const float *q_scale;        /* [H, n_q] */
+	const float *k_scale;        /* [H, kv_rows] */
+	const float *v_weight;       /* [H, kv_rows] */
+	size_t kv_rows;
 	const float *sink_v_weight;  /* [H] */
 	const float *out_scale;      /* [H] */
 	int out_bf16;                /* 0: FixedI8 bytes, 1: bf16 (out is then uint16_t*, o_stride in elements) */
@@ -470,7 +471,7 @@ static void attn_rows(size_t n_q, size_t pos0, size_t H, size_t hd,
 			uint32_t n = (uint32_t)visible + 4u;
 			float temp = base * sfu_lg2((float)n);
 			temp = temp * head_temp[h];
-			if (rs) temp = temp * rs->q_scale[r * H + h];
+			if (rs) temp = temp * rs->q_scale[h * n_q + r];
 			int32_t sdot = 0;
 			for (size_t d = 0; d < hd; ++d) sdot += (int32_t)qi[d] * (int32_t)sk[d];
 			float m = rs ? (float)sdot * (temp * 0.125f) : (float)sdot * temp;
@@ -490,7 +491,7 @@ static void attn_rows(size_t n_q, size_t pos0, size_t H, size_t hd,
 					const int8_t *kj = kv + j * kv_stride + h * 2 * hd;
 					int32_t dot = 0;
 					for (size_t d = 0; d < hd; ++d) dot += (int32_t)qi[d] * (int32_t)kj[d];
-					s[k] = rs ? ((float)dot * rs->k_scale[j * H + h]) * temp : (float)dot * temp;
+					s[k] = rs ? ((float)dot * rs->k_scale[h * rs->kv_rows + j]) * temp : (float)dot * temp;
 					tmax = fmaxf(tmax, s[k]);
 				}
 				float resc = 1.0f;
@@ -504,7 +505,7 @@ static void attn_rows(size_t n_q, size_t pos0, size_t H, size_t hd,
 				for (size_t k = 0; k < 16; ++k) {
 					float e = fast_exp ? exp2f(s[k] - m) : sfu_ex2(s[k] - m);
 					p[k] = e * 255.0f;
-					P[k] = rs && s[k] != -INFINITY ? (int32_t)rintf(p[k] * rs->v_weight[(t * 16 + k) * H + h])
+					P[k] = rs && s[k] != -INFINITY ? (int32_t)rintf(p[k] * rs->v_weight[h * rs->kv_rows + t * 16 + k])
 					                               : (int32_t)rintf(p[k]);
 				}
 				for (size_t qq = 0; qq < 4; ++qq) {
@@ -562,7 +563,7 @@ X17_EXPORT int x17o_attn_fwd_i8_row_scaled(size_t T, size_t H, size_t hd,
                                            const float *q_scale, const float *k_scale, const float *v_weight,
                                            const float *sink_v_weight, const float *out_scale, int out_bf16) {
 	if (hd > 512) return -1;
-	RowScales rs = {q_scale, k_scale, v_weight, sink_v_weight, out_scale, out_bf16};
+	RowScales rs = {q_scale, k_scale, v_weight, T, sink_v_weight, out_scale, out_bf16};
 	attn_rows(T, 0, H, hd, q, H * hd, kv, 2 * H * hd, sink_k, sink_v, head_temp,
 	          (int8_t *)out, H * hd, L, T, window, fast_exp, &rs);
 	return 0;
@@ -586,6 +587,29 @@ X17_EXPORT int x17o_attn_decode_i8(size_t S, size_t cap, const uint32_t *cache_l
 		          cache + s * cap * 2 * H * hd, 2 * H * hd,
 		          sink_k, sink_v, head_temp,
 		          out + s * H * hd, H * hd, L ? L + s * H : NULL, 1, window, fast_exp, NULL);
+	}
+	return 0;
+}
+
+/* Single-token decode over row-scaled operands: q_scale [S, H], k_scale and v_weight [S, H, cap],
+ * sink_v_weight and out_scale [H]; out is int8 or (out_bf16) bf16 bits, [S, H*hd]. */
+X17_EXPORT int x17o_attn_decode_i8_row_scaled(size_t S, size_t cap, const uint32_t *cache_len,
+                                              size_t H, size_t hd,
+                                              const int8_t *q, const int8_t *cache,
+                                              const int8_t *sink_k, const int8_t *sink_v,
+                                              const float *head_temp, void *out, float *L,
+                                              size_t window, int fast_exp,
+                                              const float *q_scale, const float *k_scale, const float *v_weight,
+                                              const float *sink_v_weight, const float *out_scale, int out_bf16) {
+	if (hd > 512) return -1;
+	size_t out_elem = out_bf16 ? 2 : 1;
+	for (size_t s = 0; s < S; ++s) {
+		if (cache_len[s] > cap) return -2;
+		RowScales rs = {q_scale + s * H, k_scale + s * H * cap, v_weight + s * H * cap, cap, sink_v_weight, out_scale, out_bf16};
+		attn_rows(1, cache_len[s], H, hd, q + s * H * hd, H * hd,
+		          cache + s * cap * 2 * H * hd, 2 * H * hd,
+		          sink_k, sink_v, head_temp,
+		          (int8_t *)out + s * H * hd * out_elem, H * hd, L ? L + s * H : NULL, 1, window, fast_exp, &rs);
 	}
 	return 0;
 }

@@ -193,7 +193,8 @@ def _row_scaled_inputs(rng, rows, h, hd):
 	sink_k = i8_codes(rng, (h, hd))
 	sink_v = i8_codes(rng, (h, hd), 1.3)
 	temp = (0.5 + rng.random(h)).astype(np.float32)
-	return qc.reshape(rows, h * hd), kv, qs, ks, vs, sink_k, sink_v, temp
+	head_major = lambda a: np.ascontiguousarray(a.T)          # the scale matrices are [H, rows], like L
+	return qc.reshape(rows, h * hd), kv, head_major(qs), head_major(ks), head_major(vs), sink_k, sink_v, temp
 
 
 def _run_row_scaled(dev, kern, q, kv, sink_k, sink_v, temp, window, qs, ks, vw, sw, osc, batch=1):
@@ -228,9 +229,9 @@ def test_attn_row_scaled_equals_plain_kernel_at_scale_one_eighth(dev):
 	rng = rng_for("attn-rows-eighth")
 	q, kv, sk, sv, temp = _attn_inputs(rng, b * t, h, hd)
 	plain, plain_l = _run_attn(dev, recipes.attn_kernel(dev, h, hd, True), q, kv, sk, sv, temp, w, batch=b)
-	eighth = np.full((b * t, h), 0.125, np.float32)
+	eighth = np.full((h, b * t), 0.125, np.float32)
 	kern = recipes.attn_row_scaled_kernel(dev, h, hd, X.INT8, True)
-	got, got_l = _run_row_scaled(dev, kern, q, kv, sk, sv, temp, w, eighth, eighth, np.ones((b * t, h)), np.ones(h), np.ones(h),
+	got, got_l = _run_row_scaled(dev, kern, q, kv, sk, sv, temp, w, eighth, eighth, np.ones((h, b * t)), np.ones(h), np.ones(h),
 	                             batch=b)
 	assert np.array_equal(got, plain)
 	assert np.array_equal(got_l.view(np.uint32), plain_l.view(np.uint32))
@@ -262,10 +263,41 @@ def test_attn_row_scaled_launch_checks(dev):
 	vw, sw, osc = recipes.attn_row_scale_operands(vs, X.BF16)
 	kern = recipes.attn_row_scaled_kernel(dev, h, hd, X.BF16, True)
 	with pytest.raises(X.X17Error):          # scale matrix of the wrong shape
-		_run_row_scaled(dev, kern, q, kv, sk, sv, temp, 0, qs[:64], ks, vw, sw, osc)
+		_run_row_scaled(dev, kern, q, kv, sk, sv, temp, 0, qs[:, :64], ks, vw, sw, osc)
 	with pytest.raises(X.X17Error):          # a plain launch of a row-scaled kernel
 		_run_attn(dev, kern, q, kv, sk, sv, temp, 0)
 	with pytest.raises(X.X17Error):          # and scales handed to a plain kernel
 		_run_row_scaled(dev, recipes.attn_kernel(dev, h, hd, True), q, kv, sk, sv, temp, 0, qs, ks, vw, sw, osc)
 	with pytest.raises(X.X17Error):          # bf16 output exists only with row scales
 		X.AttnKernel(None, "attn-bad-out", X.AttnKernelConfig(X.INT8, h, hd, h * hd, 2 * h * hd, h * hd, False, X.BF16))
+
+
+@pytest.mark.parametrize("h,hd,cap,w,out_dtype", [(4, 64, 256, 64, X.BF16), (2, 128, 512, 0, X.BF16), (4, 32, 256, 0, X.INT8)])
+def test_decode_row_scaled_bit_exact(dev, h, hd, cap, w, out_dtype):
+	s = 6
+	rng = rng_for("decode-rows", h, hd, cap, w)
+	q, kv, qs, ks, vs, sk, sv, temp = _row_scaled_inputs(rng, s * cap, h, hd)
+	cache = kv.reshape(s, cap, 2 * h * hd)
+	lens = np.array([0, 1, 17, cap // 2 + 5, cap - 1, cap], dtype=np.uint32)
+	per_cache = lambda a: np.ascontiguousarray(a.reshape(h, s, cap).transpose(1, 0, 2))      # [S, H, cap]
+	vw, sw, osc = recipes.attn_row_scale_operands(per_cache(vs), out_dtype)
+	ks3 = per_cache(ks)
+	for i, n in enumerate(lens):                    # rows past the cached length hold no scale worth reading
+		ks3[i, :, n:] = np.nan
+		vw[i, :, n:] = np.nan
+	qd, qsd = q[:s], np.ascontiguousarray(qs[:, :s].T)
+	kern = recipes.attn_decode_row_scaled_kernel(dev, h, hd, cap, out_dtype, True)
+	out = X.Tensor(dev, (s, h * hd), out_dtype)
+	l = X.Tensor(dev, (s, h), X.F32)
+	f32 = lambda a: X.Tensor.from_numpy(dev, np.ascontiguousarray(a, dtype=np.float32), X.F32)
+	kern.launch_row_scaled(X.Tensor.from_numpy(dev, qd, X.INT8), X.Tensor.from_numpy(dev, cache, X.INT8),
+	                       X.Tensor.from_numpy(dev, lens.view(np.float32), X.F32), X.Tensor.from_numpy(dev, sk, X.INT8),
+	                       X.Tensor.from_numpy(dev, sv, X.INT8), f32(temp), out, l, w, f32(qsd), f32(ks3), f32(vw), f32(sw), f32(osc))
+	want, want_l = S.attn_decode_i8_row_scaled(qd, cache, lens, sk, sv, temp, h, hd, w, qsd, ks3, vw, sw, osc,
+	                                           out_bf16=out_dtype == X.BF16)
+	assert np.array_equal(out.download(), want)
+	assert np.array_equal(l.download().view(np.uint32), want_l.view(np.uint32))
+	with pytest.raises(X.X17Error):                 # a plain launch of a row-scaled kernel
+		kern.launch(X.Tensor.from_numpy(dev, qd, X.INT8), X.Tensor.from_numpy(dev, cache, X.INT8),
+		            X.Tensor.from_numpy(dev, lens.view(np.float32), X.F32), X.Tensor.from_numpy(dev, sk, X.INT8),
+		            X.Tensor.from_numpy(dev, sv, X.INT8), f32(temp), out, l, w)

@@ -308,15 +308,16 @@ def _row_scaled_inputs(r, t, h, hd):
 	sv = S.f32_to_fixedi8((r.standard_normal((h, hd)) * 8).astype(np.float32))
 	temp = (0.5 + r.random(h)).astype(np.float32)
 	kv = np.concatenate((kc, vc), axis=2).reshape(t, -1)
-	return qc.reshape(t, -1), kv, qs, ks, vs, sk, sv, temp
+	head_major = lambda a: np.ascontiguousarray(a.T)          # the scale matrices are [H, T], like L
+	return qc.reshape(t, -1), kv, head_major(qs), head_major(ks), head_major(vs), sk, sv, temp
 
 
 def test_row_scaled_attention_reduces_to_the_reference_mode_at_scale_one_eighth():
 	t, h, hd, w = 192, 2, 64, 48
 	q, kv, sk, sv, temp = _attn_inputs(_rng(31), t, h, hd)
 	ref_out, ref_l = S.attn_fwd_i8(q, kv, sk, sv, temp, h, hd, w)
-	eighth = np.full((t, h), 0.125, np.float32)
-	ones = np.ones((t, h), np.float32)
+	eighth = np.full((h, t), 0.125, np.float32)
+	ones = np.ones((h, t), np.float32)
 	out, l = S.attn_fwd_i8_row_scaled(q, kv, sk, sv, temp, h, hd, w, eighth, eighth, ones, np.ones(h), np.ones(h))
 	assert np.array_equal(out, ref_out) and np.array_equal(l, ref_l)
 	# a power of two moves freely between the query scale and the head temperature (the key scale has no
@@ -341,7 +342,7 @@ def test_row_scaled_attention_against_dense_float64(t, h, hd, w):
 	got = bf16_bits_to_f64(out).reshape(t, h, hd)
 	kvr = kv.reshape(t, h, 2, hd)
 	for hh in range(h):
-		args = (q.reshape(t, h, hd)[:, hh], kvr[:, hh, 0], kvr[:, hh, 1], qs[:, hh], ks[:, hh], vs[:, hh],
+		args = (q.reshape(t, h, hd)[:, hh], kvr[:, hh, 0], kvr[:, hh, 1], qs[hh], ks[hh], vs[hh],
 		        sk[hh] / 8.0, sv[hh] / 8.0, float(temp[hh]), w)
 		same_grid = D.attn_one_head_row_scaled(*args, quantize_p=True)
 		exact = D.attn_one_head_row_scaled(*args, quantize_p=False)
@@ -353,3 +354,23 @@ def test_row_scaled_attention_against_dense_float64(t, h, hd, w):
 		# exact softmax: what 8-bit probabilities cost
 		err = np.abs(got[:, hh] - exact) / scale
 		assert np.sqrt(np.mean(err ** 2)) < 0.01 and err.max() < 0.06, (np.sqrt(np.mean(err ** 2)), err.max())
+
+
+def test_row_scaled_decode_is_the_row_scaled_prefill_row():
+	from x17ai_amd.recipes import attn_row_scale_operands
+	from x17ai_amd.api import BF16
+	t, h, hd, w = 128, 2, 64, 32
+	q, kv, qs, ks, vs, sk, sv, temp = _row_scaled_inputs(_rng(33), t, h, hd)
+	vw, sink_w, out_scale = attn_row_scale_operands(vs, BF16)
+	pre, pre_l = S.attn_fwd_i8_row_scaled(q, kv, sk, sv, temp, h, hd, w, qs, ks, vw, sink_w, out_scale, out_bf16=True)
+	for p in (0, 1, 17, 100):
+		cap = 112                                   # rows from p on are never read: poison them
+		cache = np.full((1, cap, 2 * h * hd), 99, np.int8)
+		cache[0, :p] = kv[:p]
+		kc = np.full((1, h, cap), np.nan, np.float32)
+		kc[0, :, :p] = ks[:, :p]
+		vc = np.full((1, h, cap), np.nan, np.float32)
+		vc[0, :, :p] = vw[:, :p]
+		out, l = S.attn_decode_i8_row_scaled(q[p:p + 1], cache, np.array([p], np.uint32), sk, sv, temp, h, hd, w,
+		                                     qs[:, p][None, :], kc, vc, sink_w, out_scale, out_bf16=True)
+		assert np.array_equal(out[0], pre[p]) and np.array_equal(l[0], pre_l[:, p])

@@ -116,6 +116,8 @@ def host() -> ctypes.CDLL:
 	h.x17h_rms_norm_kernel_free.restype = None
 	h.x17h_rms_norm_kernel_launch.argtypes = [P, P, P]
 	h.x17h_decode_kernel_new.argtypes = [P, ctypes.c_char_p, SZ, SZ, SZ, ctypes.c_int, PP]
+	h.x17h_decode_kernel_new_row_scaled.argtypes = [P, ctypes.c_char_p, SZ, SZ, SZ, ctypes.c_int, ctypes.c_int, PP]
+	h.x17h_decode_kernel_launch_row_scaled.argtypes = [P, P, P, P, P, P, P, P, P, SZ, P, P, P, P, P]
 	h.x17h_decode_kernel_free.argtypes = [P]
 	h.x17h_decode_kernel_free.restype = None
 	h.x17h_decode_kernel_launch.argtypes = [P, P, P, P, P, P, P, P, P, SZ]

@@ -338,7 +338,8 @@ class AttnKernel:
 	def launch_row_scaled(self, q: Tensor, kv: Tensor, sink_k: Tensor, sink_v: Tensor, attn_temperature: Tensor,
 	                      out: Tensor, l: Optional[Tensor], window_size: int, q_scale: Tensor, k_scale: Tensor,
 	                      v_weight: Tensor, sink_v_weight: Tensor, out_scale: Tensor, batch: int = 1) -> None:
-		"""Launch of a kernel built with config.row_scales (see recipes.attn_row_scale_operands)."""
+		"""Launch of a kernel built with config.row_scales: q_scale, k_scale, v_weight are f32 [n_heads, rows]
+		(see recipes.attn_row_scale_operands)."""
 		check(_ffi.host().x17h_attn_kernel_launch_row_scaled(
 			self._h, q._h, kv._h, sink_k._h, sink_v._h, attn_temperature._h, out._h, l._h if l is not None else None,
 			window_size, batch, q_scale._h, k_scale._h, v_weight._h, sink_v_weight._h, out_scale._h))
@@ -394,13 +395,30 @@ class AttnDecodeKernel:
 	"""Single-token decode against an int8 KV cache (no counterpart in the reference)."""
 
 	def __init__(self, device: Optional[Device], kernel_name: str, n_heads: int, head_dim: int, cache_capacity: int,
-	             strict_math: bool = True):
+	             strict_math: bool = True, row_scales: bool = False, out_dtype: int = INT8):
 		self.device = device
 		self.name = kernel_name
+		self.row_scales = row_scales
+		self.out_dtype = out_dtype
 		self._h = ctypes.c_void_p()
-		check(_ffi.host().x17h_decode_kernel_new(device._h if device is not None else None, kernel_name.encode(),
-		                                         n_heads, head_dim, cache_capacity, int(strict_math), ctypes.byref(self._h)))
+		dev_h = device._h if device is not None else None
+		if row_scales:
+			check(_ffi.host().x17h_decode_kernel_new_row_scaled(dev_h, kernel_name.encode(), n_heads, head_dim, cache_capacity,
+			                                                    int(strict_math), out_dtype, ctypes.byref(self._h)))
+		else:
+			if out_dtype != INT8:
+				raise X17Error("the decode kernel writes bf16 only with row scales")
+			check(_ffi.host().x17h_decode_kernel_new(dev_h, kernel_name.encode(), n_heads, head_dim, cache_capacity,
+			                                         int(strict_math), ctypes.byref(self._h)))
 		self.diagnostics = _ffi.last_diagnostics()
+
+	def launch_row_scaled(self, q: Tensor, cache: Tensor, cache_len: Tensor, sink_k: Tensor, sink_v: Tensor,
+	                      attn_temperature: Tensor, out: Tensor, l: Optional[Tensor], window_size: int, q_scale: Tensor,
+	                      k_scale: Tensor, v_weight: Tensor, sink_v_weight: Tensor, out_scale: Tensor) -> None:
+		"""q_scale [S, H]; k_scale, v_weight [S, H, capacity]; sink_v_weight, out_scale [H] (all f32)."""
+		check(_ffi.host().x17h_decode_kernel_launch_row_scaled(
+			self._h, q._h, cache._h, cache_len._h, sink_k._h, sink_v._h, attn_temperature._h, out._h,
+			l._h if l is not None else None, window_size, q_scale._h, k_scale._h, v_weight._h, sink_v_weight._h, out_scale._h))
 
 	def launch(self, q: Tensor, cache: Tensor, cache_len: Tensor, sink_k: Tensor, sink_v: Tensor,
 	           attn_temperature: Tensor, out: Tensor, l: Optional[Tensor], window_size: int) -> None:

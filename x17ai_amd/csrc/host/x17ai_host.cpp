@@ -991,11 +991,11 @@ Status AttnKernel::launch(AttnKernelArgs const &a) {
 		if (!a.q_scale || !a.k_scale || !a.v_weight || !a.sink_v_weight || !a.out_scale) {
 			return Status::err(TensorOpError::Other, "attention kernel " + name + " needs q_scale, k_scale, v_weight, sink_v_weight and out_scale");
 		}
-		s = tensor_check::matrix_shape("attention", "q_scale", *a.q_scale, rows, config.n_heads, *device, DType::F32, tmp);
+		s = tensor_check::matrix_shape("attention", "q_scale", *a.q_scale, config.n_heads, rows, *device, DType::F32, tmp);
 		if (!s.is_ok()) return s;
-		s = tensor_check::matrix_shape("attention", "k_scale", *a.k_scale, rows, config.n_heads, *device, DType::F32, tmp);
+		s = tensor_check::matrix_shape("attention", "k_scale", *a.k_scale, config.n_heads, rows, *device, DType::F32, tmp);
 		if (!s.is_ok()) return s;
-		s = tensor_check::matrix_shape("attention", "v_weight", *a.v_weight, rows, config.n_heads, *device, DType::F32, tmp);
+		s = tensor_check::matrix_shape("attention", "v_weight", *a.v_weight, config.n_heads, rows, *device, DType::F32, tmp);
 		if (!s.is_ok()) return s;
 		s = tensor_check::vector_shape("attention", "sink_v_weight", *a.sink_v_weight, config.n_heads, *device, DType::F32);
 		if (!s.is_ok()) return s;
@@ -1115,6 +1115,13 @@ std::unique_ptr<AttnDecodeKernel> AttnDecodeKernel::create(std::shared_ptr<HipDe
 	common << "#define X17_N_HEADS " << config.n_heads << "\n#define X17_HEAD_DIM " << config.head_dim << "\n";
 	common << "#define X17_CACHE_CAPACITY " << config.cache_capacity << "\n";
 	common << "#define X17_STRICT_MATH " << (strict_math ? 1 : 0) << "\n";
+	if (config.out_dtype != DType::Int8 && !(config.row_scales && config.out_dtype == DType::Bf16)) {
+		diag.add_error(std::string("decode kernel writes i8, or bf16 with row scales, got ") + dtype_name(config.out_dtype));
+		return nullptr;
+	}
+	if (config.row_scales) {
+		common << "#define X17_ATTN_ROW_SCALES 1\n#define X17_ATTN_OUT_BF16 " << (config.out_dtype == DType::Bf16 ? 1 : 0) << "\n";
+	}
 	auto built = kernel_build::build(kernel_name, common.str(), "attn_decode_i8.hip", "decode_meta.cpp", diag);
 	if (!built) return nullptr;
 	auto meta = kernel_build::read_metadata_json(built->meta_json_path, diag);
@@ -1159,8 +1166,30 @@ Status AttnDecodeKernel::launch(AttnDecodeArgs const &a) {
 	if (!s.is_ok()) return s;
 	s = tensor_check::vector_shape("decode", "attn_temperature", *a.attn_temperature, config.n_heads, *device, DType::F32);
 	if (!s.is_ok()) return s;
-	s = tensor_check::matrix_shape("decode", "out", *a.out, seqs, width, *device, DType::Int8, tmp);
+	s = tensor_check::matrix_shape("decode", "out", *a.out, seqs, width, *device, config.out_dtype, tmp);
 	if (!s.is_ok()) return s;
+	bool const any_scale = a.q_scale || a.k_scale || a.v_weight || a.sink_v_weight || a.out_scale;
+	if (config.row_scales) {
+		if (!a.q_scale || !a.k_scale || !a.v_weight || !a.sink_v_weight || !a.out_scale) {
+			return Status::err(TensorOpError::Other, "decode kernel " + name + " needs q_scale, k_scale, v_weight, sink_v_weight and out_scale");
+		}
+		s = tensor_check::matrix_shape("decode", "q_scale", *a.q_scale, seqs, config.n_heads, *device, DType::F32, tmp);
+		if (!s.is_ok()) return s;
+		for (auto [label, t] : {std::pair<char const *, Tensor const *>{"k_scale", a.k_scale}, {"v_weight", a.v_weight}}) {
+			if (t->shape.size() != 3 || t->shape[0] != seqs || t->shape[1] != config.n_heads || t->shape[2] != config.cache_capacity) {
+				return Status::err(TensorOpError::Other, std::string("decode input ") + label + " must have shape [" + std::to_string(seqs) + ", "
+					+ std::to_string(config.n_heads) + ", " + std::to_string(config.cache_capacity) + "], got " + tensor_check::shape_str(t->shape));
+			}
+			s = tensor_check::dtype_and_device("decode", label, *t, *device, DType::F32);
+			if (!s.is_ok()) return s;
+		}
+		s = tensor_check::vector_shape("decode", "sink_v_weight", *a.sink_v_weight, config.n_heads, *device, DType::F32);
+		if (!s.is_ok()) return s;
+		s = tensor_check::vector_shape("decode", "out_scale", *a.out_scale, config.n_heads, *device, DType::F32);
+		if (!s.is_ok()) return s;
+	} else if (any_scale) {
+		return Status::err(TensorOpError::Other, "decode kernel " + name + " was built without row scales");
+	}
 	if (a.l != nullptr) {
 		s = tensor_check::matrix_shape("decode", "l", *a.l, seqs, config.n_heads, *device, DType::F32, tmp);
 		if (!s.is_ok()) return s;
@@ -1173,7 +1202,14 @@ Status AttnDecodeKernel::launch(AttnDecodeArgs const &a) {
 	void *tp = a.attn_temperature->ptr, *out_ptr = a.out->ptr;
 	void *l_ptr = a.l != nullptr ? a.l->ptr : nullptr;
 	size_t window_arg = a.window_size;
-	void *raw_args[9] = {&q_ptr, &cache_ptr, &len_ptr, &sk, &sv, &tp, &out_ptr, &l_ptr, &window_arg};
+	void *scale_ptrs[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+	if (config.row_scales) {
+		Tensor const *t[5] = {a.q_scale, a.k_scale, a.v_weight, a.sink_v_weight, a.out_scale};
+		for (int i = 0; i < 5; ++i) scale_ptrs[i] = t[i]->ptr;
+	}
+	// the plain kernel takes the first nine arguments only
+	void *raw_args[14] = {&q_ptr, &cache_ptr, &len_ptr, &sk, &sv, &tp, &out_ptr, &l_ptr, &window_arg,
+	                      &scale_ptrs[0], &scale_ptrs[1], &scale_ptrs[2], &scale_ptrs[3], &scale_ptrs[4]};
 	size_t grid[3] = {config.n_heads / metadata.HEADS_PER_BLOCK, seqs, 1};
 	size_t block[3] = {metadata.THREADS_PER_BLOCK, 1, 1};
 	return kernel->launch(*device->stream, grid, block, metadata.SMEM_BYTES, raw_args);
@@ -1436,6 +1472,30 @@ int x17h_decode_kernel_new(X17hDevice *dev, char const *kernel_name, size_t n_he
 		*out = new X17hDecodeKernel{std::move(k)};
 		return 0;
 	} catch (std::exception const &e) { return fail(e.what()); }
+}
+int x17h_decode_kernel_new_row_scaled(X17hDevice *dev, char const *kernel_name, size_t n_heads, size_t head_dim, size_t cache_capacity,
+                                      int strict_math, int out_dtype, X17hDecodeKernel **out) {
+	try {
+		if (!valid_dtype(out_dtype)) return fail("unknown out_dtype");
+		Diagnostics diag;
+		auto k = AttnDecodeKernel::create(dev != nullptr ? dev->dev : nullptr, kernel_name,
+		                                  AttnDecodeConfig{n_heads, head_dim, cache_capacity, true, DType(out_dtype)}, strict_math != 0, diag);
+		if (!k) return fail_diag("decode", diag);
+		stash_diag(diag);
+		*out = new X17hDecodeKernel{std::move(k)};
+		return 0;
+	} catch (std::exception const &e) { return fail(e.what()); }
+}
+int x17h_decode_kernel_launch_row_scaled(X17hDecodeKernel *k, X17hTensor *q, X17hTensor *cache, X17hTensor *cache_len, X17hTensor *sink_k,
+                                         X17hTensor *sink_v, X17hTensor *temp, X17hTensor *out, X17hTensor *l, size_t window_size,
+                                         X17hTensor *q_scale, X17hTensor *k_scale, X17hTensor *v_weight,
+                                         X17hTensor *sink_v_weight, X17hTensor *out_scale) {
+	if (!q || !cache || !cache_len || !sink_k || !sink_v || !temp || !out) return fail("decode launch needs q, cache, cache_len, sinks, temperature and out");
+	if (!q_scale || !k_scale || !v_weight || !sink_v_weight || !out_scale) return fail("row-scaled decode launch needs all five scale tensors");
+	AttnDecodeArgs a{q->t.get(), cache->t.get(), cache_len->t.get(), sink_k->t.get(), sink_v->t.get(), temp->t.get(), out->t.get(),
+	                 l != nullptr ? l->t.get() : nullptr, window_size,
+	                 q_scale->t.get(), k_scale->t.get(), v_weight->t.get(), sink_v_weight->t.get(), out_scale->t.get()};
+	return from_status(k->k->launch(a));
 }
 void x17h_decode_kernel_free(X17hDecodeKernel *k) { delete k; }
 int x17h_decode_kernel_launch(X17hDecodeKernel *k, X17hTensor *q, X17hTensor *cache, X17hTensor *cache_len, X17hTensor *sink_k,

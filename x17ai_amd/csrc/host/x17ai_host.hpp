@@ -249,7 +249,7 @@ struct AttnKernelArgs {
 	Tensor const *q, *kv, *sink_k, *sink_v, *attn_temperature, *out, *l;   // l may be null
 	size_t window_size;
 	size_t batch = 1;       // extension: `batch` sequences of seq_len/batch rows, each with its own causal origin
-	// row-scaled kernels only: f32 [rows, n_heads] scales of q and k, weights (<= 1) of the value rows, and per head
+	// row-scaled kernels only: f32 [n_heads, rows] scales of q and k, weights (<= 1) of the value rows, and per head
 	// the weight of the sink value and the output scale
 	Tensor const *q_scale = nullptr, *k_scale = nullptr, *v_weight = nullptr, *sink_v_weight = nullptr, *out_scale = nullptr;
 };
@@ -285,11 +285,17 @@ struct RmsNormKernel {
 	Status launch(Tensor const &inp, Tensor const &out);
 };
 
-struct AttnDecodeConfig { size_t n_heads, head_dim, cache_capacity; };
+struct AttnDecodeConfig {
+	size_t n_heads, head_dim, cache_capacity;
+	bool row_scales = false;             // as AttnKernelConfig::row_scales
+	DType out_dtype = DType::Int8;       // Int8, or Bf16 with row scales
+};
 struct AttnDecodeMetadata { size_t THREADS_PER_BLOCK, SMEM_BYTES, HEADS_PER_BLOCK; };
 struct AttnDecodeArgs {
 	Tensor const *q, *cache, *cache_len, *sink_k, *sink_v, *attn_temperature, *out, *l;   // l may be null
 	size_t window_size;
+	// row-scaled kernels only: q_scale [S, H], k_scale and v_weight [S, H, capacity], sink_v_weight and out_scale [H]
+	Tensor const *q_scale = nullptr, *k_scale = nullptr, *v_weight = nullptr, *sink_v_weight = nullptr, *out_scale = nullptr;
 };
 
 struct AttnDecodeKernel {

@@ -22,6 +22,10 @@
 // common.h provides X17_N_HEADS, X17_HEAD_DIM, X17_CACHE_CAPACITY, X17_STRICT_MATH.
 // Layouts: q, out [S, H*hd]; cache [S, CAPACITY, H*2*hd] (per head K then V, as kv of the
 // prefill kernel); cache_len u32 [S]; L [S, H] or null.
+//
+// X17_ATTN_ROW_SCALES = 1: the row-scaled recurrence of attn_fwd_i8.hip for the one query -- q_scale
+// [S, H], k_scale and v_weight [S, H, CAPACITY], sink_v_weight and out_scale [H]; X17_ATTN_OUT_BF16 = 1
+// writes bf16 real values.  Only visible rows' scales are read (the rest of a cache may be uninitialised).
 
 #include "common.h"
 #include "x17_device.h"
@@ -37,7 +41,16 @@ constexpr u32 CAP = X17_CACHE_CAPACITY;
 constexpr u32 CPR = HD / 16;                         // lanes per key row
 constexpr u32 ROW = 2 * N_HEADS * HD;                // bytes per cache row
 constexpr u32 KEYS_PER_PASS = dt::THREADS_PER_BLOCK / CPR;
-constexpr f32 BASE_TEMPERATURE = f32(constexpr_inv_sqrt(f64(HD)) / 64.0);
+#ifndef X17_ATTN_ROW_SCALES
+#define X17_ATTN_ROW_SCALES 0
+#endif
+#ifndef X17_ATTN_OUT_BF16
+#define X17_ATTN_OUT_BF16 0
+#endif
+constexpr bool ROW_SCALES = X17_ATTN_ROW_SCALES != 0;
+constexpr bool OUT_BF16 = X17_ATTN_OUT_BF16 != 0;
+static_assert(ROW_SCALES || !OUT_BF16, "the bf16 output needs the row-scaled build (it supplies out_scale)");
+constexpr f32 BASE_TEMPERATURE = ROW_SCALES ? f32(constexpr_inv_sqrt(f64(HD))) : f32(constexpr_inv_sqrt(f64(HD)) / 64.0);
 static_assert(HD == 32 || HD == 64 || HD == 128, "head_dim must be 32, 64 or 128");
 static_assert(CAP % 16 == 0, "cache capacity must be a multiple of 16");
 static_assert(dt::CHUNK_TILES * CPR == dt::THREADS_PER_BLOCK || dt::CHUNK_TILES * CPR < dt::THREADS_PER_BLOCK,
@@ -49,6 +62,10 @@ void kernel(
 	i8 const *q, i8 const *cache, u32 const *cache_len,
 	i8 const *sink_k, i8 const *sink_v, f32 const *attn_temperature,
 	i8 *out, f32 *l_out, u32 window_size
+#if X17_ATTN_ROW_SCALES
+	,
+	f32 const *q_scale, f32 const *k_scale, f32 const *v_weight, f32 const *sink_v_weight, f32 const *out_scale
+#endif
 ) {
 	extern __shared__ __attribute__((aligned(16))) u8 smem[];
 	// the scores are dead once the probabilities exist, so the P.V partials of phase 4 reuse their space
@@ -80,6 +97,11 @@ void kernel(
 
 	f32 temperature = BASE_TEMPERATURE * strict::lg2(f32(visible + 4u));
 	temperature = temperature * attn_temperature[head];
+#if X17_ATTN_ROW_SCALES
+	temperature = temperature * q_scale[(size_t)seq * N_HEADS + head];
+	f32 const *k_scale_head = k_scale + ((size_t)seq * N_HEADS + head) * CAP;     // indexed by cache row
+	f32 const *v_weight_head = v_weight + ((size_t)seq * N_HEADS + head) * CAP;
+#endif
 
 	// this lane's 16 bytes of the query (chunk tid % CPR)
 	u32 const c = tid % CPR;
@@ -92,7 +114,7 @@ void kernel(
 		X17_UNROLL for (int w = 0; w < 4; ++w) sink_dot = __builtin_amdgcn_sdot4(qc[w], sk[w], sink_dot, false);
 		X17_UNROLL for (u32 mask = 1; mask < CPR; mask <<= 1) sink_dot += __shfl_xor(sink_dot, (int)mask, 64);
 	}
-	f32 const m0 = f32(sink_dot) * temperature;
+	f32 const m0 = ROW_SCALES ? f32(sink_dot) * (temperature * 0.125f) : f32(sink_dot) * temperature;
 
 	// ---- phase 1: scores of all keys of the walked tiles.  A thread keeps BATCH independent 16-byte
 	// loads in flight (a load per pass would leave the kernel waiting on memory latency).
@@ -100,12 +122,16 @@ void kernel(
 	constexpr u32 BATCH = 8;
 	for (u32 base = 0; base < n_keys; base += KEYS_PER_PASS * BATCH) {
 		v4i kc[BATCH];
+		[[maybe_unused]] f32 ksc[BATCH];
 		X17_UNROLL for (u32 bb = 0; bb < BATCH; ++bb) {
 			u32 kidx = base + bb * KEYS_PER_PASS + tid / CPR;
 			u32 j = t0 * 16 + kidx;
 			bool vis = kidx < n_keys && j >= j_lo && j < pos;
 			u32 j_safe = vis ? j : pos - 1;                   // a row that exists (n_tiles > 0 means pos >= 1)
 			kc[bb] = *reinterpret_cast<v4i const *>(kv_head + (size_t)j_safe * ROW + 16 * c);
+#if X17_ATTN_ROW_SCALES
+			ksc[bb] = k_scale_head[j_safe];
+#endif
 		}
 		X17_UNROLL for (u32 bb = 0; bb < BATCH; ++bb) {
 			u32 kidx = base + bb * KEYS_PER_PASS + tid / CPR;
@@ -116,7 +142,8 @@ void kernel(
 			X17_UNROLL for (int w = 0; w < 4; ++w) dot = __builtin_amdgcn_sdot4(qc[w], kc[bb][w], dot, false);
 			X17_UNROLL for (u32 mask = 1; mask < CPR; mask <<= 1) dot += __shfl_xor(dot, (int)mask, 64);
 			if (in_range && c == 0) {
-				s_score[kidx] = vis ? f32(dot) * temperature : -__builtin_inff();
+				f32 const score = ROW_SCALES ? (f32(dot) * ksc[bb]) * temperature : f32(dot) * temperature;
+				s_score[kidx] = vis ? score : -__builtin_inff();
 			}
 		}
 	}
@@ -181,6 +208,18 @@ void kernel(
 		f32 p2 = sfu::ex2(s[2] - m) * 255.0f;
 		f32 p3 = sfu::ex2(s[3] - m) * 255.0f;
 		s_quad[quad] = (p0 + p1) + (p2 + p3);
+#if X17_ATTN_ROW_SCALES
+		{
+			// the numerator takes the probabilities at the value rows' relative scales; masked keys keep 0
+			u32 const j = t0 * 16 + quad * 4;
+			// (rows of a partly visible quad are inside the cache: its capacity is a multiple of 16)
+			v4f const vw = *reinterpret_cast<v4f const *>(v_weight_head + j);
+			p0 = s[0] == -__builtin_inff() ? 0.0f : p0 * vw[0];
+			p1 = s[1] == -__builtin_inff() ? 0.0f : p1 * vw[1];
+			p2 = s[2] == -__builtin_inff() ? 0.0f : p2 * vw[2];
+			p3 = s[3] == -__builtin_inff() ? 0.0f : p3 * vw[3];
+		}
+#endif
 		u32 packed = (u32)(i32)__builtin_rintf(p0) | ((u32)(i32)__builtin_rintf(p1) << 8)
 			| ((u32)(i32)__builtin_rintf(p2) << 16) | ((u32)(i32)__builtin_rintf(p3) << 24);
 		*reinterpret_cast<u32 *>(s_prob + quad * 4) = packed;
@@ -231,6 +270,9 @@ void kernel(
 	f32 o = 0.0f;
 	if (tid < HD) {
 		o = f32((i32)sink_v[(size_t)head * HD + tid] * 255);
+#if X17_ATTN_ROW_SCALES
+		o = o * sink_v_weight[head];
+#endif
 	}
 	for (u32 chunk = 0; chunk < n_act; chunk += dt::CHUNK_TILES) {
 		u32 const tiles_here = n_act - chunk < dt::CHUNK_TILES ? n_act - chunk : dt::CHUNK_TILES;
@@ -293,6 +335,16 @@ void kernel(
 		l_out[(size_t)seq * N_HEADS + head] = strict::lg2(total) + m_final;
 	}
 	if (tid < HD) {
-		out[(size_t)seq * N_HEADS * HD + (size_t)head * HD + tid] = (i8)f32_to_fixedi8(o * strict::rcp(total));
+		size_t const idx = (size_t)seq * N_HEADS * HD + (size_t)head * HD + tid;
+#if X17_ATTN_ROW_SCALES
+		f32 const value = (o * strict::rcp(total)) * out_scale[head];
+		if constexpr (OUT_BF16) {
+			reinterpret_cast<u16 *>(out)[idx] = (u16)f32_to_bf16_rne(value);
+		} else {
+			out[idx] = (i8)f32_to_fixedi8(value);
+		}
+#else
+		out[idx] = (i8)f32_to_fixedi8(o * strict::rcp(total));
+#endif
 	}
 }

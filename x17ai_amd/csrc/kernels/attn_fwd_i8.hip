@@ -41,10 +41,11 @@
 // the rows of q / kv / out (each `seq_len` rows, own causal origin); L is [H, gridDim.z * seq_len].
 //
 // X17_ATTN_ROW_SCALES = 1 (no counterpart in the reference, whose codes share the constant scale 1/8):
-// five more parameters give one f32 scale per (row, head) for q and k, a weight <= 1 per (row, head)
-// for v, and per head the weight of the sink value and the output scale.  The recurrence becomes
-//   tq = ((f32(hd^-1/2) * lg2(n)) * head_temp[h]) * q_scale[i, h],  s_j = (f32(q_i . k_j) * k_scale[j, h]) * tq,
-//   sink score = f32(q_i . sink_k) * (tq * 0.125),  P_j = rne(p_j * v_weight[j, h]),
+// five more parameters give one f32 scale per (head, row) for q and k, a weight <= 1 per (head, row)
+// for v (all three laid out [H, rows] like L), and per head the weight of the sink value and the output
+// scale.  The recurrence becomes
+//   tq = ((f32(hd^-1/2) * lg2(n)) * head_temp[h]) * q_scale[h, i],  s_j = (f32(q_i . k_j) * k_scale[h, j]) * tq,
+//   sink score = f32(q_i . sink_k) * (tq * 0.125),  P_j = rne(p_j * v_weight[h, j]),
 //   O starts at f32(255 * sink_v) * sink_v_weight[h],  out = store((O * rcp(sum)) * out_scale[h])
 // and produces the bits of the plain kernel when every scale is 1/8 and every weight and out_scale is 1.
 // X17_ATTN_OUT_BF16 = 1 stores bf16 real values (round to nearest even) instead of FixedI8 codes.
@@ -134,9 +135,9 @@ void kernel(
 	u32 window_size
 #if X17_ATTN_ROW_SCALES
 	,
-	f32 const *q_scale,          // [rows, n_heads]
-	f32 const *k_scale,          // [rows, n_heads]
-	f32 const *v_weight,         // [rows, n_heads]
+	f32 const *q_scale,          // [n_heads, rows]
+	f32 const *k_scale,          // [n_heads, rows]
+	f32 const *v_weight,         // [n_heads, rows]
 	f32 const *sink_v_weight,    // [n_heads]
 	f32 const *out_scale         // [n_heads]
 #endif
@@ -202,7 +203,7 @@ void kernel(
 			if (wave == 0) {
 				// lanes 0..31 fetch the keys' scales, lanes 32..63 the value rows' weights: 4 bytes per lane
 				f32 const *base = half == 0 ? k_scale : v_weight;
-				f32 const *src = base + (row_base + (size_t)kb * at::KV_PER_STEP + qlane) * N_HEADS + head;
+				f32 const *src = base + (size_t)head * ((size_t)gridDim.z * seq_len) + row_base + (size_t)kb * at::KV_PER_STEP + qlane;
 				u8 *dst = smem + at::SCALE_RING_OFFSET + slot * at::SCALE_TILE_BYTES;
 				__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(src), X17_LDS_PTR(dst), 4, 0, 0);
 			}
@@ -256,7 +257,7 @@ void kernel(
 		f32 temperature = BASE_TEMPERATURE * strict::lg2(f32(visible + 4u));
 		temperature = temperature * attn_temperature[head];
 #if X17_ATTN_ROW_SCALES
-		temperature = temperature * q_scale[(row_base + qi) * N_HEADS + head];
+		temperature = temperature * q_scale[(size_t)head * ((size_t)gridDim.z * seq_len) + row_base + qi];
 #endif
 		// (the sign is the head's: lg2(visible + 4) >= 2)
 		bool const positive_temperature = __builtin_amdgcn_readfirstlane(f2u(attn_temperature[head])) - 1u < 0x7F7FFFFFu;

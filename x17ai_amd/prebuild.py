@@ -46,6 +46,8 @@ def _specs():
 		add(("attn_rows", h, hd, BF16, False))
 	for h, hd, cap in ((4, 32, 256), (4, 64, 256), (2, 128, 512)):
 		add(("decode", h, hd, cap, True))
+	for h, hd, cap, out in ((4, 64, 256, BF16), (2, 128, 512, BF16), (4, 32, 256, INT8)):
+		add(("decode_rows", h, hd, cap, out, True))
 	for d in (512, 2048, 4096):
 		add(("rms_norm", d, E4M3))
 		add(("rms_norm", d, BF16))
@@ -68,6 +70,7 @@ def _specs():
 	add(("ffn_y", 2048, 8192, False, E4M3, INT8))
 	add(("attn", 8, 64, False))
 	add(("attn_rows", 32, 128, BF16, False))
+	add(("decode_rows", 32, 128, 4096, BF16, False))
 	add(("copy_probe",))
 	# ---- tests/test_gpu_fullsize.py (the strict ffn pair, attention and decode kernels are listed above)
 	add(("attn", 16, 128, True))
@@ -104,6 +107,8 @@ def _build_one(spec) -> str:
 		return recipes.attn_row_scaled_kernel(None, spec[1], spec[2], spec[3], spec[4]).name
 	if kind == "decode":
 		return recipes.attn_decode_kernel(None, spec[1], spec[2], spec[3], spec[4]).name
+	if kind == "decode_rows":
+		return recipes.attn_decode_row_scaled_kernel(None, spec[1], spec[2], spec[3], spec[4], spec[5]).name
 	if kind == "rms_norm":
 		return recipes.rms_norm_kernel(None, spec[1], spec[2]).name
 	if kind == "dequant":

@@ -128,20 +128,28 @@ def attn_decode_kernel(device: Optional[Device], n_heads: int, head_dim: int, ca
 	                        n_heads, head_dim, cache_capacity, strict)
 
 
-def attn_row_scale_operands(v_scale, out_dtype: int):
-	"""Per-head operands of the row-scaled attention kernel from the value rows' scales.
+def attn_decode_row_scaled_kernel(device: Optional[Device], n_heads: int, head_dim: int, cache_capacity: int,
+                                  out_dtype: int = BF16, strict: bool = True) -> AttnDecodeKernel:
+	"""The decode kernel over a cache of int8 codes with one scale per (row, head)."""
+	tag = "bf16" if out_dtype == BF16 else "i8"
+	return AttnDecodeKernel(device, f"attn_decode_i8_rows-h{n_heads}-hd{head_dim}-cap{cache_capacity}-o{tag}-{_mode(strict)}",
+	                        n_heads, head_dim, cache_capacity, strict, True, out_dtype)
 
-	v_scale: float32 [rows, n_heads], real v = code * v_scale.  Returns float32 arrays
-	(v_weight [rows, n_heads], sink_v_weight [n_heads], out_scale [n_heads]): each head's largest value
-	scale becomes its reference scale v_ref, a row's 8-bit probabilities are weighted by
-	v_scale / v_ref <= 1, the sink value (a FixedI8 code, real = code / 8) enters at (1 / 8) / v_ref, and
-	the result is brought back by v_ref (bf16 output, real values) or 8 * v_ref (FixedI8 output)."""
+
+def attn_row_scale_operands(v_scale, out_dtype: int):
+	"""Per-head operands of the row-scaled attention kernels from the value rows' scales.
+
+	v_scale: float32 [n_heads, rows] (prefill) or [S, n_heads, capacity] (decode caches), real v = code * v_scale.
+	Returns float32 arrays (v_weight shaped like v_scale, sink_v_weight [n_heads], out_scale [n_heads]): each
+	head's largest value scale becomes its reference scale v_ref, a row's 8-bit probabilities are weighted by
+	v_scale / v_ref <= 1, the sink value (a FixedI8 code, real = code / 8) enters at (1 / 8) / v_ref, and the
+	result is brought back by v_ref (bf16 output, real values) or 8 * v_ref (FixedI8 output)."""
 	import numpy as np
 	v_scale = np.asarray(v_scale, dtype=np.float32)
-	if v_scale.ndim != 2 or not np.all(np.isfinite(v_scale)) or not np.all(v_scale > 0):
-		raise ValueError("v_scale must be a [rows, n_heads] array of finite positive scales")
-	v_ref = v_scale.max(axis=0)
-	v_weight = (v_scale / v_ref[None, :]).astype(np.float32)
+	if v_scale.ndim not in (2, 3) or not np.all(np.isfinite(v_scale)) or not np.all(v_scale > 0):
+		raise ValueError("v_scale must be a [n_heads, rows] or [S, n_heads, capacity] array of finite positive scales")
+	v_ref = v_scale.max(axis=-1) if v_scale.ndim == 2 else v_scale.max(axis=(0, 2))
+	v_weight = (v_scale / v_ref[:, None]).astype(np.float32)
 	sink_v_weight = (np.float32(1.0 / FIXED_I8_SCALE) / v_ref).astype(np.float32)
 	if out_dtype == BF16:
 		out_scale = v_ref
