@@ -203,3 +203,52 @@ def test_config5_decode_sampled_sequences(dev):
 	                                len(heads), hd, w)
 	assert np.array_equal(_head_columns(got, heads, hd), want)
 	assert np.array_equal(got_l[:, heads].view(np.uint32), np.asarray(want_l).reshape(s, len(heads)).view(np.uint32))
+
+
+def _scales(rng, shape):
+	return (0.125 * (0.5 + rng.random(shape))).astype(np.float32)
+
+
+def test_config5_row_scaled_prefill_and_decode_sampled_heads(dev):
+	"""benchmark config 5 with one scale per (row, head) of q, k and v and bf16 output: the 65536-token
+	prefill (one head recomputed by the oracle, all queries) and the 64-sequence decode against row-scaled
+	caches with ragged lengths (three heads of every sequence)."""
+	t, h, hd, w = 65536, 32, 128, 4096
+	rng = rng_for("full-config5-rows")
+	q, kv, sk, sv, temp = _attn_inputs(rng, t, h, hd)
+	qs, ks, vs = _scales(rng, (h, t)), _scales(rng, (h, t)), _scales(rng, (h, t))
+	vw, sw, osc = recipes.attn_row_scale_operands(vs, X.BF16)
+	out = X.Tensor(dev, q.shape, X.BF16)
+	l = X.Tensor(dev, (h, t), X.F32)
+	skt, svt, tt = _up(dev, sk, X.INT8), _up(dev, sv, X.INT8), _up(dev, temp, X.F32)
+	recipes.attn_row_scaled_kernel(dev, h, hd, X.BF16, True).launch_row_scaled(
+		_up(dev, q, X.INT8), _up(dev, kv, X.INT8), skt, svt, tt, out, l, w,
+		_up(dev, qs, X.F32), _up(dev, ks, X.F32), _up(dev, vw, X.F32), _up(dev, sw, X.F32), _up(dev, osc, X.F32))
+	got, got_l = out.download(), l.download()
+	heads = [20]
+	want, want_l = S.attn_fwd_i8_row_scaled(_head_columns(q, heads, hd), _head_columns(kv, heads, 2 * hd), sk[heads], sv[heads],
+	                                        temp[heads], len(heads), hd, w, qs[heads], ks[heads], vw[heads], sw[heads], osc[heads],
+	                                        out_bf16=True)
+	assert np.array_equal(_head_columns(got, heads, hd), want)
+	assert np.array_equal(got_l[heads].view(np.uint32), want_l.view(np.uint32))
+
+	s, cap = 64, 4096
+	qd = q[:s]
+	cache = kv.reshape(t // cap, cap, 2 * h * hd)[np.arange(s) % (t // cap)]      # the prefill's kv rows, as 64 caches
+	lens = rng.integers(1, cap + 1, s).astype(np.uint32)
+	lens[:8] = [0, 1, 15, 16, 17, 4095, 4096, 2048]
+	qsd, ksd, vsd = _scales(rng, (s, h)), _scales(rng, (s, h, cap)), _scales(rng, (s, h, cap))
+	vwd, swd, oscd = recipes.attn_row_scale_operands(vsd, X.BF16)
+	outd = X.Tensor(dev, (s, h * hd), X.BF16)
+	ld = X.Tensor(dev, (s, h), X.F32)
+	recipes.attn_decode_row_scaled_kernel(dev, h, hd, cap, X.BF16, True).launch_row_scaled(
+		_up(dev, qd, X.INT8), _up(dev, cache, X.INT8), _up(dev, lens.view(np.float32), X.F32), skt, svt, tt, outd, ld, w,
+		_up(dev, qsd, X.F32), _up(dev, ksd, X.F32), _up(dev, vwd, X.F32), _up(dev, swd, X.F32), _up(dev, oscd, X.F32))
+	gotd, gotd_l = outd.download(), ld.download()
+	heads = [1, 16, 30]
+	sub_cache = np.ascontiguousarray(np.concatenate([cache[:, :, hh * 2 * hd:(hh + 1) * 2 * hd] for hh in heads], axis=2))
+	wantd, wantd_l = S.attn_decode_i8_row_scaled(
+		_head_columns(qd, heads, hd), sub_cache, lens, sk[heads], sv[heads], temp[heads], len(heads), hd, w,
+		qsd[:, heads], ksd[:, heads], vwd[:, heads], swd[heads], oscd[heads], out_bf16=True)
+	assert np.array_equal(_head_columns(gotd, heads, hd), wantd)
+	assert np.array_equal(gotd_l[:, heads].view(np.uint32), np.asarray(wantd_l).reshape(s, len(heads)).view(np.uint32))

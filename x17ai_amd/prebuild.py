@@ -74,6 +74,8 @@ def _specs():
 	add(("copy_probe",))
 	# ---- tests/test_gpu_fullsize.py (the strict ffn pair, attention and decode kernels are listed above)
 	add(("attn", 16, 128, True))
+	add(("attn_rows", 32, 128, BF16, True))
+	add(("decode_rows", 32, 128, 4096, BF16, True))
 	add(("acc_probe_full",))
 	# ---- tests/test_gpu_gemm.py: run-time dequantisation scales, bf16 out
 	for strict in (True, False):
