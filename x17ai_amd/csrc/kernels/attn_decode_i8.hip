@@ -11,7 +11,9 @@
 //
 // The work is bandwidth: every cached K byte is read exactly once, and so is every V row whose
 // 8-bit probability is not zero (rows with probability 0 contribute nothing and are not fetched).  One workgroup
-// per (sequence, head); the recurrence is cut into phases so that only two cheap scans remain
+// of two wavefronts per (sequence, head), small enough in registers and LDS that eight share a compute unit:
+// all workgroups of 64 sequences x 32 heads are then resident together and the key stream runs without a
+// second, half-empty round.  The recurrence is cut into phases so that only two cheap scans remain
 // sequential:
 //   1  scores: HD/16 lanes per key row (16-byte coalesced loads), v_dot4 + lane reduction
 //   2  per-tile max, prefix max over tiles (exact), rescale factors, probabilities, quad sums
@@ -53,8 +55,23 @@ static_assert(ROW_SCALES || !OUT_BF16, "the bf16 output needs the row-scaled bui
 constexpr f32 BASE_TEMPERATURE = ROW_SCALES ? f32(constexpr_inv_sqrt(f64(HD))) : f32(constexpr_inv_sqrt(f64(HD)) / 64.0);
 static_assert(HD == 32 || HD == 64 || HD == 128, "head_dim must be 32, 64 or 128");
 static_assert(CAP % 16 == 0, "cache capacity must be a multiple of 16");
-static_assert(dt::CHUNK_TILES * CPR == dt::THREADS_PER_BLOCK || dt::CHUNK_TILES * CPR < dt::THREADS_PER_BLOCK,
-              "one thread per (tile, 16-dim group) of a chunk");
+static_assert(dt::CHUNK_TILES * CPR == dt::THREADS_PER_BLOCK, "one thread per (tile, 16-dim group) of a chunk");
+static_assert(HD <= dt::THREADS_PER_BLOCK, "one thread per output dimension");
+
+// LDS slot of key quad `quad` (16 bytes): four f32 scores, later {partial sum, packed probabilities, free, free}
+X17_DEV u8 *quad_slot(u8 *smem, u32 quad) { return smem + 16 * quad; }
+// int32 P.V partial of (chunk tile tl, dim d): in the free half of a slot, or in a region of its own.  Word e lives
+// in slot e / 2; the slots of one 16-dim group are permuted by the group's index so that the group-wise writes of
+// a wavefront spread over the LDS banks.
+X17_DEV i32 *pv_word(u8 *smem, u32 tl, u32 d) {
+	if constexpr (dt::PV_IN_SLOTS) {
+		u32 const group = d >> 4;
+		u32 const slot = tl * (HD / 2) + 8 * group + (((d >> 1) & 7) ^ (group & 7));
+		return reinterpret_cast<i32 *>(smem + 16 * slot + 8 + 4 * (d & 1));
+	} else {
+		return reinterpret_cast<i32 *>(smem + dt::PV_OFFSET) + tl * HD + d;
+	}
+}
 }
 
 extern "C" __global__ __launch_bounds__(dt::THREADS_PER_BLOCK)
@@ -68,16 +85,12 @@ void kernel(
 #endif
 ) {
 	extern __shared__ __attribute__((aligned(16))) u8 smem[];
-	// the scores are dead once the probabilities exist, so the P.V partials of phase 4 reuse their space
-	f32 *s_score = reinterpret_cast<f32 *>(smem);                               // [CAP]
-	i32 *s_pv = reinterpret_cast<i32 *>(smem);                                   // [CHUNK_TILES][HD]
-	u8 *s_prob = smem + dt::SCORE_PV_BYTES;                                      // [CAP]
-	f32 *s_quad = reinterpret_cast<f32 *>(s_prob + CAP);                         // [CAP / 4]
-	f32 *s_tmax = s_quad + CAP / 4;                                              // [MAX_TILES]
-	f32 *s_resc = s_tmax + dt::MAX_TILES;                                        // [MAX_TILES]
-	f32 *s_mrun = s_resc + dt::MAX_TILES;                                        // [MAX_TILES]
-	f32 *s_bmax = s_mrun + dt::MAX_TILES;                                        // [256]
-	f32 *s_sum = s_bmax + 256;                                                   // [4]
+	f32 *s_score = reinterpret_cast<f32 *>(smem);                               // [CAP], quad slots (see quad_slot)
+	f32 *s_mrun = reinterpret_cast<f32 *>(smem + dt::TILE_STATE_OFFSET);         // [MAX_TILES] tile max, then running max
+	f32 *s_tmax = s_mrun;
+	f32 *s_resc = s_mrun + dt::MAX_TILES;                                        // [MAX_TILES]
+	f32 *s_bmax = s_resc + dt::MAX_TILES;                                        // [4] one per wavefront
+	f32 *s_sum = s_bmax + 4;                                                     // [4]
 	u32 *s_nact = reinterpret_cast<u32 *>(s_sum + 4);                            // [4] (one used)
 	u16 *s_act = reinterpret_cast<u16 *>(s_nact + 4);                            // [MAX_TILES] tiles that move O
 
@@ -119,19 +132,21 @@ void kernel(
 	// ---- phase 1: scores of all keys of the walked tiles.  A thread keeps BATCH independent 16-byte
 	// loads in flight (a load per pass would leave the kernel waiting on memory latency).
 	u32 const n_keys = n_tiles * 16;
-	constexpr u32 BATCH = 8;
+	// Few loads per thread and many resident workgroups: the workgroups of one sequence then walk its rows nearly
+	// in step, which the DRAM pages like (measured: 2 loads in flight per thread beat 1, 4, 8 and 16).
+#ifndef X17_DECODE_BATCH
+#define X17_DECODE_BATCH 2
+#endif
+	constexpr u32 BATCH = X17_DECODE_BATCH;
 	for (u32 base = 0; base < n_keys; base += KEYS_PER_PASS * BATCH) {
 		v4i kc[BATCH];
-		[[maybe_unused]] f32 ksc[BATCH];
 		X17_UNROLL for (u32 bb = 0; bb < BATCH; ++bb) {
 			u32 kidx = base + bb * KEYS_PER_PASS + tid / CPR;
 			u32 j = t0 * 16 + kidx;
 			bool vis = kidx < n_keys && j >= j_lo && j < pos;
 			u32 j_safe = vis ? j : pos - 1;                   // a row that exists (n_tiles > 0 means pos >= 1)
-			kc[bb] = *reinterpret_cast<v4i const *>(kv_head + (size_t)j_safe * ROW + 16 * c);
-#if X17_ATTN_ROW_SCALES
-			ksc[bb] = k_scale_head[j_safe];
-#endif
+			// every cache byte is read once: streaming (non-temporal) loads
+			kc[bb] = __builtin_nontemporal_load(reinterpret_cast<v4i const *>(kv_head + (size_t)j_safe * ROW + 16 * c));
 		}
 		X17_UNROLL for (u32 bb = 0; bb < BATCH; ++bb) {
 			u32 kidx = base + bb * KEYS_PER_PASS + tid / CPR;
@@ -142,12 +157,23 @@ void kernel(
 			X17_UNROLL for (int w = 0; w < 4; ++w) dot = __builtin_amdgcn_sdot4(qc[w], kc[bb][w], dot, false);
 			X17_UNROLL for (u32 mask = 1; mask < CPR; mask <<= 1) dot += __shfl_xor(dot, (int)mask, 64);
 			if (in_range && c == 0) {
-				f32 const score = ROW_SCALES ? (f32(dot) * ksc[bb]) * temperature : f32(dot) * temperature;
+				// (row-scaled build: the key's scale and the temperature are applied in a pass of their own below)
+				f32 const score = ROW_SCALES ? f32(dot) : f32(dot) * temperature;
 				s_score[kidx] = vis ? score : -__builtin_inff();
 			}
 		}
 	}
 	__syncthreads();
+#if X17_ATTN_ROW_SCALES
+	// the keys' scales, four per 16-byte load; masked keys keep -inf whatever their (possibly never written) scale
+	for (u32 quad = tid; quad < n_tiles * 4; quad += dt::THREADS_PER_BLOCK) {
+		v4f const ks = __builtin_nontemporal_load(reinterpret_cast<v4f const *>(k_scale_head + t0 * 16 + quad * 4));
+		v4f sc = *reinterpret_cast<v4f const *>(s_score + quad * 4);
+		X17_UNROLL for (int i = 0; i < 4; ++i) sc[i] = sc[i] == -__builtin_inff() ? sc[i] : (sc[i] * ks[i]) * temperature;
+		*reinterpret_cast<v4f *>(s_score + quad * 4) = sc;
+	}
+	__syncthreads();
+#endif
 
 	// ---- phase 2a: per-tile max; each thread owns TPT consecutive tiles
 	constexpr u32 TPT = (dt::MAX_TILES + dt::THREADS_PER_BLOCK - 1) / dt::THREADS_PER_BLOCK;
@@ -207,13 +233,13 @@ void kernel(
 		f32 p1 = sfu::ex2(s[1] - m) * 255.0f;
 		f32 p2 = sfu::ex2(s[2] - m) * 255.0f;
 		f32 p3 = sfu::ex2(s[3] - m) * 255.0f;
-		s_quad[quad] = (p0 + p1) + (p2 + p3);
+		f32 const quad_sum = (p0 + p1) + (p2 + p3);
 #if X17_ATTN_ROW_SCALES
 		{
 			// the numerator takes the probabilities at the value rows' relative scales; masked keys keep 0
 			u32 const j = t0 * 16 + quad * 4;
 			// (rows of a partly visible quad are inside the cache: its capacity is a multiple of 16)
-			v4f const vw = *reinterpret_cast<v4f const *>(v_weight_head + j);
+			v4f const vw = __builtin_nontemporal_load(reinterpret_cast<v4f const *>(v_weight_head + j));
 			p0 = s[0] == -__builtin_inff() ? 0.0f : p0 * vw[0];
 			p1 = s[1] == -__builtin_inff() ? 0.0f : p1 * vw[1];
 			p2 = s[2] == -__builtin_inff() ? 0.0f : p2 * vw[2];
@@ -222,23 +248,36 @@ void kernel(
 #endif
 		u32 packed = (u32)(i32)__builtin_rintf(p0) | ((u32)(i32)__builtin_rintf(p1) << 8)
 			| ((u32)(i32)__builtin_rintf(p2) << 16) | ((u32)(i32)__builtin_rintf(p3) << 24);
-		*reinterpret_cast<u32 *>(s_prob + quad * 4) = packed;
+		// in place: this thread has read its quad's scores, nobody else touches the slot
+		*reinterpret_cast<v2u *>(quad_slot(smem, quad)) = v2u{f2u(quad_sum), packed};
 	}
 	__syncthreads();
 
-	// ---- phase 3: the four partial-sum chains (operands fetched eight tiles at a time, so the chain
-	// itself is the only serial part)
-	if (tid < 4) {
-		f32 sum = 63.75f;
-		u32 t = 0;
-		for (; t + 8 <= n_tiles; t += 8) {
+	// ---- phase 3: the four partial-sum chains, one per lane of the first four.  The operands of the next eight
+	// tiles are fetched while the current eight are chained, so the chain itself is the only serial part.  It runs
+	// further down, while the first value rows of phase 4 are on their way.
+	auto sum_chains = [&]() {
+		if (tid < 4) {
+			f32 sum = 63.75f;
 			f32 r[8], a[8];
-			X17_UNROLL for (int i = 0; i < 8; ++i) { r[i] = s_resc[t + i]; a[i] = s_quad[(t + i) * 4 + tid]; }
-			X17_UNROLL for (int i = 0; i < 8; ++i) sum = fmaf32(sum, r[i], a[i]);
+			auto fetch = [&](u32 t) {
+				X17_UNROLL for (int i = 0; i < 8; ++i) {
+					r[i] = s_resc[t + i];
+					a[i] = *reinterpret_cast<f32 const *>(quad_slot(smem, (t + i) * 4 + tid));
+				}
+			};
+			u32 t = 0;
+			if (n_tiles >= 8) fetch(0);
+			for (; t + 8 <= n_tiles; t += 8) {
+				f32 rc[8], ac[8];
+				X17_UNROLL for (int i = 0; i < 8; ++i) { rc[i] = r[i]; ac[i] = a[i]; }
+				if (t + 16 <= n_tiles) fetch(t + 8);
+				X17_UNROLL for (int i = 0; i < 8; ++i) sum = fmaf32(sum, rc[i], ac[i]);
+			}
+			for (; t < n_tiles; ++t) sum = fmaf32(sum, s_resc[t], *reinterpret_cast<f32 const *>(quad_slot(smem, t * 4 + tid)));
+			s_sum[tid] = sum;
 		}
-		for (; t < n_tiles; ++t) sum = fmaf32(sum, s_resc[t], s_quad[t * 4 + tid]);
-		s_sum[tid] = sum;
-	}
+	};
 
 	// ---- phase 4: O chains.  Lane d < HD owns output dim d.
 	// A tile whose sixteen probabilities all rounded to zero and whose rescale factor is exactly 1 leaves O
@@ -251,8 +290,9 @@ void kernel(
 			u32 t = base + lane;
 			bool active = false;
 			if (t < n_tiles) {
-				v4u probs = *reinterpret_cast<v4u const *>(s_prob + t * 16);
-				active = (probs[0] | probs[1] | probs[2] | probs[3]) != 0 || s_resc[t] != 1.0f;
+				u32 any = 0;
+				X17_UNROLL for (u32 k = 0; k < 4; ++k) any |= *reinterpret_cast<u32 const *>(quad_slot(smem, t * 4 + k) + 4);
+				active = any != 0 || s_resc[t] != 1.0f;
 			}
 			unsigned long long const mask = __ballot(active);
 			if (active) {
@@ -278,22 +318,28 @@ void kernel(
 		u32 const tiles_here = n_act - chunk < dt::CHUNK_TILES ? n_act - chunk : dt::CHUNK_TILES;
 		// 4a: int32 P.V of one tile x 16 dims per thread
 		u32 const tl = tid / CPR;
+		u32 probs[4] = {0, 0, 0, 0};
+		v4i vv[16];
 		if (tl < tiles_here) {
 			u32 const t = s_act[chunk + tl];
-			i32 acc[16];
-			X17_UNROLL for (int i = 0; i < 16; ++i) acc[i] = 0;
-			v4u probs = *reinterpret_cast<v4u const *>(s_prob + t * 16);
+			X17_UNROLL for (u32 k = 0; k < 4; ++k) probs[k] = *reinterpret_cast<u32 const *>(quad_slot(smem, t * 4 + k) + 4);
 			// all loads of the tile first (only rows with a nonzero probability are fetched: masked keys have
 			// p == 0 and may lie outside the cache), then the arithmetic
-			v4i vv[16];
 			X17_UNROLL for (int k = 0; k < 16; ++k) {
 				u32 p = (probs[k / 4] >> (8 * (k % 4))) & 0xFFu;
 				u32 j = (t0 + t) * 16 + k;
 				vv[k] = v4i{0, 0, 0, 0};
 				if (p != 0) {
-					vv[k] = *reinterpret_cast<v4i const *>(kv_head + (size_t)j * ROW + HD + 16 * c);
+					vv[k] = __builtin_nontemporal_load(reinterpret_cast<v4i const *>(kv_head + (size_t)j * ROW + HD + 16 * c));
 				}
 			}
+		}
+		if (chunk == 0) {
+			sum_chains();          // while the value rows are in flight
+		}
+		if (tl < tiles_here) {
+			i32 acc[16];
+			X17_UNROLL for (int i = 0; i < 16; ++i) acc[i] = 0;
 			X17_UNROLL for (int k = 0; k < 16; ++k) {
 				i32 p = (i32)((probs[k / 4] >> (8 * (k % 4))) & 0xFFu);
 				if (p != 0) {     // after the 8-bit quantisation most keys far below the maximum carry no weight
@@ -302,8 +348,8 @@ void kernel(
 					}
 				}
 			}
-			X17_UNROLL for (int i = 0; i < 16; i += 4) {
-				*reinterpret_cast<v4i *>(s_pv + tl * HD + 16 * c + i) = v4i{acc[i], acc[i + 1], acc[i + 2], acc[i + 3]};
+			X17_UNROLL for (int i = 0; i < 16; i += 2) {
+				*reinterpret_cast<v2i *>(pv_word(smem, tl, 16 * c + i)) = v2i{acc[i], acc[i + 1]};
 			}
 		}
 		__syncthreads();
@@ -313,7 +359,7 @@ void kernel(
 			for (; tl2 + 8 <= tiles_here; tl2 += 8) {
 				f32 r[8];
 				i32 a[8];
-				X17_UNROLL for (int i = 0; i < 8; ++i) { r[i] = s_resc[s_act[chunk + tl2 + i]]; a[i] = s_pv[(tl2 + i) * HD + tid]; }
+				X17_UNROLL for (int i = 0; i < 8; ++i) { r[i] = s_resc[s_act[chunk + tl2 + i]]; a[i] = *pv_word(smem, tl2 + i, tid); }
 				X17_UNROLL for (int i = 0; i < 8; ++i) {
 					o = o * r[i];
 					o = o + f32(a[i]);
@@ -321,10 +367,14 @@ void kernel(
 			}
 			for (; tl2 < tiles_here; ++tl2) {
 				o = o * s_resc[s_act[chunk + tl2]];
-				o = o + f32(s_pv[tl2 * HD + tid]);
+				o = o + f32(*pv_word(smem, tl2, tid));
 			}
 		}
 		__syncthreads();
+	}
+
+	if (n_act == 0) {
+		sum_chains();
 	}
 
 	// ---- finish (:293-351)
