@@ -253,31 +253,23 @@ void kernel(
 	}
 	__syncthreads();
 
-	// ---- phase 3: the four partial-sum chains, one per lane of the first four.  The operands of the next eight
-	// tiles are fetched while the current eight are chained, so the chain itself is the only serial part.  It runs
-	// further down, while the first value rows of phase 4 are on their way.
-	auto sum_chains = [&]() {
-		if (tid < 4) {
-			f32 sum = 63.75f;
-			f32 r[8], a[8];
-			auto fetch = [&](u32 t) {
-				X17_UNROLL for (int i = 0; i < 8; ++i) {
-					r[i] = s_resc[t + i];
-					a[i] = *reinterpret_cast<f32 const *>(quad_slot(smem, (t + i) * 4 + tid));
-				}
-			};
-			u32 t = 0;
-			if (n_tiles >= 8) fetch(0);
-			for (; t + 8 <= n_tiles; t += 8) {
-				f32 rc[8], ac[8];
-				X17_UNROLL for (int i = 0; i < 8; ++i) { rc[i] = r[i]; ac[i] = a[i]; }
-				if (t + 16 <= n_tiles) fetch(t + 8);
-				X17_UNROLL for (int i = 0; i < 8; ++i) sum = fmaf32(sum, rc[i], ac[i]);
-			}
-			for (; t < n_tiles; ++t) sum = fmaf32(sum, s_resc[t], *reinterpret_cast<f32 const *>(quad_slot(smem, t * 4 + tid)));
-			s_sum[tid] = sum;
+	// ---- phase 3: the four partial-sum chains, one per lane of the first four, while the last wavefront lists the
+	// tiles for phase 4.  The chain is serial; what costs time is fetching its operands from LDS, so they are
+	// fetched 32 tiles at a time (the registers are free at this point) and the chain waits once per 32 steps.
+	if (tid < 4) {
+		constexpr u32 STEPS = 32;
+		f32 sum = 63.75f;
+		u32 t = 0;
+		for (; t + STEPS <= n_tiles; t += STEPS) {
+			v4f r[STEPS / 4];
+			f32 a[STEPS];
+			X17_UNROLL for (u32 i = 0; i < STEPS / 4; ++i) r[i] = *reinterpret_cast<v4f const *>(s_resc + t + 4 * i);
+			X17_UNROLL for (u32 i = 0; i < STEPS; ++i) a[i] = *reinterpret_cast<f32 const *>(quad_slot(smem, (t + i) * 4 + tid));
+			X17_UNROLL for (u32 i = 0; i < STEPS; ++i) sum = fmaf32(sum, r[i / 4][i % 4], a[i]);
 		}
-	};
+		for (; t < n_tiles; ++t) sum = fmaf32(sum, s_resc[t], *reinterpret_cast<f32 const *>(quad_slot(smem, t * 4 + tid)));
+		s_sum[tid] = sum;
+	}
 
 	// ---- phase 4: O chains.  Lane d < HD owns output dim d.
 	// A tile whose sixteen probabilities all rounded to zero and whose rescale factor is exactly 1 leaves O
@@ -314,17 +306,17 @@ void kernel(
 		o = o * sink_v_weight[head];
 #endif
 	}
-	for (u32 chunk = 0; chunk < n_act; chunk += dt::CHUNK_TILES) {
+	// 4a: int32 P.V of one tile x 16 dims per thread.  The value rows of a chunk are requested (only rows with a
+	// nonzero probability: masked keys have p == 0 and may lie outside the cache) while the previous chunk's chain
+	// runs, so that a workgroup with many listed tiles waits for memory once, not once per chunk.
+	u32 const tl = tid / CPR;
+	u32 probs[4] = {0, 0, 0, 0};
+	v4i vv[16];
+	auto request_rows = [&](u32 chunk) {
 		u32 const tiles_here = n_act - chunk < dt::CHUNK_TILES ? n_act - chunk : dt::CHUNK_TILES;
-		// 4a: int32 P.V of one tile x 16 dims per thread
-		u32 const tl = tid / CPR;
-		u32 probs[4] = {0, 0, 0, 0};
-		v4i vv[16];
 		if (tl < tiles_here) {
 			u32 const t = s_act[chunk + tl];
 			X17_UNROLL for (u32 k = 0; k < 4; ++k) probs[k] = *reinterpret_cast<u32 const *>(quad_slot(smem, t * 4 + k) + 4);
-			// all loads of the tile first (only rows with a nonzero probability are fetched: masked keys have
-			// p == 0 and may lie outside the cache), then the arithmetic
 			X17_UNROLL for (int k = 0; k < 16; ++k) {
 				u32 p = (probs[k / 4] >> (8 * (k % 4))) & 0xFFu;
 				u32 j = (t0 + t) * 16 + k;
@@ -334,9 +326,12 @@ void kernel(
 				}
 			}
 		}
-		if (chunk == 0) {
-			sum_chains();          // while the value rows are in flight
-		}
+	};
+	if (n_act > 0) {
+		request_rows(0);
+	}
+	for (u32 chunk = 0; chunk < n_act; chunk += dt::CHUNK_TILES) {
+		u32 const tiles_here = n_act - chunk < dt::CHUNK_TILES ? n_act - chunk : dt::CHUNK_TILES;
 		if (tl < tiles_here) {
 			i32 acc[16];
 			X17_UNROLL for (int i = 0; i < 16; ++i) acc[i] = 0;
@@ -353,6 +348,9 @@ void kernel(
 			}
 		}
 		__syncthreads();
+		if (chunk + dt::CHUNK_TILES < n_act) {
+			request_rows(chunk + dt::CHUNK_TILES);
+		}
 		// 4b: one f32 multiply (rescale) and one f32 add per tile (:247-252, :588-605)
 		if (tid < HD) {
 			u32 tl2 = 0;
@@ -371,10 +369,6 @@ void kernel(
 			}
 		}
 		__syncthreads();
-	}
-
-	if (n_act == 0) {
-		sum_chains();
 	}
 
 	// ---- finish (:293-351)
