@@ -77,6 +77,12 @@ def _specs():
 	add(("attn_rows", 32, 128, BF16, True))
 	add(("decode_rows", 32, 128, 4096, BF16, True))
 	add(("acc_probe_full",))
+	# ---- tests/test_gpu_refconfig.py: the reference's own configuration (64 heads of 32, widths 2048)
+	add(("attn_kv", 2048, 4096, 32))
+	add(("attn", 64, 32, True))
+	add(("attn_y", 2048, 2048, True, E4M3))
+	add(("ffn_f", 2048, 4096, True, E4M3))
+	add(("ffn_y", 2048, 2048, True, E4M3, INT8))
 	# ---- tests/test_gpu_gemm.py: run-time dequantisation scales, bf16 out
 	for strict in (True, False):
 		add(("dequant", 1024, 512, INT8, INT8, False, strict))
