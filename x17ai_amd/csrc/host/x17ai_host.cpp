@@ -734,6 +734,13 @@ std::unique_ptr<GemmKernel> GemmKernel::create(std::shared_ptr<HipDevice> device
 	common << "#define X17_EPILOGUE " << kind << "\n";
 	common << "#define X17_STORE " << (g.c_dtype == DType::E4m3 ? 1 : (g.c_dtype == DType::Bf16 ? 2 : 0)) << "\n";
 	common << "#define X17_STRICT_MATH " << (strict_math ? 1 : 0) << "\n";
+	// e4m3 activations x int8 weights run on the f16 matrix cores with both operands widened in registers, and
+	// widening an int8 byte costs 2.5 times what an e4m3 byte costs.  A weight row is widened by every wave that
+	// shares it, so these kernels use waves of 128 tokens x 64 columns (two waves per weight row, four per
+	// token row) instead of 64 x 128.  (Scale, GeGLU and Residual writers; the others are written for 128 columns.)
+	if (g.a.dtype == DType::E4m3 && g.b.dtype == DType::Int8 && kind <= 2) {
+		common << "#define X17_GEMM_WAVES_M 2\n#define X17_GEMM_WAVES_N 4\n";
+	}
 
 	auto finite_pos = [](double v) { return std::isfinite(v) && v > 0.0; };
 	size_t head_dim = 0, sep_dim = 0;

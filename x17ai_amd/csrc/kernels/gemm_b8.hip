@@ -76,16 +76,19 @@ constexpr u32 UNITS = ROWS_PER_WAVE / 8;                    // 8-row direct-to-L
 using Acc = __attribute__((ext_vector_type(16))) int;       // raw 16 registers; reinterpreted as f32 when ACC_F32
 
 // ------------------------------------------------------------------ epilogues
-// Each receives, for ONE token row, 64 accumulators of 64 consecutive raw columns starting at
-// raw column `n`, already converted to f32 (i32 -> f32 is the reference's implicit RNE cast).
+// Each receives, for ONE token row, the accumulators of LANE_COLS (64, or 32 for 64-column waves)
+// consecutive raw columns starting at raw column `n`, already converted to f32 (i32 -> f32 is the
+// reference's implicit RNE cast).
+constexpr int BN = gt::WAVE_N / 32;                         // 32-column MFMA blocks per wave
+constexpr int LANE_COLS = 16 * BN;                          // consecutive raw columns a lane ends up with
 
 // ScaledMatrixWriter, cuda/gemm_b8.cuh:291-339
 struct ScaleEpilogue {
 	static constexpr f64 SCALE = f64(X17_INP_SCALE) * f64(X17_OUT_SCALE);
 	static constexpr u32 OUT_COLS = N_RAW;
-	X17_DEV static void run(f32 const (&x)[64], u8 *c, u32 row, u32 n, void const *) {
+	X17_DEV static void run(f32 const (&x)[LANE_COLS], u8 *c, u32 row, u32 n, void const *) {
 		u8 *dst = c + (size_t)row * OUT_COLS + n;
-		X17_UNROLL for (int v = 0; v < 4; ++v) {
+		X17_UNROLL for (int v = 0; v < LANE_COLS / 16; ++v) {
 			v4u pack;
 			X17_UNROLL for (int w = 0; w < 4; ++w) {
 				f32 y[4];
@@ -130,9 +133,9 @@ struct GeGluEpilogue {
 			return (g * v) * hw::rcp(d);
 		}
 	}
-	X17_DEV static void run(f32 const (&x)[64], u8 *c, u32 row, u32 n, void const *) {
+	X17_DEV static void run(f32 const (&x)[LANE_COLS], u8 *c, u32 row, u32 n, void const *) {
 		u8 *dst = c + (size_t)row * OUT_COLS + n / 2;
-		X17_UNROLL for (int v = 0; v < 2; ++v) {
+		X17_UNROLL for (int v = 0; v < LANE_COLS / 32; ++v) {
 			v4u pack;
 			X17_UNROLL for (int w = 0; w < 4; ++w) {
 				f32 y[4];
@@ -170,11 +173,11 @@ struct ResidualEpilogue {
 		f32 new_w = fmaf32(sfu::lg2(1.0f + sfu::ex2(-__builtin_fabsf(g * SP_INP_SCALE))), SP_OUT_SCALE, line);
 		return fmaf32(new_w, v, old_w * r);
 	}
-	X17_DEV static void run(f32 const (&x)[64], u8 *c, u32 row, u32 n, void const *extra) {
+	X17_DEV static void run(f32 const (&x)[LANE_COLS], u8 *c, u32 row, u32 n, void const *extra) {
 		size_t off = (size_t)row * OUT_COLS + n / 2;
 		i8 const *res = reinterpret_cast<i8 const *>(extra) + off;
 		u8 *dst = c + off;
-		X17_UNROLL for (int v = 0; v < 2; ++v) {
+		X17_UNROLL for (int v = 0; v < LANE_COLS / 32; ++v) {
 			v4u rv = *reinterpret_cast<v4u const *>(res + 16 * v);
 			v4u pack;
 			X17_UNROLL for (int w = 0; w < 4; ++w) {
@@ -196,6 +199,7 @@ struct ResidualEpilogue {
 // run-time-scale superset for symmetric per-row / per-channel int8 quantisation (bf16 store precedent:
 // cuda/gemm_b16.cuh:264-294).  t = (x * row_scale) * col_scale, two f32 multiplies in that order.
 #if X17_EPILOGUE == 4
+static_assert(LANE_COLS == 64, "the dequantising writer is written for 128-column waves");
 struct DequantEpilogue {
 	static constexpr bool GEGLU = X17_DEQ_GEGLU != 0;
 	static constexpr u32 OUT_COLS = GEGLU ? N_RAW / 2 : N_RAW;
@@ -235,6 +239,7 @@ struct DequantEpilogue {
 
 // The l2norm epilogue needs more than one lane for head_dim > 64 and is handled in the kernel body.
 #if X17_EPILOGUE == 3
+static_assert(LANE_COLS == 64, "the l2norm writer is written for 128-column waves");
 constexpr u32 HEAD_DIM = X17_HEAD_DIM;
 static_assert(HEAD_DIM == 32 || HEAD_DIM == 64 || HEAD_DIM == 128, "head_dim must be 32, 64 or 128");
 #endif
@@ -265,9 +270,10 @@ struct LaneOffsets {
 // Direct-to-LDS load `i` (0 .. LOADS_PER_STAGE-1) of this wave's share of one stage: first the token
 // units, then the weight units.  Wave w copies token rows [X_UNITS * UNIT_ROWS * w, +X_UNITS * UNIT_ROWS)
 // and as many LDS weight rows.
-// LDS weight row R = 128*wn + 32*bn + i holds weight row 128*wn + 64*((i/4)%2) + 16*bn + 4*(i/8) + i%4:
-// the MFMA hands output row i = 8*(r/4) + 4*(lane/32) + r%4 to register r, so a lane collects columns
-// 64*(lane/32) + 16*bn + r.  For the rows of one load unit the lane-dependent part is constant.
+// With WN = WAVE_N columns per wave, LDS weight row R = WN*wn + 32*bn + i holds weight row
+// WN*wn + (WN/2)*((i/4)%2) + 16*bn + 4*(i/8) + i%4: the MFMA hands output row i = 8*(r/4) + 4*(lane/32) + r%4
+// to register r, so a lane collects columns (WN/2)*(lane/32) + 16*bn + r.  For the rows of one load unit the
+// lane-dependent part is constant.
 template <u32 I>
 X17_DEV void issue_stage_load(
 	u8 const *a_tile, u8 const *b_tile, u8 *stage, u32 k0, u32 wave, LaneOffsets const &lo
@@ -280,7 +286,7 @@ X17_DEV void issue_stage_load(
 	} else {
 		constexpr u32 u = I - X_UNITS;
 		u32 r0 = (wave * W_UNITS + u) * UNIT_ROWS;
-		u32 n_uniform = 128 * (r0 / 128) + 16 * ((r0 % 128) / 32) + 4 * ((r0 % 32) / 8);
+		u32 n_uniform = gt::WAVE_N * (r0 / gt::WAVE_N) + 16 * ((r0 % gt::WAVE_N) / 32) + 4 * ((r0 % 32) / 8);
 		u8 *w_lds = stage + X_TILE_BYTES + r0 * ROW_BYTES;
 		u8 const *w_src = b_tile + (size_t)n_uniform * K_TOTAL + k0;
 		__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(w_src + lo.w_src[u & 1]), X17_LDS_PTR(w_lds), 16, 0, 0);
@@ -352,28 +358,28 @@ constexpr u32 CHUNKS_PER_FRAG = SLICE_BYTES / 32;           // 16-byte chunks a 
 static_assert(SLICES % 2 == 0, "the fragment double buffer needs an even number of slices per step");
 
 struct Frags {
-	v4i w[4][CHUNKS_PER_FRAG];
+	v4i w[BN][CHUNKS_PER_FRAG];
 	v4i x[BM][CHUNKS_PER_FRAG];
 };
 
 X17_DEV void load_frags(Frags &f, u8 const *w_tile, u8 const *x_tile, u32 s, LaneOffsets const &lo) {
 	X17_UNROLL for (u32 c = 0; c < CHUNKS_PER_FRAG; ++c) {
 		u32 kc = CHUNKS_PER_FRAG * (2 * s + lo.half) + c;
-		X17_UNROLL for (int bn = 0; bn < 4; ++bn) f.w[bn][c] = lds_chunk(w_tile, bn * 32 * ROW_BYTES, kc, lo.swz);
+		X17_UNROLL for (int bn = 0; bn < BN; ++bn) f.w[bn][c] = lds_chunk(w_tile, bn * 32 * ROW_BYTES, kc, lo.swz);
 		X17_UNROLL for (int bm = 0; bm < BM; ++bm) f.x[bm][c] = lds_chunk(x_tile, bm * 32 * ROW_BYTES, kc, lo.swz);
 	}
 }
 
-X17_DEV void mma_slice(Frags const &f, Acc (&acc)[4][BM]) {
+X17_DEV void mma_slice(Frags const &f, Acc (&acc)[BN][BM]) {
 	if constexpr (MMA == 0) {
-		X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
+		X17_UNROLL for (int bn = 0; bn < BN; ++bn) {
 			X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
 				acc[bn][bm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w[bn][0], f.x[bm][0], acc[bn][bm], 0, 0, 0);
 			}
 		}
 	} else if constexpr (MMA == 1) {
-		v8i wf[4], xf[BM];
-		X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
+		v8i wf[BN], xf[BM];
+		X17_UNROLL for (int bn = 0; bn < BN; ++bn) {
 			v4i l = f.w[bn][0], h = f.w[bn][CHUNKS_PER_FRAG - 1];
 			wf[bn] = v8i{l[0], l[1], l[2], l[3], h[0], h[1], h[2], h[3]};
 		}
@@ -381,7 +387,7 @@ X17_DEV void mma_slice(Frags const &f, Acc (&acc)[4][BM]) {
 			v4i l = f.x[bm][0], h = f.x[bm][CHUNKS_PER_FRAG - 1];
 			xf[bm] = v8i{l[0], l[1], l[2], l[3], h[0], h[1], h[2], h[3]};
 		}
-		X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
+		X17_UNROLL for (int bn = 0; bn < BN; ++bn) {
 			X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
 				v16f r = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
 					wf[bn], xf[bm], __builtin_bit_cast(v16f, acc[bn][bm]), 0, 0, 0, 0, 0, 0);
@@ -390,10 +396,10 @@ X17_DEV void mma_slice(Frags const &f, Acc (&acc)[4][BM]) {
 		}
 	} else {
 		X17_UNROLL for (int h = 0; h < 2; ++h) {                // two f16 MFMAs of K = 16
-			v8h wf[4], xf[BM];
-			X17_UNROLL for (int bn = 0; bn < 4; ++bn) wf[bn] = widen8(f.w[bn][0][2 * h], f.w[bn][0][2 * h + 1], B_KIND);
+			v8h wf[BN], xf[BM];
+			X17_UNROLL for (int bn = 0; bn < BN; ++bn) wf[bn] = widen8(f.w[bn][0][2 * h], f.w[bn][0][2 * h + 1], B_KIND);
 			X17_UNROLL for (int bm = 0; bm < BM; ++bm) xf[bm] = widen8(f.x[bm][0][2 * h], f.x[bm][0][2 * h + 1], A_KIND);
-			X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
+			X17_UNROLL for (int bn = 0; bn < BN; ++bn) {
 				X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
 					v16f r = __builtin_amdgcn_mfma_f32_32x32x16_f16(
 						wf[bn], xf[bm], __builtin_bit_cast(v16f, acc[bn][bm]), 0, 0, 0);
@@ -411,8 +417,8 @@ X17_DEV void mma_slice(Frags const &f, Acc (&acc)[4][BM]) {
 template <u32 N_LOADS>
 X17_DEV void interleave_slice(bool with_reads) {
 	if constexpr (MMA != 2) {
-		constexpr int READS = (4 + BM) * CHUNKS_PER_FRAG;
-		constexpr int MFMAS = 4 * BM;
+		constexpr int READS = (BN + BM) * CHUNKS_PER_FRAG;
+		constexpr int MFMAS = BN * BM;
 		constexpr int GROUPS = MFMAS < READS ? MFMAS : READS;
 		if (with_reads) {
 			X17_UNROLL for (int i = 0; i < GROUPS; ++i) {
@@ -490,7 +496,7 @@ void kernel(
 			u32 key = ((odd * UNIT_ROWS + j) >> SWZ_SHIFT) & (CHUNKS - 1);
 			u32 chunk = p ^ key;
 			lo.x_src[odd] = j * K_TOTAL + 16 * chunk;
-			lo.w_src[odd] = (64 * ((j >> 2) & 1) + 4 * (j >> 3) + (j & 3)) * K_TOTAL + 16 * chunk;
+			lo.w_src[odd] = ((gt::WAVE_N / 2) * ((j >> 2) & 1) + 4 * (j >> 3) + (j & 3)) * K_TOTAL + 16 * chunk;
 		}
 		lo.frag_row = (lane % 32) * ROW_BYTES;
 		lo.half = lane / 32;
@@ -508,7 +514,7 @@ void kernel(
 	constexpr bool CROSS_TILE = K_STEPS >= gt::STAGES;
 	constexpr u32 PROLOGUE_STAGES = CROSS_TILE ? gt::STAGES : K_STEPS;
 	u32 const x_off = wm * gt::WAVE_M * ROW_BYTES + lo.frag_row;
-	u32 const w_off = X_TILE_BYTES + wn * 128 * ROW_BYTES + lo.frag_row;
+	u32 const w_off = X_TILE_BYTES + wn * gt::WAVE_N * ROW_BYTES + lo.frag_row;
 
 	u32 tile_m, tile_n;
 	tile_coords(group, tile_m, tile_n);
@@ -547,8 +553,8 @@ void kernel(
 			}
 		}
 
-		Acc acc[4][BM];   // [bn][bm]
-		X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
+		Acc acc[BN][BM];   // [bn][bm]
+		X17_UNROLL for (int bn = 0; bn < BN; ++bn) {
 			X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
 				X17_UNROLL for (int r = 0; r < 16; ++r) acc[bn][bm][r] = 0;
 			}
@@ -603,14 +609,14 @@ void kernel(
 		}
 
 	// ---- epilogue.  Lane owns token (32*bm + lane%32) of its wave and raw columns
-	// 64*(lane/32) + 16*bn + r of its wave, r = accumulator register index.
+	// LANE_COLS*(lane/32) + 16*bn + r of its wave, r = accumulator register index.
 	u32 const row0 = tile_m * gt::M_PER_BLOCK + wm * gt::WAVE_M + lane % 32;
-	u32 const n0 = tile_n * gt::N_PER_BLOCK + wn * 128 + 64 * lo.half;
+	u32 const n0 = tile_n * gt::N_PER_BLOCK + wn * gt::WAVE_N + LANE_COLS * lo.half;
 
 	X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
 		u32 row = row0 + 32 * bm;
-		f32 x[64];
-		X17_UNROLL for (int bn = 0; bn < 4; ++bn) {
+		f32 x[LANE_COLS];
+		X17_UNROLL for (int bn = 0; bn < BN; ++bn) {
 			// (bit-casting a single vector element in place reads element 0; cast the whole vector first)
 			v16f const as_f32 = __builtin_bit_cast(v16f, acc[bn][bm]);
 			X17_UNROLL for (int r = 0; r < 16; ++r) {
