@@ -131,7 +131,9 @@ def test_attn_launch_rejects_bad_arguments(dev):
 
 # ---------------------------------------------------------------- decode
 
-@pytest.mark.parametrize("h,hd,cap,w", [(4, 32, 256, 0), (4, 64, 256, 64), (2, 128, 512, 128), (2, 128, 512, 0)])
+# (the last two cases have a cache large enough for the P.V partials to live in the free halves of the LDS slots)
+@pytest.mark.parametrize("h,hd,cap,w", [(4, 32, 256, 0), (4, 64, 256, 64), (2, 128, 512, 128), (2, 128, 512, 0),
+                                        (2, 32, 4096, 0), (2, 64, 4096, 2048)])
 def test_decode_bit_exact_and_equals_prefill_row(dev, h, hd, cap, w):
 	s = 6
 	rng = rng_for("decode", h, hd, cap, w)

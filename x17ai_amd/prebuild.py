@@ -44,7 +44,7 @@ def _specs():
 		add(("attn_rows", h, hd, out, True))
 	for h, hd in ((8, 64), (2, 128)):
 		add(("attn_rows", h, hd, BF16, False))
-	for h, hd, cap in ((4, 32, 256), (4, 64, 256), (2, 128, 512)):
+	for h, hd, cap in ((4, 32, 256), (4, 64, 256), (2, 128, 512), (2, 32, 4096), (2, 64, 4096)):
 		add(("decode", h, hd, cap, True))
 	for h, hd, cap, out in ((4, 64, 256, BF16), (2, 128, 512, BF16), (4, 32, 256, INT8)):
 		add(("decode_rows", h, hd, cap, out, True))
