@@ -7,17 +7,18 @@
 //
 // Design, MI355X-first (nothing here is derived from the SM80 kernel):
 //   * One workgroup = a 256 (tokens) x 256 (raw columns) output tile, by default 8 wavefronts of
-//     64 x 128 (two per SIMD; gemm_tile.h can also build 4 wavefronts of 128 x 128); in the 4-wave form each
-//     wavefront owns 128 x 128 as a 4 x 4 grid of 32x32 MFMA blocks (256 accumulator
-//     registers per lane, one wavefront per SIMD).
+//     64 x 128 (two per SIMD); gemm_tile.h can also build 8 wavefronts of 128 x 64 (the mixed e4m3 x int8
+//     kernels: fewer waves then widen the same weight row) or 4 wavefronts of 128 x 128 (a 4 x 4 grid of
+//     32x32 MFMA blocks, 256 accumulator registers per lane, one wavefront per SIMD).
 //   * The WEIGHTS are the MFMA "A" operand and the TOKENS the "B" operand, i.e. the matrix
 //     cores compute C^T.  A lane then owns one token and, per MFMA block, 16 output columns;
-//     weight rows are permuted on their way into LDS so that those are 64 CONSECUTIVE
-//     columns across the four blocks.  Gate/value pairs, whole K|V heads and 16-byte output
+//     weight rows are permuted on their way into LDS so that those are 64 (32 for 64-column waves)
+//     CONSECUTIVE columns across the blocks.  Gate/value pairs, whole K|V heads and 16-byte output
 //     vectors all live inside one lane: the epilogues need no cross-lane shuffles (the SM80
 //     code needs a 4x4 shuffle transpose per 32x32 tile, cuda/gemm_b8.cuh:411, 570, 592).
 //   * Global -> LDS goes through the gfx950 16-byte direct-to-LDS load (no register staging) into
-//     a ring of LDS stages (gemm_tile.h: K_STEP bytes of K per step), one barrier per step;
+//     rings of LDS tiles (gemm_tile.h: K_STEP bytes of K per step; by default three token tiles and two
+//     weight tiles of 32 KB, which is all 160 KB of a compute unit), one barrier per step;
 //     16-byte chunks are XOR-swizzled so that ds_read_b128 is conflict-free.
 //   * int8: v_mfma_i32_32x32x32_i8.  e4m3 x e4m3: v_mfma_f32_32x32x64_f8f6f4.  Mixed
 //     e4m3 x int8: both widened exactly to f16 in registers, v_mfma_f32_32x32x16_f16
@@ -65,7 +66,9 @@ static_assert(N_RAW % gt::N_PER_BLOCK == 0, "raw output columns must be a multip
 constexpr u32 ROW_BYTES = gt::K_STEP;                       // one LDS row = one step of K
 constexpr u32 X_TILE_BYTES = gt::M_PER_BLOCK * ROW_BYTES;   // tokens
 constexpr u32 W_TILE_BYTES = gt::N_PER_BLOCK * ROW_BYTES;   // weights
-constexpr u32 STAGE_BYTES = X_TILE_BYTES + W_TILE_BYTES;
+constexpr u32 XS = gt::X_STAGES;                             // ring depth of the token tiles
+constexpr u32 WS = gt::STAGES;                               // ring depth of the weight tiles
+constexpr u32 W_RING_OFFSET = XS * X_TILE_BYTES;             // LDS: XS token tiles, then WS weight tiles
 constexpr u32 K_STEPS = K_TOTAL / gt::K_STEP;
 
 constexpr int BM = gt::WAVE_M / 32;                         // 32-token MFMA blocks per wave
@@ -274,32 +277,33 @@ struct LaneOffsets {
 // WN*wn + (WN/2)*((i/4)%2) + 16*bn + 4*(i/8) + i%4: the MFMA hands output row i = 8*(r/4) + 4*(lane/32) + r%4
 // to register r, so a lane collects columns (WN/2)*(lane/32) + 16*bn + r.  For the rows of one load unit the
 // lane-dependent part is constant.
-template <u32 I>
-X17_DEV void issue_stage_load(
-	u8 const *a_tile, u8 const *b_tile, u8 *stage, u32 k0, u32 wave, LaneOffsets const &lo
-) {
-	if constexpr (I < X_UNITS) {
-		constexpr u32 u = I;
-		u8 *x_lds = stage + (wave * X_UNITS + u) * UNIT_ROWS * ROW_BYTES;
-		u8 const *x_src = a_tile + (size_t)((wave * X_UNITS + u) * UNIT_ROWS) * K_TOTAL + k0;
-		__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(x_src + lo.x_src[u & 1]), X17_LDS_PTR(x_lds), 16, 0, 0);
-	} else {
-		constexpr u32 u = I - X_UNITS;
-		u32 r0 = (wave * W_UNITS + u) * UNIT_ROWS;
-		u32 n_uniform = gt::WAVE_N * (r0 / gt::WAVE_N) + 16 * ((r0 % gt::WAVE_N) / 32) + 4 * ((r0 % 32) / 8);
-		u8 *w_lds = stage + X_TILE_BYTES + r0 * ROW_BYTES;
-		u8 const *w_src = b_tile + (size_t)n_uniform * K_TOTAL + k0;
-		__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(w_src + lo.w_src[u & 1]), X17_LDS_PTR(w_lds), 16, 0, 0);
+template <u32 U>
+X17_DEV void issue_x_load(u8 const *a_tile, u8 *x_tile, u32 k0, u32 wave, LaneOffsets const &lo) {
+	u8 *x_lds = x_tile + (wave * X_UNITS + U) * UNIT_ROWS * ROW_BYTES;
+	u8 const *x_src = a_tile + (size_t)((wave * X_UNITS + U) * UNIT_ROWS) * K_TOTAL + k0;
+	__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(x_src + lo.x_src[U & 1]), X17_LDS_PTR(x_lds), 16, 0, 0);
+}
+template <u32 U>
+X17_DEV void issue_w_load(u8 const *b_tile, u8 *w_tile, u32 k0, u32 wave, LaneOffsets const &lo) {
+	u32 r0 = (wave * W_UNITS + U) * UNIT_ROWS;
+	u32 n_uniform = gt::WAVE_N * (r0 / gt::WAVE_N) + 16 * ((r0 % gt::WAVE_N) / 32) + 4 * ((r0 % 32) / 8);
+	u8 *w_lds = w_tile + r0 * ROW_BYTES;
+	u8 const *w_src = b_tile + (size_t)n_uniform * K_TOTAL + k0;
+	__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(w_src + lo.w_src[U & 1]), X17_LDS_PTR(w_lds), 16, 0, 0);
+}
+// this wave's share of one token tile / one weight tile of one step
+template <u32 FIRST = 0>
+X17_DEV void issue_x_loads(u8 const *a_tile, u8 *x_tile, u32 k0, u32 wave, LaneOffsets const &lo) {
+	if constexpr (FIRST < X_UNITS) {
+		issue_x_load<FIRST>(a_tile, x_tile, k0, wave, lo);
+		issue_x_loads<FIRST + 1>(a_tile, x_tile, k0, wave, lo);
 	}
 }
-
-template <u32 FIRST, u32 LAST>
-X17_DEV void issue_stage_loads(
-	u8 const *a_tile, u8 const *b_tile, u8 *stage, u32 k0, u32 wave, LaneOffsets const &lo
-) {
-	if constexpr (FIRST < LAST) {
-		issue_stage_load<FIRST>(a_tile, b_tile, stage, k0, wave, lo);
-		issue_stage_loads<FIRST + 1, LAST>(a_tile, b_tile, stage, k0, wave, lo);
+template <u32 FIRST = 0>
+X17_DEV void issue_w_loads(u8 const *b_tile, u8 *w_tile, u32 k0, u32 wave, LaneOffsets const &lo) {
+	if constexpr (FIRST < W_UNITS) {
+		issue_w_load<FIRST>(b_tile, w_tile, k0, wave, lo);
+		issue_w_loads<FIRST + 1>(b_tile, w_tile, k0, wave, lo);
 	}
 }
 
@@ -309,15 +313,24 @@ X17_DEV void wait_vmcnt() {
 	static_assert(N < 64);
 	__builtin_amdgcn_s_waitcnt((N & 15u) | ((N >> 4) << 14) | 0x0F70u);
 }
-// wait until at most `later` younger stages are still in flight
-X17_DEV void wait_stage(u32 later) {
-	if constexpr (gt::STAGES >= 4) {
-		if (later >= 2) { wait_vmcnt<2 * LOADS_PER_STAGE>(); return; }
+// Loads complete in issue order.  Behind every barrier a wave issues its share of one weight tile (step + WS)
+// and then of one token tile (step + XS).  The tiles of step ks+1 are awaited with everything issued after
+// the weight tile of that step still allowed in flight: the token tile issued with it when the token ring
+// is the deeper one, and `later` whole steps.
+X17_DEV void wait_step(u32 later, bool token_tile_behind) {
+	if constexpr (WS >= 4) {
+		if (later >= 2) {
+			if (XS > WS && token_tile_behind) { wait_vmcnt<2 * LOADS_PER_STAGE + X_UNITS>(); } else { wait_vmcnt<2 * LOADS_PER_STAGE>(); }
+			return;
+		}
 	}
-	if constexpr (gt::STAGES >= 3) {
-		if (later >= 1) { wait_vmcnt<LOADS_PER_STAGE>(); return; }
+	if constexpr (WS >= 3) {
+		if (later >= 1) {
+			if (XS > WS && token_tile_behind) { wait_vmcnt<LOADS_PER_STAGE + X_UNITS>(); } else { wait_vmcnt<LOADS_PER_STAGE>(); }
+			return;
+		}
 	}
-	wait_vmcnt<0>();
+	if (XS > WS && token_tile_behind) { wait_vmcnt<X_UNITS>(); } else { wait_vmcnt<0>(); }
 }
 
 // One 16-byte operand chunk: row `row_off` (bytes), logical chunk `kc` of the row.
@@ -503,41 +516,45 @@ void kernel(
 		lo.swz = ((lane % 32) >> SWZ_SHIFT) & (CHUNKS - 1);
 	}
 
-	// ---- main loop.  A ring of STAGES LDS buffers; step ks consumes buffer ks % STAGES while the loads of
-	// steps ks+1 .. ks+STAGES-1 are in flight.  The one barrier per step sits before the last slice's
-	// MFMAs, when every wave holds the last fragments of the step in registers: behind it the buffer is
-	// free, so the loads of step ks+STAGES are issued there -- a full step before they are waited for --
-	// and the first fragments of step ks+1 are fetched, so LDS latency is covered by matrix-core time across
-	// the step boundary too.  The load stream runs across tile boundaries: the last steps of a tile
-	// already fetch the first stages of the workgroup's next tile, which land while the epilogue runs.
-	// (a K shorter than the ring cannot prefetch across tiles: each tile then starts with its own prologue)
-	constexpr bool CROSS_TILE = K_STEPS >= gt::STAGES;
-	constexpr u32 PROLOGUE_STAGES = CROSS_TILE ? gt::STAGES : K_STEPS;
+	// ---- main loop.  Rings of XS token tiles and WS weight tiles in LDS; step ks consumes ring positions
+	// ks % XS and ks % WS while the tiles of the following steps are in flight.  The one barrier per step sits
+	// before the last slice's MFMAs, when every wave holds the last fragments of the step in registers: behind
+	// it both positions are free, so the weight tile of step ks+WS and the token tile of step ks+XS are
+	// requested there, and the first fragments of step ks+1 are fetched, so LDS latency is covered by
+	// matrix-core time across the step boundary too.  The load stream runs across tile boundaries: the last
+	// steps of a tile already fetch the first steps of the workgroup's next tile, which land while the epilogue
+	// runs.  (a K shorter than the ring cannot prefetch across tiles: each tile then starts with its own prologue)
+	static_assert(XS == WS || WS == 2, "a deeper token ring is supported on top of a two-deep weight ring");
+	constexpr bool CROSS_TILE = K_STEPS >= XS;
 	u32 const x_off = wm * gt::WAVE_M * ROW_BYTES + lo.frag_row;
-	u32 const w_off = X_TILE_BYTES + wn * gt::WAVE_N * ROW_BYTES + lo.frag_row;
+	u32 const w_off = W_RING_OFFSET + wn * gt::WAVE_N * ROW_BYTES + lo.frag_row;
 
 	u32 tile_m, tile_n;
 	tile_coords(group, tile_m, tile_n);
 	u8 const *a_tile = a + (size_t)(tile_m * gt::M_PER_BLOCK) * K_TOTAL;
 	u8 const *b_tile = b + (size_t)(tile_n * gt::N_PER_BLOCK) * K_TOTAL;
+	// the first steps of a tile nobody prefetched, in the order the waits of the main loop assume
+	// (token tile s, weight tile s, ..., then the extra token tile of a deeper token ring)
 	auto prologue = [&]() {
-		X17_UNROLL for (u32 s = 0; s < PROLOGUE_STAGES; ++s) {
-			issue_stage_loads<0, LOADS_PER_STAGE>(a_tile, b_tile, smem + s * STAGE_BYTES, s * gt::K_STEP, wave, lo);
+		X17_UNROLL for (u32 s = 0; s < WS; ++s) {
+			if (s < K_STEPS) {
+				issue_x_loads(a_tile, smem + s * X_TILE_BYTES, s * gt::K_STEP, wave, lo);
+				issue_w_loads(b_tile, smem + W_RING_OFFSET + s * W_TILE_BYTES, s * gt::K_STEP, wave, lo);
+			}
 		}
-		if constexpr (CROSS_TILE) {
-			wait_stage(gt::STAGES - 1);                // stage 0 has landed ...
-		} else {
-			wait_vmcnt<0>();
+		if constexpr (XS > WS && CROSS_TILE) {
+			issue_x_loads(a_tile, smem + WS * X_TILE_BYTES, WS * gt::K_STEP, wave, lo);
 		}
-		__builtin_amdgcn_s_barrier();                  // ... for every wave
+		wait_vmcnt<0>();
+		__builtin_amdgcn_s_barrier();
 	};
 	prologue();
 
-	u32 buf = 0;                                   // ring position of the step being consumed
+	u32 xb = 0, wb = 0;                            // ring positions of the step being consumed
 	for (u32 lin = group; lin < total; lin += n_groups) {
 		bool const first_tile = lin == group;
 		bool const more_tiles = lin + n_groups < total;
-		bool const has_next = CROSS_TILE && more_tiles;      // prefetch the next tile's first stages
+		bool const has_next = CROSS_TILE && more_tiles;      // prefetch the next tile's first steps
 		u32 next_m = 0, next_n = 0;
 		if (more_tiles) {
 			tile_coords(lin + n_groups, next_m, next_n);
@@ -548,7 +565,8 @@ void kernel(
 			if (!first_tile) {
 				__builtin_amdgcn_s_waitcnt(0xC07F);        // lgkmcnt(0)
 				__builtin_amdgcn_s_barrier();              // nobody still reads the previous tile's buffers
-				buf = 0;
+				xb = 0;
+				wb = 0;
 				prologue();
 			}
 		}
@@ -560,38 +578,51 @@ void kernel(
 			}
 		}
 
-		// (stage 0 of this tile is visible: the wait and the barrier were the previous tile's last ones)
+		// (step 0 of this tile is visible: the wait and the barrier were the previous tile's last ones)
 		Frags frags[2];
-		load_frags(frags[0], smem + buf * STAGE_BYTES + w_off, smem + buf * STAGE_BYTES + x_off, 0, lo);
+		load_frags(frags[0], smem + wb * W_TILE_BYTES + w_off, smem + xb * X_TILE_BYTES + x_off, 0, lo);
 
 		X17_K_LOOP_PRAGMA
 		for (u32 ks = 0; ks < K_STEPS; ++ks) {
-			u32 const next_buf = buf + 1 == gt::STAGES ? 0 : buf + 1;
-			u32 const load_step = ks + gt::STAGES;                       // the step whose loads go out behind this barrier
-			bool const this_tile = load_step < K_STEPS;
-			bool const more_loads = this_tile || has_next;
-			u8 const *la = this_tile ? a_tile : a_next;
-			u8 const *lb = this_tile ? b_tile : b_next;
-			u32 const load_k0 = (this_tile ? load_step : load_step - K_STEPS) * gt::K_STEP;
-			u8 *stage = smem + buf * STAGE_BYTES;
+			u32 const next_xb = xb + 1 == XS ? 0 : xb + 1;
+			u32 const next_wb = wb + 1 == WS ? 0 : wb + 1;
+			// the tiles requested behind this step's barrier: weight step ks+WS, token step ks+XS (of this
+			// output tile or of the workgroup's next one)
+			u32 const w_step = ks + WS, x_step = ks + XS;
+			bool const w_here = w_step < K_STEPS, x_here = x_step < K_STEPS;
+			u8 const *lw = w_here ? b_tile : b_next;
+			u8 const *lx = x_here ? a_tile : a_next;
+			u32 const w_k0 = (w_here ? w_step : w_step - K_STEPS) * gt::K_STEP;
+			u32 const x_k0 = (x_here ? x_step : x_step - K_STEPS) * gt::K_STEP;
+			u8 const *w_tile = smem + wb * W_TILE_BYTES + w_off;
+			u8 const *x_tile = smem + xb * X_TILE_BYTES + x_off;
 			X17_UNROLL for (u32 s = 0; s < SLICES; ++s) {
 				bool reads = true;
 				if (s + 1 < SLICES) {
-					load_frags(frags[(s + 1) & 1], stage + w_off, stage + x_off, s + 1, lo);
+					load_frags(frags[(s + 1) & 1], w_tile, x_tile, s + 1, lo);
 				} else if (ks + 1 < K_STEPS || has_next) {
-					// step ks+1 (or the next tile's step 0) must have landed; younger stages may stay in flight.
-					// After an epilogue its stores share the counter with the loads: wait for everything then.
-					u32 in_flight = has_next ? gt::STAGES : K_STEPS - 2 - ks;     // stages issued after the awaited one
-					bool const stores_pending = !first_tile && ks + 1 < gt::STAGES;
-					wait_stage(stores_pending ? 0 : (in_flight < gt::STAGES - 2 ? in_flight : gt::STAGES - 2));
-					__builtin_amdgcn_s_waitcnt(0xC07F);    // lgkmcnt(0): this wave is done reading buffer `buf`
+					// Step ks+1 (or the next tile's step 0) must have landed; what was requested after its weight
+					// tile may stay in flight: the token tile of step ks+2 when the token ring is the deeper one,
+					// and up to WS-2 whole steps.  After an epilogue its stores share the counter with the loads:
+					// wait for everything then.
+					u32 const later_steps = has_next ? WS - 2 : (K_STEPS - 2 - ks < WS - 2 ? K_STEPS - 2 - ks : WS - 2);
+					bool const token_tile_behind = has_next || ks + 2 < K_STEPS;
+					bool const stores_pending = !first_tile && ks + 1 < WS;
+					if (stores_pending) {
+						wait_vmcnt<0>();
+					} else {
+						wait_step(later_steps, token_tile_behind);
+					}
+					__builtin_amdgcn_s_waitcnt(0xC07F);    // lgkmcnt(0): this wave is done reading this step's tiles
 					__builtin_amdgcn_s_barrier();
-					if (more_loads) {
-						issue_stage_loads<0, LOADS_PER_STAGE>(la, lb, stage, load_k0, wave, lo);
+					if (w_here || has_next) {
+						issue_w_loads(lw, smem + W_RING_OFFSET + wb * W_TILE_BYTES, w_k0, wave, lo);
+					}
+					if (x_here || has_next) {
+						issue_x_loads(lx, smem + xb * X_TILE_BYTES, x_k0, wave, lo);
 					}
 					if (ks + 1 < K_STEPS) {
-						u8 const *next = smem + next_buf * STAGE_BYTES;
-						load_frags(frags[(s + 1) & 1], next + w_off, next + x_off, 0, lo);
+						load_frags(frags[(s + 1) & 1], smem + next_wb * W_TILE_BYTES + w_off, smem + next_xb * X_TILE_BYTES + x_off, 0, lo);
 					} else {
 						reads = false;
 					}
@@ -605,7 +636,8 @@ void kernel(
 					interleave_slice<LOADS_PER_STAGE>(reads);
 				}
 			}
-			buf = next_buf;
+			xb = next_xb;
+			wb = next_wb;
 		}
 
 	// ---- epilogue.  Lane owns token (32*bm + lane%32) of its wave and raw columns

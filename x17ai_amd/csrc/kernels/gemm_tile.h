@@ -7,7 +7,8 @@
 //
 // A build may override the geometry with -DX17_GEMM_M_PER_BLOCK (128 or 256 tokens per workgroup),
 // -DX17_GEMM_WAVES_M / -DX17_GEMM_WAVES_N (wavefronts along the tokens / along the raw output columns),
-// -DX17_GEMM_K_STEP (64 or 128 bytes of K per pipeline step) and -DX17_GEMM_STAGES (LDS ring depth).
+// -DX17_GEMM_K_STEP (64 or 128 bytes of K per pipeline step), -DX17_GEMM_STAGES (LDS ring depth) and
+// -DX17_GEMM_X_STAGES (ring depth of the token operand alone: STAGES or STAGES + 1).  Needs X17_A_COLS too.
 #pragma once
 
 namespace x17 { namespace gemm_tile {
@@ -41,7 +42,17 @@ constexpr unsigned WAVE_N = N_PER_BLOCK / WAVES_N;       // raw output columns p
 constexpr unsigned K_STEP = X17_GEMM_K_STEP;             // bytes of K staged per pipeline step
 constexpr unsigned STAGES = X17_GEMM_STAGES;
 
-constexpr unsigned SMEM_BYTES = STAGES * (M_PER_BLOCK + N_PER_BLOCK) * K_STEP;
+// The token tiles may have a ring one deeper than the weight tiles: 3 x 32 KB + 2 x 32 KB fill the 160 KB of
+// LDS of a compute unit exactly, and the token loads then have two steps to arrive, the weight loads one
+// (with two stages of both, a step's 64 KB of loads have a single step -- about their own latency -- to land).
+#ifndef X17_GEMM_X_STAGES
+#define X17_GEMM_X_STAGES \
+	((X17_GEMM_STAGES == 2 && X17_GEMM_K_STEP == 128 && X17_GEMM_M_PER_BLOCK == 256 && (X17_A_COLS) / 128 >= 3) ? 3 : X17_GEMM_STAGES)
+#endif
+constexpr unsigned X_STAGES = X17_GEMM_X_STAGES;
+static_assert(X_STAGES == STAGES || X_STAGES == STAGES + 1, "the token ring is as deep as the weight ring or one deeper");
+
+constexpr unsigned SMEM_BYTES = (X_STAGES * M_PER_BLOCK + STAGES * N_PER_BLOCK) * K_STEP;
 
 // The kernel is persistent (a workgroup walks tiles g, g + G, ...): the launcher starts at most this
 // many workgroups, one per compute unit of an MI355X.
