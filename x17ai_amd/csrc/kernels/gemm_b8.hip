@@ -73,8 +73,6 @@ constexpr u32 K_STEPS = K_TOTAL / gt::K_STEP;
 
 constexpr int BM = gt::WAVE_M / 32;                         // 32-token MFMA blocks per wave
 constexpr u32 WAVES = gt::WAVES_M * gt::WAVES_N;
-constexpr u32 ROWS_PER_WAVE = 256 / WAVES;                  // rows of each tile a wave copies per stage
-constexpr u32 UNITS = ROWS_PER_WAVE / 8;                    // 8-row direct-to-LDS loads per wave and tile
 
 using Acc = __attribute__((ext_vector_type(16))) int;       // raw 16 registers; reinterpreted as f32 when ACC_F32
 
@@ -257,8 +255,13 @@ static_assert(HEAD_DIM == 32 || HEAD_DIM == 64 || HEAD_DIM == 128, "head_dim mus
 constexpr u32 CHUNKS = gt::K_STEP / 16;
 constexpr u32 SWZ_SHIFT = gt::K_STEP == 128 ? 1 : 2;
 constexpr u32 UNIT_ROWS = 64 / CHUNKS;                      // rows one 64-lane x 16-byte direct-to-LDS load fills
-constexpr u32 X_UNITS = gt::M_PER_BLOCK / UNIT_ROWS / WAVES; // such loads per wave, stage and tile
-constexpr u32 W_UNITS = gt::N_PER_BLOCK / UNIT_ROWS / WAVES;
+// With two waves per SIMD only the first of each pair (waves 0 .. WAVES/2 - 1) requests tiles.  The arbiter serves
+// that wave first: with the loads shared evenly it ended its step early and sat at the barrier while its partner,
+// the same loads to issue between its MFMAs, finished alone.  (Splitting the weight units 6:2, 4:4, 2:6 or 0:8
+// between the two measured the same as 8:0.)
+constexpr u32 LOADER_WAVES = gt::WAVES_PER_SIMD == 2 ? WAVES / 2 : WAVES;
+constexpr u32 X_UNITS = gt::M_PER_BLOCK / UNIT_ROWS / LOADER_WAVES; // such loads per loading wave, step and tile
+constexpr u32 W_UNITS = gt::N_PER_BLOCK / UNIT_ROWS / LOADER_WAVES;
 constexpr u32 LOADS_PER_STAGE = X_UNITS + W_UNITS;
 static_assert((X_UNITS * UNIT_ROWS) % 16 == 0 && (W_UNITS * UNIT_ROWS) % 16 == 0, "a wave's share must keep the swizzle phase");
 
@@ -270,9 +273,8 @@ struct LaneOffsets {
 	u32 swz;        // swizzle key of the fragment row this lane reads
 };
 
-// Direct-to-LDS load `i` (0 .. LOADS_PER_STAGE-1) of this wave's share of one stage: first the token
-// units, then the weight units.  Wave w copies token rows [X_UNITS * UNIT_ROWS * w, +X_UNITS * UNIT_ROWS)
-// and as many LDS weight rows.
+// Direct-to-LDS loads of a loading wave's share of one token tile / one weight tile: loading wave w copies
+// token rows [X_UNITS * UNIT_ROWS * w, +X_UNITS * UNIT_ROWS) and as many LDS weight rows.
 // With WN = WAVE_N columns per wave, LDS weight row R = WN*wn + 32*bn + i holds weight row
 // WN*wn + (WN/2)*((i/4)%2) + 16*bn + 4*(i/8) + i%4: the MFMA hands output row i = 8*(r/4) + 4*(lane/32) + r%4
 // to register r, so a lane collects columns (WN/2)*(lane/32) + 16*bn + r.  For the rows of one load unit the
@@ -293,17 +295,28 @@ X17_DEV void issue_w_load(u8 const *b_tile, u8 *w_tile, u32 k0, u32 wave, LaneOf
 }
 // this wave's share of one token tile / one weight tile of one step
 template <u32 FIRST = 0>
-X17_DEV void issue_x_loads(u8 const *a_tile, u8 *x_tile, u32 k0, u32 wave, LaneOffsets const &lo) {
+X17_DEV void issue_x_units(u8 const *a_tile, u8 *x_tile, u32 k0, u32 wave, LaneOffsets const &lo) {
 	if constexpr (FIRST < X_UNITS) {
 		issue_x_load<FIRST>(a_tile, x_tile, k0, wave, lo);
-		issue_x_loads<FIRST + 1>(a_tile, x_tile, k0, wave, lo);
+		issue_x_units<FIRST + 1>(a_tile, x_tile, k0, wave, lo);
 	}
 }
 template <u32 FIRST = 0>
-X17_DEV void issue_w_loads(u8 const *b_tile, u8 *w_tile, u32 k0, u32 wave, LaneOffsets const &lo) {
+X17_DEV void issue_w_units(u8 const *b_tile, u8 *w_tile, u32 k0, u32 wave, LaneOffsets const &lo) {
 	if constexpr (FIRST < W_UNITS) {
 		issue_w_load<FIRST>(b_tile, w_tile, k0, wave, lo);
-		issue_w_loads<FIRST + 1>(b_tile, w_tile, k0, wave, lo);
+		issue_w_units<FIRST + 1>(b_tile, w_tile, k0, wave, lo);
+	}
+}
+// (the other waves have nothing in flight: their waits on the load counter fall through)
+X17_DEV void issue_x_loads(u8 const *a_tile, u8 *x_tile, u32 k0, u32 wave, LaneOffsets const &lo) {
+	if (wave < LOADER_WAVES) {
+		issue_x_units(a_tile, x_tile, k0, wave, lo);
+	}
+}
+X17_DEV void issue_w_loads(u8 const *b_tile, u8 *w_tile, u32 k0, u32 wave, LaneOffsets const &lo) {
+	if (wave < LOADER_WAVES) {
+		issue_w_units(b_tile, w_tile, k0, wave, lo);
 	}
 }
 
