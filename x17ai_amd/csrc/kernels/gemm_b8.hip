@@ -279,11 +279,20 @@ struct LaneOffsets {
 // WN*wn + (WN/2)*((i/4)%2) + 16*bn + 4*(i/8) + i%4: the MFMA hands output row i = 8*(r/4) + 4*(lane/32) + r%4
 // to register r, so a lane collects columns (WN/2)*(lane/32) + 16*bn + r.  For the rows of one load unit the
 // lane-dependent part is constant.
+// One 16-byte-per-lane direct-to-LDS load: LDS destination in M0 (wave-uniform; lane l lands 16 * l bytes further),
+// global source = uniform 64-bit base in scalar registers + a 32-bit offset per lane.  Written out because the
+// compiler's own selection forms a 64-bit address per lane in ONE vector register pair for every load: a 64-bit
+// vector add per load, each waiting until the previous load has read the pair (measured 3-5 % of the kernel).
+X17_DEV void load_to_lds_16(u8 *lds_uniform, u8 const *src_uniform, u32 lane_offset) {
+	asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+	             :: "s"((u32)(size_t)X17_LDS_PTR(lds_uniform)), "v"(lane_offset), "s"(src_uniform) : "memory", "m0");
+}
+
 template <u32 U>
 X17_DEV void issue_x_load(u8 const *a_tile, u8 *x_tile, u32 k0, u32 wave, LaneOffsets const &lo) {
 	u8 *x_lds = x_tile + (wave * X_UNITS + U) * UNIT_ROWS * ROW_BYTES;
 	u8 const *x_src = a_tile + (size_t)((wave * X_UNITS + U) * UNIT_ROWS) * K_TOTAL + k0;
-	__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(x_src + lo.x_src[U & 1]), X17_LDS_PTR(x_lds), 16, 0, 0);
+	load_to_lds_16(x_lds, x_src, lo.x_src[U & 1]);
 }
 template <u32 U>
 X17_DEV void issue_w_load(u8 const *b_tile, u8 *w_tile, u32 k0, u32 wave, LaneOffsets const &lo) {
@@ -291,7 +300,7 @@ X17_DEV void issue_w_load(u8 const *b_tile, u8 *w_tile, u32 k0, u32 wave, LaneOf
 	u32 n_uniform = gt::WAVE_N * (r0 / gt::WAVE_N) + 16 * ((r0 % gt::WAVE_N) / 32) + 4 * ((r0 % 32) / 8);
 	u8 *w_lds = w_tile + r0 * ROW_BYTES;
 	u8 const *w_src = b_tile + (size_t)n_uniform * K_TOTAL + k0;
-	__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(w_src + lo.w_src[U & 1]), X17_LDS_PTR(w_lds), 16, 0, 0);
+	load_to_lds_16(w_lds, w_src, lo.w_src[U & 1]);
 }
 // this wave's share of one token tile / one weight tile of one step
 template <u32 FIRST = 0>
