@@ -255,11 +255,11 @@ static_assert(HEAD_DIM == 32 || HEAD_DIM == 64 || HEAD_DIM == 128, "head_dim mus
 constexpr u32 CHUNKS = gt::K_STEP / 16;
 constexpr u32 SWZ_SHIFT = gt::K_STEP == 128 ? 1 : 2;
 constexpr u32 UNIT_ROWS = 64 / CHUNKS;                      // rows one 64-lane x 16-byte direct-to-LDS load fills
-// With two waves per SIMD only the first of each pair (waves 0 .. WAVES/2 - 1) requests tiles.  The arbiter serves
+// With eight waves, two per SIMD, only the first of each pair (waves 0 .. 3) requests tiles.  The arbiter serves
 // that wave first: with the loads shared evenly it ended its step early and sat at the barrier while its partner,
 // the same loads to issue between its MFMAs, finished alone.  (Splitting the weight units 6:2, 4:4, 2:6 or 0:8
 // between the two measured the same as 8:0.)
-constexpr u32 LOADER_WAVES = gt::WAVES_PER_SIMD == 2 ? WAVES / 2 : WAVES;
+constexpr u32 LOADER_WAVES = WAVES == 8 ? 4 : WAVES;      // (a four-wave workgroup has one wave per SIMD)
 constexpr u32 X_UNITS = gt::M_PER_BLOCK / UNIT_ROWS / LOADER_WAVES; // such loads per loading wave, step and tile
 constexpr u32 W_UNITS = gt::N_PER_BLOCK / UNIT_ROWS / LOADER_WAVES;
 constexpr u32 LOADS_PER_STAGE = X_UNITS + W_UNITS;
