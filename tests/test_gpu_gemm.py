@@ -154,6 +154,30 @@ def test_mixed_e4m3_i8_residual(dev, m, k, n):
 	assert neq < 5e-3 and beyond == 0.0, (neq, beyond)
 
 
+@pytest.mark.parametrize("geglu", [False, True])
+def test_mixed_e4m3_i8_scale_and_geglu(dev, geglu):
+	"""The e4m3 x int8 operand mix (waves of 128 tokens x 64 columns) under the Scale and GeGLU writers."""
+	m, k, n = 512, 1024, 512
+	rng = rng_for("mixed-writers", geglu)
+	a = e4m3_bytes(rng, (m, k), 0.6)
+	b = i8_codes(rng, (n, k))
+	acc = S.gemm_f32_seq(a, True, b, False)
+	inp = 1.0 / math.sqrt(k) / 8.0
+	kern = recipes.mixed_gemm_kernel(dev, k, n, geglu, True)
+	if geglu:
+		want = S.epilogue_geglu(acc, inp, 1.0, S.STORE_E4M3)
+		c = X.Tensor(dev, (m, n // 2), X.E4M3)
+		kern.launch(_up(dev, a, X.E4M3), _up(dev, b, X.INT8), c)
+		neq, beyond = e4m3_compare(c.download(), want)
+		assert neq < 5e-3 and beyond == 0.0, (neq, beyond)
+	else:
+		want = S.epilogue_scale(acc, inp, 8.0)
+		c = X.Tensor(dev, (m, n), X.INT8)
+		kern.launch(_up(dev, a, X.E4M3), _up(dev, b, X.INT8), c)
+		d = np.abs(c.download().astype(np.int32) - want.astype(np.int32))
+		assert d.max() <= 1 and np.mean(d > 0) < 5e-3, (d.max(), np.mean(d > 0))
+
+
 @pytest.mark.parametrize("m,k,n", [(256, 512, 256), (512, 4096, 512)])
 def test_fp8_geglu(dev, m, k, n):
 	"""All-fp8 ffn_f: e4m3 x e4m3 on the fp8 matrix cores, f32 accumulate, GeGLU -> e4m3."""

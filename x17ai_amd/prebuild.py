@@ -28,6 +28,8 @@ def _specs():
 				add(("ffn_f", k, n, strict, store))
 				add(("attn_y", n // 2, k, strict, store))
 	add(("acc_probe",))
+	for geglu in (False, True):
+		add(("mixed", 1024, 512, geglu))
 	for hd in (32, 64, 128):
 		for k in (512, 2048):
 			add(("attn_kv", k, 512, hd))
@@ -107,6 +109,8 @@ def _build_one(spec) -> str:
 		return recipes.attn_kv_kernel(None, spec[1], spec[2], spec[3]).name
 	if kind == "ffn_y":
 		return recipes.ffn_y_kernel(None, spec[1], spec[2], spec[3], spec[4], spec[5]).name
+	if kind == "mixed":
+		return recipes.mixed_gemm_kernel(None, spec[1], spec[2], spec[3]).name
 	if kind == "ffn_f_f8":
 		return recipes.ffn_f_f8_kernel(None, spec[1], spec[2], spec[3]).name
 	if kind == "attn":

@@ -107,6 +107,17 @@ def ffn_f_f8_kernel(device: Optional[Device], model_dim: int, ffn_f_proj_outputs
 	                  _gemm(E4M3, E4M3, E4M3, model_dim, ffn_f_proj_outputs), cfg, strict)
 
 
+def mixed_gemm_kernel(device: Optional[Device], k: int, n_raw: int, geglu: bool, strict: bool = True) -> GemmKernel:
+	"""e4m3 activations x int8 weights with the Scale writer (-> FixedI8) or the GeGLU writer (-> e4m3): the
+	operand mix of ffn_y_fwd_f8 (cuda/gemm_b16.cuh:72-185) under the other two writers that accept f32 sums."""
+	inp = _inv_sqrt(k) / FIXED_I8_SCALE
+	if geglu:
+		return GemmKernel(device, f"mixed_geglu-k{k}-n{n_raw}-{_mode(strict)}", _gemm(E4M3, INT8, E4M3, k, n_raw),
+		                  GeGluConfig(inp, 1.0), strict)
+	return GemmKernel(device, f"mixed_scale-k{k}-n{n_raw}-{_mode(strict)}", _gemm(E4M3, INT8, INT8, k, n_raw),
+	                  ScaleConfig(inp, FIXED_I8_SCALE), strict)
+
+
 def dequant_gemm_kernel(device: Optional[Device], k: int, n_raw: int, a_dtype: int = INT8, b_dtype: int = INT8,
                         geglu: bool = False, strict: bool = True) -> GemmKernel:
 	"""No counterpart in src/main.rs: a[M, k] . b[n_raw, k]^T with run-time per-row and per-column f32
