@@ -120,6 +120,34 @@ def cpu_baseline():
 	        "sample": f"{M} of 8192 token rows of config 2 (both GEMMs + epilogues), {dt:.1f} s of CPU time"}
 
 
+def mfma_probe(dev, X):
+	"""Loops of nothing but MFMAs on register operands, all-zero and Gaussian data: what the matrix cores of this
+	machine sustain (the clock under dense MFMA load depends on how much the operands toggle)."""
+	from x17ai_amd.api import MfmaProbe
+	rng = np.random.default_rng(7)
+	out = X.Tensor(dev, (256 * 512,), X.F32)
+	result = {}
+	for kind, name, peak in ((0, "int8", PEAK_INT8_TOPS), (1, "e4m3", PEAK_INT8_TOPS), (2, "f16", PEAK_INT8_TOPS / 2)):
+		probe = MfmaProbe(dev, kind)
+		if kind == 0:
+			gauss = _rand_codes(rng, (12 * 512 * 16,))
+		elif kind == 1:
+			gauss = rng.integers(0x20, 0x50, 12 * 512 * 16).astype(np.uint8).view(np.int8)       # normal e4m3 codes
+			gauss = np.where(rng.random(gauss.shape) < 0.5, gauss, gauss | np.int8(-128)).astype(np.int8)
+		else:
+			gauss = rng.standard_normal(12 * 512 * 8).astype(np.float16).view(np.int8)
+		for data_name, data in (("zeros", np.zeros(12 * 512 * 16, np.int8)), ("gaussian", gauss)):
+			operands = X.Tensor.from_numpy(dev, np.ascontiguousarray(data), X.INT8)
+			ops = [0.0]
+
+			def fn():
+				ops[0] = probe.launch(operands, out, 4096)
+			med, mn = _median_launch(dev, X, fn, 10, 3)
+			result[f"{name}_{data_name}"] = {"median_us": med * 1e6, "tops": ops[0] / med / 1e12,
+			                                 "frac_of_nominal_peak": ops[0] / med / 1e12 / peak}
+	return result
+
+
 def extras(dev, X, recipes):
 	out = {}
 	rng = np.random.default_rng(3000)
@@ -312,6 +340,8 @@ def extras(dev, X, recipes):
 	med, _ = _median_launch(dev, X, lambda: kd_rows.launch_row_scaled(qd, cache, lens, sk5, sv5, tp5, odb, None, W5, *rsd), 10, 3)
 	c5["decode_row_scaled_bf16_us"] = med * 1e6
 	out["config5_long_context"] = c5
+	# what the matrix cores sustain with no memory traffic at all, beside the nominal peaks used above
+	out["mfma_probe"] = mfma_probe(dev, X)
 	return out
 
 
@@ -386,6 +416,9 @@ def main():
 	ap.add_argument("--no-cpu", action="store_true")
 	ap.add_argument("--copy-probe", action="store_true",
 	                help="only run a 1 GiB device-to-device copy kernel (calibrates the HBM traffic counters)")
+	ap.add_argument("--mfma-probe", action="store_true",
+	                help="only run loops of nothing but MFMAs on register operands (all-zero and Gaussian data; int8, "
+	                     "e4m3, f16): what the matrix cores of this machine sustain, beside the nominal peaks")
 	ap.add_argument("--only", choices=ONLY_TARGETS,
 	                help="launch one kernel of one workload --steps times and print its median (used for the profiles)")
 	args = ap.parse_args()
@@ -407,6 +440,9 @@ def main():
 			probe.launch(src, dst)
 		dev.synchronize()
 		print(json.dumps({"copy_probe_bytes_read": n, "copy_probe_bytes_written": n, "launches": 5}))
+		return
+	if args.mfma_probe:
+		print(json.dumps({"mfma_probe": mfma_probe(dev, X)}))
 		return
 	if args.only:
 		single(dev, X, recipes, args.only, args.steps)

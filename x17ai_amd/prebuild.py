@@ -74,6 +74,8 @@ def _specs():
 	add(("attn_rows", 32, 128, BF16, False))
 	add(("decode_rows", 32, 128, 4096, BF16, False))
 	add(("copy_probe",))
+	for kind in (0, 1, 2):
+		add(("mfma_probe", kind))
 	# ---- tests/test_gpu_fullsize.py (the strict ffn pair, attention and decode kernels are listed above)
 	add(("attn", 16, 128, True))
 	add(("attn_rows", 32, 128, BF16, True))
@@ -125,6 +127,10 @@ def _build_one(spec) -> str:
 		return recipes.rms_norm_kernel(None, spec[1], spec[2]).name
 	if kind == "dequant":
 		return recipes.dequant_gemm_kernel(None, spec[1], spec[2], spec[3], spec[4], spec[5], spec[6]).name
+	if kind == "mfma_probe":
+		from .api import MfmaProbe
+		MfmaProbe(None, spec[1])
+		return f"mfma_probe-kind{spec[1]}"
 	if kind == "copy_probe":
 		from .api import CopyProbe
 		CopyProbe(None)
