@@ -53,7 +53,6 @@ constexpr u32 K_TOTAL = X17_A_COLS;
 constexpr u32 N_RAW = X17_B_ROWS;
 constexpr int A_KIND = X17_A_KIND;
 constexpr int B_KIND = X17_B_KIND;
-constexpr int EPILOGUE = X17_EPILOGUE;
 constexpr int STORE = X17_STORE;
 
 // 0: int8 MFMA, 1: fp8 MFMA, 2: f16 MFMA after widening
@@ -365,7 +364,7 @@ X17_DEV v4i lds_chunk(u8 const *tile, u32 row_off, u32 kc, u32 swz) {
 //         reference's encoder produces (no subnormals, no NaN, no -0) mean the same in both.
 //   int8: flip the sign bit (b + 128 as an unsigned byte u), splice u under the f16 exponent of 1024
 //         (0x6400 | u == 1024 + u) and subtract 1152 -- five instructions per four bytes.
-X17_DEV v8h widen8(u32 lo, u32 hi, int kind) {
+[[maybe_unused]] X17_DEV v8h widen8(u32 lo, u32 hi, int kind) {
 	v2h p[4];
 	if (kind == 1) {
 		p[0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, false);
