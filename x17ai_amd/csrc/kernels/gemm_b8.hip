@@ -264,9 +264,18 @@ constexpr u32 W_UNITS = gt::N_PER_BLOCK / UNIT_ROWS / LOADER_WAVES;
 constexpr u32 LOADS_PER_STAGE = X_UNITS + W_UNITS;
 static_assert((X_UNITS * UNIT_ROWS) % 16 == 0 && (W_UNITS * UNIT_ROWS) % 16 == 0, "a wave's share must keep the swizzle phase");
 
+// A wave that has a SIMD to itself has registers to spare: it keeps one lane offset per load unit, the unit's
+// own row offset included, and all loads of a tile share ONE scalar base (no scalar add per load, two scalar
+// register pairs instead of sixteen).
+constexpr bool LANE_UNIT_OFFSETS = gt::WAVES_PER_SIMD == 1;
+constexpr u32 X_OFFSETS = LANE_UNIT_OFFSETS ? X_UNITS : 2;
+constexpr u32 W_OFFSETS = LANE_UNIT_OFFSETS ? W_UNITS : 2;
+X17_DEV constexpr u32 w_unit_row(u32 r0) {   // weight row that LDS weight row r0 (a multiple of the unit) starts from
+	return gt::WAVE_N * (r0 / gt::WAVE_N) + 16 * ((r0 % gt::WAVE_N) / 32) + 4 * ((r0 % 32) / 8);
+}
 struct LaneOffsets {
-	u32 x_src[2];   // per-lane byte offset into A for a direct-to-LDS load (even / odd load unit)
-	u32 w_src[2];   // per-lane byte offset into B
+	u32 x_src[X_OFFSETS];   // per-lane byte offset into A for a direct-to-LDS load (even / odd load unit, or per unit)
+	u32 w_src[W_OFFSETS];   // per-lane byte offset into B
 	u32 frag_row;   // (lane % 32) * ROW_BYTES
 	u32 half;       // lane / 32
 	u32 swz;        // swizzle key of the fragment row this lane reads
@@ -290,23 +299,30 @@ X17_DEV void load_to_lds_16(u8 *lds_uniform, u8 const *src_uniform, u32 lane_off
 template <u32 U>
 X17_DEV void issue_x_load(u8 const *a_tile, u8 *x_tile, u32 k0, u32 wave, LaneOffsets const &lo) {
 	u8 *x_lds = x_tile + (wave * X_UNITS + U) * UNIT_ROWS * ROW_BYTES;
-	u8 const *x_src = a_tile + (size_t)((wave * X_UNITS + U) * UNIT_ROWS) * K_TOTAL + k0;
-	load_to_lds_16(x_lds, x_src, lo.x_src[U & 1]);
+	if constexpr (LANE_UNIT_OFFSETS) {
+		load_to_lds_16(x_lds, a_tile + (size_t)(wave * X_UNITS * UNIT_ROWS) * K_TOTAL + k0, lo.x_src[U]);
+	} else {
+		u8 const *x_src = a_tile + (size_t)((wave * X_UNITS + U) * UNIT_ROWS) * K_TOTAL + k0;
+		load_to_lds_16(x_lds, x_src, lo.x_src[U & 1]);
+	}
 }
 template <u32 U>
 X17_DEV void issue_w_load(u8 const *b_tile, u8 *w_tile, u32 k0, u32 wave, LaneOffsets const &lo) {
 	u32 r0 = (wave * W_UNITS + U) * UNIT_ROWS;
-	u32 n_uniform = gt::WAVE_N * (r0 / gt::WAVE_N) + 16 * ((r0 % gt::WAVE_N) / 32) + 4 * ((r0 % 32) / 8);
 	u8 *w_lds = w_tile + r0 * ROW_BYTES;
-	u8 const *w_src = b_tile + (size_t)n_uniform * K_TOTAL + k0;
-	load_to_lds_16(w_lds, w_src, lo.w_src[U & 1]);
+	if constexpr (LANE_UNIT_OFFSETS) {
+		load_to_lds_16(w_lds, b_tile + (size_t)w_unit_row(wave * W_UNITS * UNIT_ROWS) * K_TOTAL + k0, lo.w_src[U]);
+	} else {
+		u8 const *w_src = b_tile + (size_t)w_unit_row(r0) * K_TOTAL + k0;
+		load_to_lds_16(w_lds, w_src, lo.w_src[U & 1]);
+	}
 }
 // this wave's share of one token tile / one weight tile of one step
-template <u32 FIRST = 0>
+template <u32 FIRST = 0, u32 LAST = X_UNITS>
 X17_DEV void issue_x_units(u8 const *a_tile, u8 *x_tile, u32 k0, u32 wave, LaneOffsets const &lo) {
-	if constexpr (FIRST < X_UNITS) {
+	if constexpr (FIRST < LAST) {
 		issue_x_load<FIRST>(a_tile, x_tile, k0, wave, lo);
-		issue_x_units<FIRST + 1>(a_tile, x_tile, k0, wave, lo);
+		issue_x_units<FIRST + 1, LAST>(a_tile, x_tile, k0, wave, lo);
 	}
 }
 template <u32 FIRST = 0>
@@ -397,10 +413,14 @@ struct Frags {
 };
 
 X17_DEV void load_frags(Frags &f, u8 const *w_tile, u8 const *x_tile, u32 s, LaneOffsets const &lo) {
-	X17_UNROLL for (u32 c = 0; c < CHUNKS_PER_FRAG; ++c) {
-		u32 kc = CHUNKS_PER_FRAG * (2 * s + lo.half) + c;
-		X17_UNROLL for (int bn = 0; bn < BN; ++bn) f.w[bn][c] = lds_chunk(w_tile, bn * 32 * ROW_BYTES, kc, lo.swz);
-		X17_UNROLL for (int bm = 0; bm < BM; ++bm) f.x[bm][c] = lds_chunk(x_tile, bm * 32 * ROW_BYTES, kc, lo.swz);
+	// in the order the MFMAs of a slice want them: w0, every x, then the other w
+	u32 const kc0 = CHUNKS_PER_FRAG * (2 * s + lo.half);
+	X17_UNROLL for (u32 c = 0; c < CHUNKS_PER_FRAG; ++c) f.w[0][c] = lds_chunk(w_tile, 0, kc0 + c, lo.swz);
+	X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
+		X17_UNROLL for (u32 c = 0; c < CHUNKS_PER_FRAG; ++c) f.x[bm][c] = lds_chunk(x_tile, bm * 32 * ROW_BYTES, kc0 + c, lo.swz);
+	}
+	X17_UNROLL for (int bn = 1; bn < BN; ++bn) {
+		X17_UNROLL for (u32 c = 0; c < CHUNKS_PER_FRAG; ++c) f.w[bn][c] = lds_chunk(w_tile, bn * 32 * ROW_BYTES, kc0 + c, lo.swz);
 	}
 }
 
@@ -468,6 +488,75 @@ X17_DEV void interleave_slice(bool with_reads) {
 	}
 }
 
+// ---- the paced form of a slice (int8 and e4m3 arithmetic): every MFMA is followed by its share of the next
+// fragments' LDS reads and of the tile requests, and nothing may move across the group boundaries, so a
+// wave that has a SIMD to itself for a while keeps the matrix core fed instead of issuing requests in a burst.
+constexpr int MFMAS_PER_SLICE = BN * BM;
+constexpr int READS_PER_SLICE = (BN + BM) * (int)CHUNKS_PER_FRAG;
+
+template <int I>
+X17_DEV void mma_one(Frags const &f, Acc (&acc)[BN][BM]) {
+	constexpr int bn = I / BM, bm = I % BM;
+	if constexpr (MMA == 0) {
+		acc[bn][bm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w[bn][0], f.x[bm][0], acc[bn][bm], 0, 0, 0);
+	} else {
+		v4i wl = f.w[bn][0], wh = f.w[bn][CHUNKS_PER_FRAG - 1];
+		v4i xl = f.x[bm][0], xh = f.x[bm][CHUNKS_PER_FRAG - 1];
+		v8i wf = v8i{wl[0], wl[1], wl[2], wl[3], wh[0], wh[1], wh[2], wh[3]};
+		v8i xf = v8i{xl[0], xl[1], xl[2], xl[3], xh[0], xh[1], xh[2], xh[3]};
+		v16f r = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf, xf, __builtin_bit_cast(v16f, acc[bn][bm]), 0, 0, 0, 0, 0, 0);
+		acc[bn][bm] = __builtin_bit_cast(Acc, r);
+	}
+}
+// read number J of a slice's fragments, in the order the MFMAs want them: w0, every x, then the other w
+template <int J>
+X17_DEV void read_one(Frags &f, u8 const *w_tile, u8 const *x_tile, u32 s, LaneOffsets const &lo) {
+	constexpr int q = J / (int)CHUNKS_PER_FRAG;
+	constexpr u32 c = J % CHUNKS_PER_FRAG;
+	u32 const kc = CHUNKS_PER_FRAG * (2 * s + lo.half) + c;
+	if constexpr (q == 0) {
+		f.w[0][c] = lds_chunk(w_tile, 0, kc, lo.swz);
+	} else if constexpr (q <= BM) {
+		f.x[q - 1][c] = lds_chunk(x_tile, (q - 1) * 32 * ROW_BYTES, kc, lo.swz);
+	} else {
+		f.w[q - BM][c] = lds_chunk(w_tile, (q - BM) * 32 * ROW_BYTES, kc, lo.swz);
+	}
+}
+template <int FIRST, int LAST>
+X17_DEV void read_range(Frags &f, u8 const *w_tile, u8 const *x_tile, u32 s, LaneOffsets const &lo) {
+	if constexpr (FIRST < LAST) {
+		read_one<FIRST>(f, w_tile, x_tile, s, lo);
+		read_range<FIRST + 1, LAST>(f, w_tile, x_tile, s, lo);
+	}
+}
+template <u32 FIRST, u32 LAST>
+X17_DEV void issue_w_range(u8 const *b_tile, u8 *w_tile, u32 k0, u32 wave, LaneOffsets const &lo) {
+	if constexpr (FIRST < LAST) {
+		issue_w_load<FIRST>(b_tile, w_tile, k0, wave, lo);
+		issue_w_range<FIRST + 1, LAST>(b_tile, w_tile, k0, wave, lo);
+	}
+}
+// KIND 0: no requests, 1: token units [FIRST, FIRST + COUNT), 2: weight units [FIRST, FIRST + COUNT)
+template <int I, bool READS, int KIND, u32 FIRST, u32 COUNT>
+X17_DEV void paced_slice(Frags const &cur, Frags &next, u8 const *nw, u8 const *nx, u32 ns, LaneOffsets const &lo,
+                         Acc (&acc)[BN][BM], u8 const *src, u8 *dst, u32 k0, u32 wave) {
+	if constexpr (I < MFMAS_PER_SLICE) {
+		mma_one<I>(cur, acc);
+		if constexpr (READS) {
+			constexpr int R0 = I * READS_PER_SLICE / MFMAS_PER_SLICE, R1 = (I + 1) * READS_PER_SLICE / MFMAS_PER_SLICE;
+			read_range<R0, R1>(next, nw, nx, ns, lo);
+		}
+		constexpr u32 L0 = FIRST + I * COUNT / MFMAS_PER_SLICE, L1 = FIRST + (I + 1) * COUNT / MFMAS_PER_SLICE;
+		if constexpr (KIND == 1) {
+			issue_x_units<L0, L1>(src, dst, k0, wave, lo);
+		} else if constexpr (KIND == 2) {
+			issue_w_range<L0, L1>(src, dst, k0, wave, lo);
+		}
+		__builtin_amdgcn_sched_barrier(0);
+		paced_slice<I + 1, READS, KIND, FIRST, COUNT>(cur, next, nw, nx, ns, lo, acc, src, dst, k0, wave);
+	}
+}
+
 } // namespace
 
 extern "C" __global__ __launch_bounds__(gt::THREADS_PER_BLOCK)
@@ -526,11 +615,24 @@ void kernel(
 	LaneOffsets lo;
 	{
 		u32 j = lane / CHUNKS, p = lane % CHUNKS;     // row inside a load unit, stored chunk position
+		u32 even_odd_x[2], even_odd_w[2];
 		X17_UNROLL for (u32 odd = 0; odd < 2; ++odd) {
 			u32 key = ((odd * UNIT_ROWS + j) >> SWZ_SHIFT) & (CHUNKS - 1);
 			u32 chunk = p ^ key;
-			lo.x_src[odd] = j * K_TOTAL + 16 * chunk;
-			lo.w_src[odd] = ((gt::WAVE_N / 2) * ((j >> 2) & 1) + 4 * (j >> 3) + (j & 3)) * K_TOTAL + 16 * chunk;
+			even_odd_x[odd] = j * K_TOTAL + 16 * chunk;
+			even_odd_w[odd] = ((gt::WAVE_N / 2) * ((j >> 2) & 1) + 4 * (j >> 3) + (j & 3)) * K_TOTAL + 16 * chunk;
+		}
+		if constexpr (LANE_UNIT_OFFSETS) {
+			u32 const w_first = wave * W_UNITS * UNIT_ROWS;
+			X17_UNROLL for (u32 u = 0; u < X_UNITS; ++u) lo.x_src[u] = even_odd_x[u & 1] + u * UNIT_ROWS * K_TOTAL;
+			X17_UNROLL for (u32 u = 0; u < W_UNITS; ++u) {
+				lo.w_src[u] = even_odd_w[u & 1] + (w_unit_row(w_first + u * UNIT_ROWS) - w_unit_row(w_first)) * K_TOTAL;
+			}
+		} else {
+			X17_UNROLL for (u32 odd = 0; odd < 2; ++odd) {
+				lo.x_src[odd] = even_odd_x[odd];
+				lo.w_src[odd] = even_odd_w[odd];
+			}
 		}
 		lo.frag_row = (lane % 32) * ROW_BYTES;
 		lo.half = lane / 32;
@@ -547,6 +649,13 @@ void kernel(
 	// runs.  (a K shorter than the ring cannot prefetch across tiles: each tile then starts with its own prologue)
 	static_assert(XS == WS || WS == 2, "a deeper token ring is supported on top of a two-deep weight ring");
 	constexpr bool CROSS_TILE = K_STEPS >= XS;
+	// Paced form: a step requests its token tile (step + XS - 1, into the position the PREVIOUS step's barrier
+	// freed) during its first slices and its weight tile (step + WS) behind its own barrier, every request behind
+	// an MFMA.  The pattern is the same in every step of every tile -- where nothing is left to fetch the request
+	// is repeated from the tile's start into a position that no step reads again -- so no branch sits between
+	// the MFMAs and the wait before a barrier is always "all but the token tile just requested".
+	// (e4m3 fragments are twice the size: two such waves per SIMD do not fit the pinned order into 256 registers)
+	constexpr bool PACED = MMA != 2 && WS == 2 && XS == 3 && CROSS_TILE && SLICES >= 2 && (MMA == 0 || gt::WAVES_PER_SIMD == 1);
 	u32 const x_off = wm * gt::WAVE_M * ROW_BYTES + lo.frag_row;
 	u32 const w_off = W_RING_OFFSET + wn * gt::WAVE_N * ROW_BYTES + lo.frag_row;
 
@@ -556,14 +665,14 @@ void kernel(
 	u8 const *b_tile = b + (size_t)(tile_n * gt::N_PER_BLOCK) * K_TOTAL;
 	// the first steps of a tile nobody prefetched, in the order the waits of the main loop assume
 	// (token tile s, weight tile s, ..., then the extra token tile of a deeper token ring)
-	auto prologue = [&]() {
+	auto prologue = [&]() __attribute__((always_inline)) {
 		X17_UNROLL for (u32 s = 0; s < WS; ++s) {
 			if (s < K_STEPS) {
 				issue_x_loads(a_tile, smem + s * X_TILE_BYTES, s * gt::K_STEP, wave, lo);
 				issue_w_loads(b_tile, smem + W_RING_OFFSET + s * W_TILE_BYTES, s * gt::K_STEP, wave, lo);
 			}
 		}
-		if constexpr (XS > WS && CROSS_TILE) {
+		if constexpr (XS > WS && CROSS_TILE && !PACED) {
 			issue_x_loads(a_tile, smem + WS * X_TILE_BYTES, WS * gt::K_STEP, wave, lo);
 		}
 		wait_vmcnt<0>();
@@ -603,6 +712,64 @@ void kernel(
 		Frags frags[2];
 		load_frags(frags[0], smem + wb * W_TILE_BYTES + w_off, smem + xb * X_TILE_BYTES + x_off, 0, lo);
 
+		auto paced_k_loop = [&]<bool LOADER>() __attribute__((always_inline)) {
+			constexpr u32 X_SLICES = SLICES >= 4 ? 2 : 1;                 // slices that carry token requests
+			constexpr u32 X_PER_SLICE = X_UNITS / X_SLICES;
+			// (values, not the captured variables: a choice between two captured pointers would keep them in memory)
+			u8 const *const at = a_tile, *const an = a_next, *const bt = b_tile, *const bnx = b_next;
+			bool const hn = has_next;
+			// (no unroll pragma here: with the issue order pinned, unrolling a short loop completely costs no registers,
+			// and the rolled form of this loop spills)
+			for (u32 ks = 0; ks < K_STEPS; ++ks) {
+				u32 const next_xb = xb + 1 == XS ? 0 : xb + 1;
+				u32 const next_wb = wb + 1 == WS ? 0 : wb + 1;
+				u32 const prev_xb = xb == 0 ? XS - 1 : xb - 1;
+				u32 const x_step = ks + XS - 1, w_step = ks + WS;
+				bool const x_here = x_step < K_STEPS, w_here = w_step < K_STEPS;
+				u8 const *lx = (x_here || !hn) ? at : an;
+				u8 const *lw = (w_here || !hn) ? bt : bnx;
+				u32 const x_k0 = (x_here ? x_step : (hn ? x_step - K_STEPS : 0)) * gt::K_STEP;
+				u32 const w_k0 = (w_here ? w_step : (hn ? w_step - K_STEPS : 0)) * gt::K_STEP;
+				u8 *x_dst = smem + prev_xb * X_TILE_BYTES;
+				u8 *w_dst = smem + W_RING_OFFSET + wb * W_TILE_BYTES;
+				u8 const *w_tile = smem + wb * W_TILE_BYTES + w_off;
+				u8 const *x_tile = smem + xb * X_TILE_BYTES + x_off;
+				u8 const *nw_tile = smem + next_wb * W_TILE_BYTES + w_off;
+				u8 const *nx_tile = smem + next_xb * X_TILE_BYTES + x_off;
+				auto slices = [&]<u32 S>(auto &&self) __attribute__((always_inline)) {
+					if constexpr (S + 1 < SLICES) {
+						constexpr int KIND = LOADER && S < X_SLICES ? 1 : 0;
+						paced_slice<0, true, KIND, S * X_PER_SLICE, X_PER_SLICE>(
+							frags[S & 1], frags[(S + 1) & 1], w_tile, x_tile, S + 1, lo, acc, lx, x_dst, x_k0, wave);
+						self.template operator()<S + 1>(self);
+					} else {
+						// the next step's tiles have landed once all but the token tile just requested have;
+						// this wave is done reading this step's tiles
+						wait_vmcnt<X_UNITS>();
+						__builtin_amdgcn_s_waitcnt(0xC07F);
+						__builtin_amdgcn_s_barrier();
+						constexpr int KIND = LOADER ? 2 : 0;
+						if (ks + 1 < K_STEPS) {
+							paced_slice<0, true, KIND, 0, W_UNITS>(
+								frags[S & 1], frags[(S + 1) & 1], nw_tile, nx_tile, 0, lo, acc, lw, w_dst, w_k0, wave);
+						} else {
+							paced_slice<0, false, KIND, 0, W_UNITS>(
+								frags[S & 1], frags[(S + 1) & 1], nw_tile, nx_tile, 0, lo, acc, lw, w_dst, w_k0, wave);
+						}
+					}
+				};
+				slices.template operator()<0>(slices);
+				xb = next_xb;
+				wb = next_wb;
+			}
+		};
+		if constexpr (PACED) {
+			if (WAVES == LOADER_WAVES || wave < LOADER_WAVES) {
+				paced_k_loop.template operator()<true>();
+			} else {
+				paced_k_loop.template operator()<false>();
+			}
+		} else {
 		X17_K_LOOP_PRAGMA
 		for (u32 ks = 0; ks < K_STEPS; ++ks) {
 			u32 const next_xb = xb + 1 == XS ? 0 : xb + 1;
@@ -659,6 +826,7 @@ void kernel(
 			}
 			xb = next_xb;
 			wb = next_wb;
+		}
 		}
 
 	// ---- epilogue.  Lane owns token (32*bm + lane%32) of its wave and raw columns
@@ -768,4 +936,6 @@ void kernel(
 		a_tile = a_next;
 		b_tile = b_next;
 	}
+	// the paced form's last requests go nowhere useful, but they write LDS: they must land before the workgroup ends
+	wait_vmcnt<0>();
 }
