@@ -37,7 +37,7 @@ PEAK_BF16_TFLOPS = 2500.0    # dense bf16
 PEAK_HBM_GBS = 8000.0        # HBM3E
 
 # HBM bytes per ffn_f launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), or None
-FFN_F_TRAFFIC_BYTES = int((196704 * 2.0 + 65536 * 1.0) * 1024)
+FFN_F_TRAFFIC_BYTES = int((198254 * 2.0 + 65536 * 1.0) * 1024)
 # HBM bytes one decode launch of config 5 fetches (profiles/attn_decode_i8_config5.txt): all K rows plus the
 # V rows with a nonzero 8-bit probability -- about half of the 2 GiB cache for the synthetic Gaussian codes
 DECODE_TRAFFIC_BYTES = int(529500 * 2.0 * 1024)
