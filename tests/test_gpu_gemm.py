@@ -192,6 +192,29 @@ def test_fp8_geglu(dev, m, k, n):
 	assert neq < 5e-3 and beyond == 0.0, (neq, beyond)
 
 
+def test_more_tiles_than_workgroups_with_the_shortest_ring_of_three(dev):
+	"""K = 384 is three K steps: the first K the three-deep token ring is built for, where every request of a tile's
+	last two steps already belongs to the workgroup's NEXT tile.  260 tiles on at most 256 persistent workgroups:
+	four of them walk two tiles, the others end after one (their last requests go to a ring position nobody reads)."""
+	m, k, n = 256 * 65, 384, 1024
+	rng = rng_for("ring3", m, k, n)
+	a, b = i8_codes(rng, (m, k)), i8_codes(rng, (n, k))
+	kern = recipes.attn_q_kernel(dev, k, n)
+	c = X.Tensor(dev, (m, n), X.INT8)
+	kern.launch(_up(dev, a, X.INT8), _up(dev, b, X.INT8), c)
+	want = S.epilogue_scale(S.gemm_i32(a, b), 1.0 / math.sqrt(k) / 64.0, 8.0)
+	assert np.array_equal(c.download(), want)
+	# the same walk in the four-wave e4m3 form (130 x 2 tiles)
+	m, n = 256 * 130, 512
+	a8, b8 = e4m3_bytes(rng, (m, k)), e4m3_bytes(rng, (n, k))
+	want = S.epilogue_geglu(S.gemm_f32_seq(a8, True, b8, True), 1.0 / math.sqrt(k), 1.0, S.STORE_E4M3)
+	kern = recipes.ffn_f_f8_kernel(dev, k, n, True)
+	c = X.Tensor(dev, (m, n // 2), X.E4M3)
+	kern.launch(_up(dev, a8, X.E4M3), _up(dev, b8, X.E4M3), c)
+	neq, beyond = e4m3_compare(c.download(), want)
+	assert neq < 5e-3 and beyond == 0.0, (neq, beyond)
+
+
 def _absmax_quantize(x, axis):
 	"""Symmetric int8 with scale = absmax / 127 along `axis` (f32 arithmetic)."""
 	x = x.astype(np.float32)

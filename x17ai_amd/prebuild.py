@@ -37,6 +37,8 @@ def _specs():
 		add(("ffn_y", n // 2, k, True, E4M3, INT8))
 	for k, n in ((512, 256), (4096, 512)):
 		add(("ffn_f_f8", k, n, True))
+	add(("attn_q", 384, 1024))           # the shortest K with the deeper token ring, more tiles than workgroups
+	add(("ffn_f_f8", 384, 512, True))
 	# ---- tests/test_gpu_attn.py
 	for h, hd in ((4, 32), (2, 64), (2, 128), (8, 64)):
 		add(("attn", h, hd, True))
