@@ -14,7 +14,7 @@ import pytest
 import x17ai_amd as X
 from x17ai_amd import recipes
 from oracle import strict as S
-from tests.gpu_common import i8_codes, rng_for
+from tests.gpu_common import e4m3_bytes, e4m3_compare, i8_codes, rng_for
 
 pytestmark = pytest.mark.gpu
 
@@ -58,6 +58,35 @@ def test_config2_ffn_pair_sampled_rows(dev):
 	assert np.array_equal(got_y[rows], want_y)
 	# every tile wrote something plausible: no output row is left at the allocator's fill
 	assert np.count_nonzero(np.abs(got_f.astype(np.int32)).sum(axis=1) == 0) == 0
+
+
+def test_config3_fp8_ffn_pair_sampled_rows(dev):
+	"""benchmark config 3: tokens 16384, d_model 4096, d_ff 16384, e4m3 x e4m3 with f32 accumulation (four waves of
+	128 x 128 per workgroup, eight and four tiles per workgroup): ffn_f (GeGLU -> e4m3) and ffn_y (gated residual ->
+	e4m3), strict builds, 48 sampled token rows of each against the oracle.  The matrix cores add the products of a
+	K slice in their own order, the oracle one by one: outputs may sit one e4m3 step apart in under 0.5 % of the
+	elements and never further."""
+	m, d, f = 16384, 4096, 16384
+	rng = rng_for("full-config3")
+	x, w1, w2 = e4m3_bytes(rng, (m, d)), e4m3_bytes(rng, (2 * f, d)), e4m3_bytes(rng, (2 * d, f))
+	res = i8_codes(rng, (m, d))
+	k1 = recipes.ffn_f_f8_kernel(dev, d, 2 * f, True)
+	k2 = recipes.ffn_y_kernel(dev, d, f, True, X.E4M3, X.E4M3)
+	ft = X.Tensor(dev, (m, f), X.E4M3)
+	yt = X.Tensor(dev, (m, d), X.E4M3)
+	k1.launch(_up(dev, x, X.E4M3), _up(dev, w1, X.E4M3), ft)
+	k2.launch(ft, _up(dev, w2, X.E4M3), yt, _up(dev, res, X.INT8))
+	got_f, got_y = ft.download(), yt.download()
+	rows = _sample_rows(rng, m, 48)
+	want_f = S.epilogue_geglu(S.gemm_f32_seq(x[rows], True, w1, True), 1.0 / math.sqrt(d), 1.0, S.STORE_E4M3)
+	neq, beyond = e4m3_compare(got_f[rows], want_f)
+	assert neq < 5e-3 and beyond == 0.0, (neq, beyond)
+	inp_y = math.sqrt(recipes.GELU_VAR_FIX_2 / f)
+	want_y = S.epilogue_residual(S.gemm_f32_seq(got_f[rows], True, w2, True), res[rows], inp_y, 1.0, S.STORE_E4M3)
+	neq, beyond = e4m3_compare(got_y[rows], want_y)
+	assert neq < 5e-3 and beyond == 0.0, (neq, beyond)
+	# every tile wrote: no output row of f is all zero bytes
+	assert np.count_nonzero((got_f != 0).sum(axis=1) == 0) == 0
 
 
 def test_config2_literal_per_token_per_channel_scales(dev):

@@ -66,6 +66,8 @@ def _specs():
 		add(("decode", 32, 128, 4096, strict))
 	add(("ffn_f_f8", 4096, 32768, False))
 	add(("ffn_y", 4096, 16384, False, E4M3, E4M3))
+	add(("ffn_f_f8", 4096, 32768, True))                 # tests/test_gpu_fullsize.py: config 3, strict builds
+	add(("ffn_y", 4096, 16384, True, E4M3, E4M3))
 	add(("attn_q", 2048, 2048))
 	add(("attn_kv", 2048, 4096, 128))
 	add(("attn", 16, 128, False))
