@@ -190,9 +190,7 @@ def extras(dev, X, recipes):
 	# ---- config 3: all-fp8 FFN, tokens=16384, d_model=4096, d_ff=16384
 	M3, D3, F3 = 16384, 4096, 16384
 	def e4m3_rand(shape):
-		# valid reference-dialect e4m3 bytes with magnitudes in [0.25, 3.75]: exponent field 5..8
-		b = (rng.integers(5, 9, size=shape, dtype=np.uint8) << 3) | rng.integers(0, 8, size=shape, dtype=np.uint8)
-		return b | (rng.integers(0, 2, size=shape, dtype=np.uint8) << 7)
+		return _rand_e4m3(rng, shape)
 	x3 = X.Tensor.from_numpy(dev, e4m3_rand((M3, D3)), X.E4M3)
 	w13 = X.Tensor.from_numpy(dev, e4m3_rand((2 * F3, D3)), X.E4M3)
 	f3 = X.Tensor(dev, (M3, F3), X.E4M3)
@@ -345,6 +343,12 @@ def extras(dev, X, recipes):
 	return out
 
 
+def _rand_e4m3(rng, shape):
+	"""valid reference-dialect e4m3 bytes with magnitudes in [0.25, 3.75]: exponent field 5..8"""
+	b = (rng.integers(5, 9, size=shape, dtype=np.uint8) << 3) | rng.integers(0, 8, size=shape, dtype=np.uint8)
+	return b | (rng.integers(0, 2, size=shape, dtype=np.uint8) << 7)
+
+
 def single(dev, X, recipes, name, iters):
 	"""One kernel of one benchmark workload, launched `iters` times: what the rocprofv3 summaries under
 	profiles/ are taken from (every code object exports the entry `kernel`, so a profile of several
@@ -358,6 +362,13 @@ def single(dev, X, recipes, name, iters):
 		c = X.Tensor(dev, (M, F), X.INT8)
 		k = recipes.ffn_f_kernel(dev, D, 2 * F, False, X.INT8)
 		fn, work, unit = (lambda: k.launch(a, b, c)), k.n_ops(a, b) / 1e12, "TOPS"
+	elif name == "ffn_f_f8_config3":
+		M, D3, F3 = 16384, 4096, 16384
+		a = X.Tensor.from_numpy(dev, _rand_e4m3(rng, (M, D3)), X.E4M3)
+		b = X.Tensor.from_numpy(dev, _rand_e4m3(rng, (2 * F3, D3)), X.E4M3)
+		c = X.Tensor(dev, (M, F3), X.E4M3)
+		k = recipes.ffn_f_f8_kernel(dev, D3, 2 * F3, False)
+		fn, work, unit = (lambda: k.launch(a, b, c)), k.n_ops(a, b) / 1e12, "TFLOP/s"
 	elif name == "ffn_y_f8_config4":
 		M = 32768
 		a = X.Tensor.from_numpy(dev, rng.integers(0x20, 0x50, (M, F), dtype=np.uint8), X.E4M3)
@@ -404,7 +415,7 @@ def single(dev, X, recipes, name, iters):
 	                  "rate": work / med, "unit": unit}))
 
 
-ONLY_TARGETS = ("ffn_f_config2", "ffn_y_f8_config4", "attn_config4", "attn_config5", "decode_config5", "rms_norm_config4")
+ONLY_TARGETS = ("ffn_f_config2", "ffn_f_f8_config3", "ffn_y_f8_config4", "attn_config4", "attn_config5", "decode_config5", "rms_norm_config4")
 
 
 def main():
