@@ -737,18 +737,14 @@ std::unique_ptr<GemmKernel> GemmKernel::create(std::shared_ptr<HipDevice> device
 	common << "#define X17_EPILOGUE " << kind << "\n";
 	common << "#define X17_STORE " << (g.c_dtype == DType::E4m3 ? 1 : (g.c_dtype == DType::Bf16 ? 2 : 0)) << "\n";
 	common << "#define X17_STRICT_MATH " << (strict_math ? 1 : 0) << "\n";
-	// e4m3 activations x int8 weights run on the f16 matrix cores with both operands widened in registers, and
-	// widening an int8 byte costs 2.5 times what an e4m3 byte costs.  A weight row is widened by every wave that
-	// shares it, so these kernels use waves of 128 tokens x 64 columns (two waves per weight row, four per
-	// token row) instead of 64 x 128.  (Scale, GeGLU and Residual writers; the others are written for 128 columns.)
-	if (g.a.dtype == DType::E4m3 && g.b.dtype == DType::Int8 && kind <= 2) {
-		common << "#define X17_GEMM_WAVES_M 2\n#define X17_GEMM_WAVES_N 4\n";
-	}
-	// e4m3 x e4m3: four waves of 128 x 128, one per SIMD with all 512 registers (accumulators in the second half of
-	// the register file).  With the issue order of a K step pinned, a lone wave keeps the matrix core busier than
-	// two waves that take turns at the barrier, and the fragments (32 bytes per lane and operand row) of two such
-	// waves would not fit: measured 7-8 % faster than eight waves of 64 x 128.
-	if (g.a.dtype == DType::E4m3 && g.b.dtype == DType::E4m3) {
+	// One wavefront per SIMD (four waves of 128 x 128, accumulators in the second half of the register file) wherever
+	// an operand is e4m3.  e4m3 x e4m3: with the issue order of a K step pinned, a lone wave keeps the matrix core
+	// busier than two waves that take turns at the barrier, and the fragments (32 bytes per lane and operand row) of
+	// two such waves would not fit: 7-8 % faster than eight waves of 64 x 128.  e4m3 x int8 (f16 matrix cores, both
+	// operands widened in registers): a weight row is widened by two waves and a token row by two, 3.5 vector
+	// instructions per MFMA instead of 6.4, issued a piece behind each MFMA one round ahead: 7-8 % faster than eight
+	// waves of 128 x 64 with the compiler's schedule.
+	if (g.a.dtype == DType::E4m3 || g.b.dtype == DType::E4m3) {
 		common << "#define X17_GEMM_WAVES_M 2\n#define X17_GEMM_WAVES_N 2\n";
 	}
 

@@ -558,6 +558,80 @@ X17_DEV void paced_slice(Frags const &cur, Frags &next, u8 const *nw, u8 const *
 	}
 }
 
+// ---- the paced form for the mixed arithmetic (e4m3 x int8 widened to f16; one wave per SIMD).  A slice of 32 bytes
+// of K is two rounds of BN x BM f16 MFMAs (K = 16 each).  The operands of a round are widened one round ahead, a
+// piece of four bytes behind each MFMA, so the conversions run in the shadow of the matrix core instead of in
+// front of it; the raw fragments of the next slice are read during the first round, tiles requested in the second.
+struct Wide {
+	v8h w[BN];
+	v8h x[BM];
+};
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+
+// four 8-bit values -> four f16, exact (see widen8)
+X17_DEV v4h widen4(u32 word, int kind) {
+	v2h lo2, hi2;
+	if (kind == 1) {
+		lo2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(word, 1.0f, false);
+		hi2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(word, 1.0f, true);
+	} else {
+		v2h const bias = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+		u32 const u = word ^ 0x80808080u;
+		lo2 = __builtin_bit_cast(v2h, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) + bias;
+		hi2 = __builtin_bit_cast(v2h, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) + bias;
+	}
+	return v4h{lo2[0], lo2[1], hi2[0], hi2[1]};
+}
+constexpr int WIDEN_PIECES = 2 * (BN + BM);      // per round: every fragment in two pieces of four bytes
+// piece P of the operands of round H (0 / 1: bytes 0..7 / 8..15 of the lane's 16) of the raw fragments `f`,
+// fragments in the order the MFMAs want them: w0, every x, then the other w
+template <int P, int H>
+X17_DEV void widen_piece(Wide &wd, Frags const &f) {
+	constexpr int q = P / 2, p = P % 2, dw = 2 * H + p;
+	if constexpr (q == 0 || q > BM) {
+		constexpr int bn = q == 0 ? 0 : q - BM;
+		v4h const r = widen4((u32)f.w[bn][0][dw], B_KIND);
+		X17_UNROLL for (int i = 0; i < 4; ++i) wd.w[bn][4 * p + i] = r[i];
+	} else {
+		v4h const r = widen4((u32)f.x[q - 1][0][dw], A_KIND);
+		X17_UNROLL for (int i = 0; i < 4; ++i) wd.x[q - 1][4 * p + i] = r[i];
+	}
+}
+template <int FIRST, int LAST, int H>
+X17_DEV void widen_range(Wide &wd, Frags const &f) {
+	if constexpr (FIRST < LAST) {
+		widen_piece<FIRST, H>(wd, f);
+		widen_range<FIRST + 1, LAST, H>(wd, f);
+	}
+}
+// One round.  NEXT_H < 0: nothing to widen (the tile's last round); else the next round's operands are round NEXT_H
+// of `raw`.  READS: the raw fragments `rd` of slice `ns` of tiles (nw, nx) are read behind the first MFMAs.
+// KIND / FIRST / COUNT: tile requests as in paced_slice.
+template <int I, int NEXT_H, bool READS, int KIND, u32 FIRST, u32 COUNT>
+X17_DEV void mixed_round(Wide const &cur, Wide &nxt, Frags const &raw, Frags &rd, u8 const *nw, u8 const *nx, u32 ns,
+                         LaneOffsets const &lo, Acc (&acc)[BN][BM], u8 const *src, u8 *dst, u32 k0, u32 wave) {
+	if constexpr (I < MFMAS_PER_SLICE) {
+		constexpr int bn = I / BM, bm = I % BM;
+		v16f const r = __builtin_amdgcn_mfma_f32_32x32x16_f16(cur.w[bn], cur.x[bm], __builtin_bit_cast(v16f, acc[bn][bm]), 0, 0, 0);
+		acc[bn][bm] = __builtin_bit_cast(Acc, r);
+		if constexpr (NEXT_H >= 0) {
+			widen_range<I * WIDEN_PIECES / MFMAS_PER_SLICE, (I + 1) * WIDEN_PIECES / MFMAS_PER_SLICE, NEXT_H>(nxt, raw);
+		}
+		if constexpr (READS) {
+			constexpr int R0 = I * READS_PER_SLICE / MFMAS_PER_SLICE, R1 = (I + 1) * READS_PER_SLICE / MFMAS_PER_SLICE;
+			read_range<R0, R1>(rd, nw, nx, ns, lo);
+		}
+		constexpr u32 L0 = FIRST + I * COUNT / MFMAS_PER_SLICE, L1 = FIRST + (I + 1) * COUNT / MFMAS_PER_SLICE;
+		if constexpr (KIND == 1) {
+			issue_x_units<L0, L1>(src, dst, k0, wave, lo);
+		} else if constexpr (KIND == 2) {
+			issue_w_range<L0, L1>(src, dst, k0, wave, lo);
+		}
+		__builtin_amdgcn_sched_barrier(0);
+		mixed_round<I + 1, NEXT_H, READS, KIND, FIRST, COUNT>(cur, nxt, raw, rd, nw, nx, ns, lo, acc, src, dst, k0, wave);
+	}
+}
+
 } // namespace
 
 extern "C" __global__ __launch_bounds__(gt::THREADS_PER_BLOCK)
@@ -656,7 +730,7 @@ void kernel(
 	// is repeated from the tile's start into a position that no step reads again -- so no branch sits between
 	// the MFMAs and the wait before a barrier is always "all but the token tile just requested".
 	// (e4m3 fragments are twice the size: two such waves per SIMD do not fit the pinned order into 256 registers)
-	constexpr bool PACED = MMA != 2 && WS == 2 && XS == 3 && CROSS_TILE && SLICES >= 2 && (MMA == 0 || gt::WAVES_PER_SIMD == 1);
+	constexpr bool PACED = WS == 2 && XS == 3 && CROSS_TILE && SLICES >= 2 && (MMA == 0 || gt::WAVES_PER_SIMD == 1);
 	u32 const x_off = wm * gt::WAVE_M * ROW_BYTES + lo.frag_row;
 	u32 const w_off = W_RING_OFFSET + wn * gt::WAVE_N * ROW_BYTES + lo.frag_row;
 
@@ -712,6 +786,10 @@ void kernel(
 		// (step 0 of this tile is visible: the wait and the barrier were the previous tile's last ones)
 		Frags frags[2];
 		load_frags(frags[0], smem + wb * W_TILE_BYTES + w_off, smem + xb * X_TILE_BYTES + x_off, 0, lo);
+		[[maybe_unused]] Wide wide[2];
+		if constexpr (PACED && MMA == 2) {
+			widen_range<0, WIDEN_PIECES, 0>(wide[0], frags[0]);      // (the only conversions of a tile no MFMA covers)
+		}
 
 		auto paced_k_loop = [&]<bool LOADER>() __attribute__((always_inline)) {
 			constexpr u32 X_SLICES = SLICES >= 4 ? 2 : 1;                 // slices that carry token requests
@@ -738,7 +816,30 @@ void kernel(
 				u8 const *nw_tile = smem + next_wb * W_TILE_BYTES + w_off;
 				u8 const *nx_tile = smem + next_xb * X_TILE_BYTES + x_off;
 				auto slices = [&]<u32 S>(auto &&self) __attribute__((always_inline)) {
-					if constexpr (S + 1 < SLICES) {
+					if constexpr (MMA == 2) {
+						// first round: the operands of the second round are widened from the same raw fragments, the
+						// next slice's raw fragments are read (behind the step's barrier when they belong to the next
+						// step); second round: the next slice's first operands are widened, tiles are requested
+						constexpr bool LAST = S + 1 == SLICES;
+						constexpr int KIND = !LOADER ? 0 : (LAST ? 2 : (S < X_SLICES ? 1 : 0));
+						constexpr u32 FIRST = LAST ? 0 : S * X_PER_SLICE, COUNT = LAST ? W_UNITS : X_PER_SLICE;
+						u8 const *src = LAST ? lw : lx;
+						u8 *dst = LAST ? w_dst : x_dst;
+						u32 const k0 = LAST ? w_k0 : x_k0;
+						if constexpr (LAST) {
+							wait_vmcnt<X_UNITS>();
+							__builtin_amdgcn_s_waitcnt(0xC07F);
+							__builtin_amdgcn_s_barrier();
+							// (the same code in a tile's last step, where what it reads and widens is never used: two
+							// copies of the rounds would have to agree on where 256 accumulators live when they meet)
+							mixed_round<0, 1, true, 0, 0, 0>(wide[0], wide[1], frags[S & 1], frags[(S + 1) & 1], nw_tile, nx_tile, 0, lo, acc, src, dst, k0, wave);
+							mixed_round<0, 0, false, KIND, FIRST, COUNT>(wide[1], wide[0], frags[(S + 1) & 1], frags[S & 1], nw_tile, nx_tile, 0, lo, acc, src, dst, k0, wave);
+						} else {
+							mixed_round<0, 1, true, 0, 0, 0>(wide[0], wide[1], frags[S & 1], frags[(S + 1) & 1], w_tile, x_tile, S + 1, lo, acc, src, dst, k0, wave);
+							mixed_round<0, 0, false, KIND, FIRST, COUNT>(wide[1], wide[0], frags[(S + 1) & 1], frags[S & 1], w_tile, x_tile, S + 1, lo, acc, src, dst, k0, wave);
+							self.template operator()<S + 1>(self);
+						}
+					} else if constexpr (S + 1 < SLICES) {
 						constexpr int KIND = LOADER && S < X_SLICES ? 1 : 0;
 						paced_slice<0, true, KIND, S * X_PER_SLICE, X_PER_SLICE>(
 							frags[S & 1], frags[(S + 1) & 1], w_tile, x_tile, S + 1, lo, acc, lx, x_dst, x_k0, wave);
@@ -836,6 +937,14 @@ void kernel(
 	u32 const n0 = tile_n * gt::N_PER_BLOCK + wn * gt::WAVE_N + LANE_COLS * lo.half;
 
 	X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
+		if constexpr (gt::WAVES_PER_SIMD == 1) {
+			// Accumulators in the second half of the register file (where the vector ALU cannot read them) are copied
+			// out row by row: pinning the later rows where they are keeps the register allocator from copying all
+			// 256 out at once behind the K loop, which leaves no register for anything else.
+			X17_UNROLL for (int later = bm + 1; later < BM; ++later) {
+				X17_UNROLL for (int bn = 0; bn < BN; ++bn) asm volatile("" : "+a"(acc[bn][later]));
+			}
+		}
 		u32 row = row0 + 32 * bm;
 		f32 x[LANE_COLS];
 		X17_UNROLL for (int bn = 0; bn < BN; ++bn) {
