@@ -156,7 +156,7 @@ def test_mixed_e4m3_i8_residual(dev, m, k, n):
 
 @pytest.mark.parametrize("geglu", [False, True])
 def test_mixed_e4m3_i8_scale_and_geglu(dev, geglu):
-	"""The e4m3 x int8 operand mix (waves of 128 tokens x 64 columns) under the Scale and GeGLU writers."""
+	"""The e4m3 x int8 operand mix under the Scale and GeGLU writers (K of eight steps: the paced rounds, fully unrolled)."""
 	m, k, n = 512, 1024, 512
 	rng = rng_for("mixed-writers", geglu)
 	a = e4m3_bytes(rng, (m, k), 0.6)

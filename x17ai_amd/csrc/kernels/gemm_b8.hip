@@ -7,9 +7,9 @@
 //
 // Design, MI355X-first (nothing here is derived from the SM80 kernel):
 //   * One workgroup = a 256 (tokens) x 256 (raw columns) output tile, by default 8 wavefronts of
-//     64 x 128 (two per SIMD); gemm_tile.h can also build 8 wavefronts of 128 x 64 (the mixed e4m3 x int8
-//     kernels: fewer waves then widen the same weight row) or 4 wavefronts of 128 x 128 (a 4 x 4 grid of
-//     32x32 MFMA blocks, 256 accumulator registers per lane, one wavefront per SIMD: the e4m3 x e4m3 kernels).
+//     64 x 128 (two per SIMD); gemm_tile.h can also build 8 wavefronts of 128 x 64 or 4 wavefronts of 128 x 128
+//     (a 4 x 4 grid of 32x32 MFMA blocks, 256 accumulator registers per lane, one wavefront per SIMD: what the
+//     host picks whenever an operand is e4m3).
 //   * The WEIGHTS are the MFMA "A" operand and the TOKENS the "B" operand, i.e. the matrix
 //     cores compute C^T.  A lane then owns one token and, per MFMA block, 16 output columns;
 //     weight rows are permuted on their way into LDS so that those are 64 (32 for 64-column waves)
@@ -20,7 +20,8 @@
 //     rings of LDS tiles (gemm_tile.h: K_STEP bytes of K per step; by default three token tiles and two
 //     weight tiles of 32 KB, which is all 160 KB of a compute unit), one barrier per step;
 //     16-byte chunks are XOR-swizzled so that ds_read_b128 is conflict-free.  In the int8 and e4m3 kernels the
-//     issue order of a K step is pinned: each MFMA is followed by its share of the LDS reads and tile requests.
+//     issue order of a K step is pinned: each MFMA is followed by its share of the LDS reads and tile requests
+//     (and, in the mixed arithmetic, of the next round's conversions to f16).
 //   * int8: v_mfma_i32_32x32x32_i8.  e4m3 x e4m3: v_mfma_f32_32x32x64_f8f6f4.  Mixed
 //     e4m3 x int8: both widened exactly to f16 in registers, v_mfma_f32_32x32x16_f16
 //     (int8 codes need 7 significand bits, e4m3 has 4; every e4m3 value is a normal f16).
