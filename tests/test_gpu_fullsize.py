@@ -89,6 +89,35 @@ def test_config3_fp8_ffn_pair_sampled_rows(dev):
 	assert np.count_nonzero((got_f != 0).sum(axis=1) == 0) == 0
 
 
+def test_repeated_launches_give_the_same_bytes(dev):
+	"""The LDS rings are recycled behind one barrier per K step and the tile requests run ahead across tile
+	boundaries: an ordering mistake there would show as output that depends on timing.  Each arithmetic at a size
+	where every workgroup walks eight tiles, launched eight times back to back: every output equals the first."""
+	rng = rng_for("repeat")
+	m = 8192
+	cases = (
+		("int8", recipes.ffn_f_kernel(dev, 2048, 16384, False, X.INT8), i8_codes(rng, (m, 2048)), X.INT8,
+		 i8_codes(rng, (16384, 2048)), X.INT8, (m, 8192), X.INT8, None),
+		("e4m3", recipes.ffn_f_f8_kernel(dev, 4096, 32768, False), e4m3_bytes(rng, (m, 4096)), X.E4M3,
+		 e4m3_bytes(rng, (32768, 4096)), X.E4M3, (m, 16384), X.E4M3, None),
+		("e4m3 x int8", recipes.ffn_y_kernel(dev, 2048, 8192, False), e4m3_bytes(rng, (m, 8192)), X.E4M3,
+		 i8_codes(rng, (4096, 8192)), X.INT8, (m, 2048), X.E4M3, i8_codes(rng, (m, 2048))),
+	)
+	for name, kern, a, a_dt, b, b_dt, out_shape, out_dt, res in cases:
+		at, bt = _up(dev, a, a_dt), _up(dev, b, b_dt)
+		rt = None if res is None else _up(dev, res, X.INT8)
+		outs = [X.Tensor(dev, out_shape, out_dt) for _ in range(8)]
+		for o in outs:
+			if rt is None:
+				kern.launch(at, bt, o)
+			else:
+				kern.launch(at, bt, o, rt)
+		first = outs[0].download()
+		assert np.count_nonzero(first) > first.size // 2, name
+		for i, o in enumerate(outs[1:], 1):
+			assert np.array_equal(o.download(), first), (name, i)
+
+
 def test_config2_literal_per_token_per_channel_scales(dev):
 	"""benchmark config 2 as worded: x ~ N(0,1) per-token int8 (absmax / 127), W1 [2048 x 8192 (x2 gated)] and
 	W2 [8192 x 2048] ~ N(0, 1/sqrt(fan_in)) per-output-channel int8, int32 accumulate, fused dequantisation +
