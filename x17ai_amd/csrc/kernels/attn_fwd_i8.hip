@@ -489,9 +489,9 @@ void kernel(
 			u16 *o_row = reinterpret_cast<u16 *>(out) + (row_base + qi) * O_STRIDE + (size_t)head * HD;
 			X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
 				X17_UNROLL for (int g = 0; g < 4; ++g) {
-					u32 b[4];
-					X17_UNROLL for (int e = 0; e < 4; ++e) b[e] = f32_to_bf16_rne((o_acc[db][4 * g + e] * inv) * head_out_scale);
-					v2u pair = {b[0] | (b[1] << 16), b[2] | (b[3] << 16)};
+					f32 b[4];
+					X17_UNROLL for (int e = 0; e < 4; ++e) b[e] = (o_acc[db][4 * g + e] * inv) * head_out_scale;
+					v2u pair = {pack2_bf16_rne(b[0], b[1]), pack2_bf16_rne(b[2], b[3])};
 					*reinterpret_cast<v2u *>(o_row + 32 * db + 8 * g + 4 * half) = pair;
 				}
 			}

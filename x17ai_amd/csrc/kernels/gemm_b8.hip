@@ -218,9 +218,7 @@ struct DequantEpilogue {
 				v4u pack;
 				X17_UNROLL for (int w = 0; w < 4; ++w) {
 					int j = 8 * v + 2 * w;
-					u32 lo = f32_to_bf16_rne(GeGluEpilogue::gated(t[2 * j], t[2 * j + 1]));
-					u32 hi = f32_to_bf16_rne(GeGluEpilogue::gated(t[2 * j + 2], t[2 * j + 3]));
-					pack[w] = lo | (hi << 16);
+					pack[w] = pack2_bf16_rne(GeGluEpilogue::gated(t[2 * j], t[2 * j + 1]), GeGluEpilogue::gated(t[2 * j + 2], t[2 * j + 3]));
 				}
 				*reinterpret_cast<v4u *>(dst + 16 * v) = pack;
 			}
@@ -230,7 +228,7 @@ struct DequantEpilogue {
 				v4u pack;
 				X17_UNROLL for (int w = 0; w < 4; ++w) {
 					int j = 8 * v + 2 * w;
-					pack[w] = f32_to_bf16_rne(t[j]) | (f32_to_bf16_rne(t[j + 1]) << 16);
+					pack[w] = pack2_bf16_rne(t[j], t[j + 1]);
 				}
 				*reinterpret_cast<v4u *>(dst + 16 * v) = pack;
 			}

@@ -95,6 +95,13 @@ X17_DEV u32 f32_to_bf16_rne(f32 v) {
 	u32 b = f2u(v);
 	return (b + 0x7FFFu + ((b >> 16) & 1u)) >> 16;
 }
+// Two of them packed into one word, `lo` in the low half: the gfx950 packed conversion (one instruction for the
+// pair; round to nearest even like the above).
+X17_DEV u32 pack2_bf16_rne(f32 lo, f32 hi) {
+	typedef float pair_f32 __attribute__((ext_vector_type(2)));
+	typedef __bf16 pair_bf16 __attribute__((ext_vector_type(2)));
+	return __builtin_bit_cast(u32, __builtin_convertvector(pair_f32{lo, hi}, pair_bf16));
+}
 
 // Four FixedI8 codes packed into one word (a in the low byte).  Same values as f32_to_fixedi8:
 // clamp, then add 1.5 * 2^23 -- the add rounds to an integer, ties to even, exactly like rint, and
