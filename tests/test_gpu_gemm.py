@@ -192,6 +192,33 @@ def test_fp8_geglu(dev, m, k, n):
 	assert neq < 5e-3 and beyond == 0.0, (neq, beyond)
 
 
+def test_e4m3_store_keeps_the_dialect_over_the_whole_range(dev):
+	"""GeGLU outputs from far below the smallest e4m3 magnitude to far above 448.  The hardware-transcendental build
+	stores through the gfx950 conversion instruction: it must still produce the reference's dialect (no subnormal
+	codes, no negative zero, no NaN code, saturation at +-448) and sit within one grid step of the strict build,
+	which equals the oracle bit for bit."""
+	m, k, n = 256, 128, 256
+	rng = rng_for("e4m3-range")
+	a, b = i8_codes(rng, (m, k)), i8_codes(rng, (n, k))
+	want = S.epilogue_geglu(S.gemm_i32(a, b), 1.0 / 32.0, 1.0, S.STORE_E4M3)
+	assert np.mean((want & 0x7F) == 0x7E) > 0.01 and np.mean(want == 0) > 0.05
+	cfg = X.GemmConfig(X.GemmInputConfig(X.INT8, k, None, False), X.GemmInputConfig(X.INT8, k, n, True), X.E4M3)
+	got = {}
+	for mode, strict in (("strict", True), ("fast", False)):
+		kern = X.GemmKernel(dev, f"e4m3_range-{mode}", cfg, X.GeGluConfig(1.0 / 32.0, 1.0), strict)
+		c = X.Tensor(dev, (m, n // 2), X.E4M3)
+		kern.launch(_up(dev, a, X.INT8), _up(dev, b, X.INT8), c)
+		got[mode] = c.download()
+	assert np.array_equal(got["strict"], want)
+	fast = got["fast"]
+	assert not np.any((fast & 0x7F) == 0x7F)                                   # NaN code
+	assert not np.any(((fast & 0x78) == 0) & (fast != 0))                      # subnormal codes and -0
+	neq, beyond = e4m3_compare(fast, want)
+	assert neq < 5e-3 and beyond == 0.0, (neq, beyond)
+	sat = (want & 0x7F) == 0x7E
+	assert np.mean(fast[sat] != want[sat]) < 5e-3
+
+
 def test_more_tiles_than_workgroups_with_the_shortest_ring_of_three(dev):
 	"""K = 384 is three K steps: the first K the three-deep token ring is built for, where every request of a tile's
 	last two steps already belongs to the workgroup's NEXT tile.  260 tiles on at most 256 persistent workgroups:

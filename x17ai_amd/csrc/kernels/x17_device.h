@@ -117,9 +117,28 @@ X17_DEV u32 pack4_fixedi8(f32 a, f32 b, f32 c, f32 d) {
 	return lo | hi;
 }
 
+// The same encoder on the gfx950 conversion instruction, for the hardware-transcendental builds: magnitudes below
+// the reference's threshold (1.9375 * 2^-7) are zeroed first (the instruction would produce subnormal codes, the
+// reference's dialect has none), the rest is clamped to +-448 (the instruction answers overflow with NaN) and
+// converted two at a time.  One difference remains: a value exactly half way between two e4m3 neighbours goes to
+// the even one here and away from zero in the reference's encoder (one f32 in 2^20 of a binade).
+X17_DEV f32 e4m3_flush_clamp(f32 v) {
+	f32 const kept = __builtin_fabsf(v) < 0.01513671875f ? 0.0f : v;          // 1.9375 * 2^-7 (bits 0x3C780000)
+	return __builtin_amdgcn_fmed3f(kept, -448.0f, 448.0f);
+}
+X17_DEV u32 pack4_e4m3_hw(f32 a, f32 b, f32 c, f32 d) {
+	int w = __builtin_amdgcn_cvt_pk_fp8_f32(e4m3_flush_clamp(a), e4m3_flush_clamp(b), 0, false);
+	w = __builtin_amdgcn_cvt_pk_fp8_f32(e4m3_flush_clamp(c), e4m3_flush_clamp(d), w, true);
+	return (u32)w;
+}
+
 template<int STORE> X17_DEV u32 pack4_store(f32 a, f32 b, f32 c, f32 d) {
 	if constexpr (STORE == 1) {
+#if defined(X17_STRICT_MATH) && !X17_STRICT_MATH
+		return pack4_e4m3_hw(a, b, c, d);
+#else
 		return f32_to_e4m3(a) | (f32_to_e4m3(b) << 8) | (f32_to_e4m3(c) << 16) | (f32_to_e4m3(d) << 24);
+#endif
 	} else {
 		return pack4_fixedi8(a, b, c, d);
 	}

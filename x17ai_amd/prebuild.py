@@ -10,7 +10,7 @@ import os
 import subprocess
 
 from . import recipes
-from .api import E4M3, INT8, BF16, GemmConfig, GemmInputConfig, GemmKernel, ScaleConfig
+from .api import E4M3, INT8, BF16, GeGluConfig, GemmConfig, GemmInputConfig, GemmKernel, ScaleConfig
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
@@ -28,6 +28,7 @@ def _specs():
 				add(("ffn_f", k, n, strict, store))
 				add(("attn_y", n // 2, k, strict, store))
 	add(("acc_probe",))
+	add(("e4m3_range",))
 	for geglu in (False, True):
 		add(("mixed", 1024, 512, geglu))
 	for hd in (32, 64, 128):
@@ -144,6 +145,10 @@ def _build_one(spec) -> str:
 		cfg = GemmConfig(GemmInputConfig(INT8, k, None, False), GemmInputConfig(INT8, k, n, True), INT8)
 		GemmKernel(None, f"acc_probe-k{k}-n{n}", cfg, ScaleConfig(1.0, 1.0))
 		return GemmKernel(None, f"acc_probe2-k{k}-n{n}", cfg, ScaleConfig(1.0 / (k * 127.0), 1.0)).name
+	if kind == "e4m3_range":
+		cfg = GemmConfig(GemmInputConfig(INT8, 128, None, False), GemmInputConfig(INT8, 128, 256, True), E4M3)
+		GemmKernel(None, "e4m3_range-strict", cfg, GeGluConfig(1.0 / 32.0, 1.0), True)
+		return GemmKernel(None, "e4m3_range-fast", cfg, GeGluConfig(1.0 / 32.0, 1.0), False).name
 	if kind == "acc_probe_full":
 		k, n = 2048, 16384
 		cfg = GemmConfig(GemmInputConfig(INT8, k, None, False), GemmInputConfig(INT8, k, n, True), INT8)
