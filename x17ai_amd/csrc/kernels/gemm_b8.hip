@@ -167,6 +167,22 @@ struct ResidualEpilogue {
 	static constexpr u32 OUT_COLS = N_RAW / 2;
 
 	X17_DEV static f32 mix(f32 g, f32 v, f32 r) {
+		if constexpr (X17_STRICT_MATH == 0) {
+			// Speed build: both weights from one exponential.  With u = 2 I g and E = 2^-|u|:
+			//   1 + tanh(-I ln2 g) = 2 / (1 + 2^u) = 2 (u >= 0 ? E : 1) / (1 + E)       -> old_w
+			//   lg2(1 + 2^-|u|)    = lg2(1 + E)                                          -> new_w
+			// three transcendentals (ex2, rcp, lg2) instead of four.
+			f32 const u = g * SP_INP_SCALE;
+			f32 const e = hw::ex2(-__builtin_fabsf(u));
+			f32 const d = 1.0f + e;
+			f32 const old_w = (f32(2.0 * SG_HALF) * hw::rcp(d)) * (u >= 0.0f ? e : 1.0f);
+			f32 line = __builtin_fmaxf(0.0f, g);
+			if constexpr (SP_LINE != 1.0f) {
+				line = line * SP_LINE;
+			}
+			f32 const new_w = fmaf32(hw::lg2(d), SP_OUT_SCALE, line);
+			return fmaf32(new_w, v, old_w * r);
+		}
 		f32 old_w = fmaf32(f32(SG_HALF), sfu::tanh(f32(SG_IN) * g), f32(SG_HALF));
 		f32 line = __builtin_fmaxf(0.0f, g);
 		if constexpr (SP_LINE != 1.0f) {
