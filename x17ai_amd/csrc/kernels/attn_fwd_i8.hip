@@ -165,6 +165,7 @@ void kernel(
 
 	// cuda/attn_fwd_i8.cuh:408-412 -- window 0 means "no window"; otherwise rounded up to 16
 	u32 const wr = window_size == 0 ? 0xFFFFFFFFu : ((window_size - 1) / 16 + 1) * 16;
+	u32 const vis_bound = wr - 1 < 0x7FFFFFFFu ? wr - 1 : 0x7FFFFFFFu;
 
 	// key blocks (32 keys) the workgroup walks, and the sub-range this wave needs
 	u32 const kb_begin = (q_block0 - (q_block0 < wr ? q_block0 : wr)) / at::KV_PER_STEP;
@@ -366,10 +367,13 @@ void kernel(
 							X17_UNROLL for (u32 r = 0; r < 8; ++r) s[r] = f32(s_acc[8 * tile + r]) * temperature;
 						}
 						if (need_mask) {
+							// key j is visible iff j < qi and qi - j <= wr, i.e. iff the distance qi - 1 - j, taken as an
+							// unsigned number, is at most wr - 1 (a key at or behind the query wraps to a huge distance;
+							// the bound is capped at 2^31 - 1 so that an unlimited window cannot meet it)
+							u32 const first = qi - 1 - (key0 + 16 * tile + 4 * half);
 							X17_UNROLL for (u32 r = 0; r < 8; ++r) {
-								u32 j = key0 + 16 * tile + 8 * (r / 4) + 4 * half + (r % 4);
-								bool vis = j < qi && (qi - j) <= wr;
-								s[r] = vis ? s[r] : -__builtin_inff();
+								u32 const distance = first - (8 * (r / 4) + (r % 4));
+								s[r] = distance <= vis_bound ? s[r] : -__builtin_inff();
 							}
 						}
 						f32 lmax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fmaxf(s[0], s[1]), __builtin_fmaxf(s[2], s[3])),
