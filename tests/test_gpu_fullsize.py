@@ -315,3 +315,24 @@ def test_config5_row_scaled_prefill_and_decode_sampled_heads(dev):
 		qsd[:, heads], ksd[:, heads], vwd[:, heads], swd[heads], oscd[heads], out_bf16=True)
 	assert np.array_equal(_head_columns(gotd, heads, hd), wantd)
 	assert np.array_equal(gotd_l[:, heads].view(np.uint32), np.asarray(wantd_l).reshape(s, len(heads)).view(np.uint32))
+
+
+def test_config4_block_chain(dev):
+	"""benchmark config 4 as one chain (tests/config4_chain.py): seeded bf16 residual stream [4 x 8192, 2048] through
+	x17ai_amd.block.Block -- rms_norm, q, kv (head_dim 128, 4096 raw columns, a 16-tile-wide persistent walk),
+	attention, attn_y, ffn_f -> e4m3, e4m3 x int8 ffn_y -- strict builds, each stage against the oracle on the GPU's
+	own upstream output: sampled token rows bit for bit (ffn_y: one e4m3 code, < 0.5 %), three attention heads over
+	all 8192 queries of their sequence.  Then the speed build of each stage against the strict one over the whole
+	tensors, with the bounds the speed builds are documented to keep."""
+	from tests import config4_chain as C
+	inp = C.inputs()
+	got = C.run_strict(dev, inp)
+	C.check_strict(inp, got)
+	rep = C.fast_vs_strict(dev, inp, got)
+	# no approximate operation upstream of these stores
+	assert rep["attn_q"]["mismatched"] == 0 and rep["attn_kv"]["mismatched"] == 0 and rep["attn_kv"]["rrms_bits_equal"]
+	a = rep["attn_fwd_i8"]
+	assert a["hist_abs_code_diff_0_1_2_3_more"][2:] == [0, 0, 0] and a["mismatched"] < 0.02 * a["elements"], a
+	for name in ("attn_y", "ffn_f", "ffn_y_f8"):
+		r = rep[name]
+		assert r["frac_mismatched"] < 5e-3 and r["frac_beyond_one_code"] == 0.0, (name, r)

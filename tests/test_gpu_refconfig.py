@@ -19,7 +19,7 @@ import numpy as np
 import pytest
 
 import x17ai_amd as X
-from x17ai_amd import recipes
+from x17ai_amd.block import Block, BlockConfig
 from oracle import dense as D
 from oracle import strict as S
 from tests import refconfig as R
@@ -46,29 +46,14 @@ def _up(dev, arr, dtype):
 
 @pytest.fixture(scope="module")
 def stages(dev, ref):
-	"""q, kv (+ rrms), attention (+ L), attn_y, ffn_f, ffn_y of the reference run, computed on the GPU."""
-	t, d, h, hd, f = R.SEQ_LEN, R.MODEL_DIM, R.N_HEADS, R.HEAD_DIM, R.F_WIDTH
-	x = _up(dev, ref["x"], X.INT8)
-	out = {}
-	q = X.Tensor(dev, (t, h * hd), X.INT8)
-	recipes.attn_q_kernel(dev, d, h * hd).launch(x, _up(dev, ref["attn_q_weights"], X.INT8), q)
-	kv = X.Tensor(dev, (t, 2 * h * hd), X.INT8)
-	rrms = X.Tensor(dev, (t, h), X.F32)
-	recipes.attn_kv_kernel(dev, d, 2 * h * hd, hd).launch(x, _up(dev, ref["attn_kv_weights"], X.INT8), kv, rrms)
-	ao = X.Tensor(dev, (t, h * hd), X.INT8)
-	al = X.Tensor(dev, (h, t), X.F32)
-	recipes.attn_kernel(dev, h, hd, True).launch(q, kv, _up(dev, ref["sinks_k"], X.INT8), _up(dev, ref["sinks_v"], X.INT8),
-	                                             _up(dev, ref["attn_temperature"], X.F32), ao, al, 0)
-	ay = X.Tensor(dev, (t, d), X.E4M3)
-	recipes.attn_y_kernel(dev, d, h * hd, True).launch(ao, _up(dev, ref["attn_y_weights"], X.INT8), ay, x)
-	ff = X.Tensor(dev, (t, f), X.E4M3)
-	recipes.ffn_f_kernel(dev, d, 2 * f, True).launch(x, _up(dev, ref["ffn_f_weights"], X.INT8), ff)
-	fy = X.Tensor(dev, (t, d), X.E4M3)
-	recipes.ffn_y_kernel(dev, d, f, True).launch(ff, _up(dev, ref["ffn_y_weights"], X.INT8), fy, x)
-	for name, tensor in (("q", q), ("kv", kv), ("rrms", rrms), ("attn_out", ao), ("attn_l", al), ("attn_y", ay),
-	                     ("ffn_f", ff), ("ffn_y", fy)):
-		out[name] = tensor.download()
-	return out
+	"""q, kv (+ rrms), attention (+ L), attn_y, ffn_f, ffn_y of the reference run, computed on the GPU by the block
+	object in main.rs's stage order (src/main.rs:193-263)."""
+	block = Block(dev, BlockConfig(R.MODEL_DIM, R.N_HEADS, R.HEAD_DIM, R.F_WIDTH, 0, 1, None, True))
+	w = {k: _up(dev, v, X.F32 if k == "attn_temperature" else X.INT8) for k, v in ref.items() if k != "x"}
+	out = block.forward(_up(dev, ref["x"], X.INT8), w)
+	names = {"q": "q", "kv": "kv", "k_rrms": "rrms", "attn_out": "attn_out", "attn_l": "attn_l", "attn_y": "attn_y",
+	         "ffn_f": "ffn_f", "ffn_y": "ffn_y"}
+	return {names[k]: t.download() for k, t in out.items()}
 
 
 INP = 1.0 / math.sqrt(R.MODEL_DIM) / 64.0        # src/main.rs:412-416, 461-469, 599-603

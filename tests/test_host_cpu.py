@@ -232,3 +232,31 @@ def test_reference_tensor_file_conventions(tmp_path):
 def test_bench_refuses_more_than_one_gpu():
 	r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
 	assert r.returncode != 0 and "one GPU" in r.stderr
+
+
+def test_safetensors_header_that_overflows_is_rejected_before_anything_is_allocated(tmp_path):
+	"""A header whose shape times the element size wraps around usize, or whose data lies beyond the end of the
+	file, is an error (never a tensor whose shape disagrees with its allocation)."""
+	import json
+	import struct
+
+	def write(name, header: dict, payload: bytes = b""):
+		text = json.dumps(header).encode()
+		text += b" " * (-len(text) % 8)
+		p = tmp_path / name
+		p.write_bytes(struct.pack("<Q", len(text)) + text + payload)
+		return str(p)
+
+	wraps = write("wrap_f32.safetensors", {"t": {"dtype": "F32", "shape": [2 ** 62], "data_offsets": [0, 0]}})
+	with pytest.raises(X.X17Error, match="invalid safetensors file"):
+		X.Tensor.from_safetensors_file(wraps, None)
+	wraps2 = write("wrap2_i8.safetensors", {"t": {"dtype": "I8", "shape": [2 ** 33, 2 ** 33], "data_offsets": [0, 0]}})
+	with pytest.raises(X.X17Error, match="invalid safetensors file"):
+		X.Tensor.from_safetensors_file(wraps2, None)
+	short = write("short_i8.safetensors", {"t": {"dtype": "I8", "shape": [1 << 20], "data_offsets": [0, 1 << 20]}}, b"\0" * 16)
+	with pytest.raises(X.X17Error, match="truncated tensor data"):
+		X.Tensor.from_safetensors_file(short, None)
+	with pytest.raises(X.X17Error, match="overflows"):
+		X.Tensor(None, (2 ** 62,), X.F32)
+	ok = write("ok_i8.safetensors", {"t": {"dtype": "I8", "shape": [2, 8], "data_offsets": [0, 16]}}, bytes(range(16)))
+	assert X.Tensor.from_safetensors_file(ok, None).download().ravel().tolist() == list(range(16))

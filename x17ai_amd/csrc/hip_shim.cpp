@@ -24,6 +24,7 @@
 #include <string>
 #include <string_view>
 #include <utility>
+#include <vector>
 
 #include "../../include/x17ai_hip_shim.h"
 
@@ -117,15 +118,18 @@ struct Timer {
 	hipEvent_t end;
 };
 
-struct Module {
-	int device;
-	hipModule_t module;
-};
-
 struct Kernel {
 	int device;
 	hipFunction_t function;
 	size_t max_dynamic_smem;
+};
+
+// The reference's kernel handle is the CUfunction itself (cpp/cuda_shim.cpp:903) and the ABI has no call that
+// releases one; here a handle is a small record, owned by its module and freed with it in x17ai_hip_del_module.
+struct Module {
+	int device;
+	hipModule_t module;
+	std::vector<std::unique_ptr<Kernel>> kernels;
 };
 
 // Makes `device` current for the scope, restores the previous device afterwards.
@@ -569,7 +573,8 @@ X17KernelResult x17ai_hip_get_kernel(X17HipModuleHandle *module_c, char const *n
 				);
 			}
 			result->max_dynamic_smem = smem_size;
-			out = result.release();
+			out = result.get();
+			module->kernels.push_back(std::move(result));
 			return nullptr;
 		} X17_CATCH("x17ai_hip_get_kernel()")
 	};

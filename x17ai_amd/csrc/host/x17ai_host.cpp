@@ -217,6 +217,7 @@ Result<std::shared_ptr<Tensor>> Tensor::new_empty(std::vector<size_t> shape, DTy
 		if (d != 0 && n > SIZE_MAX / d) return R::err(ErrPack{TensorOpError::Other, "tensor shape overflows usize", nullptr});
 		n *= d;
 	}
+	if (n > SIZE_MAX / dtype_bytes(dtype)) return R::err(ErrPack{TensorOpError::Other, "tensor size in bytes overflows usize", nullptr});
 	size_t bytes = n * dtype_bytes(dtype);
 	auto buf = device->new_buffer(bytes);
 	if (!buf.is_ok()) return R::err(*buf.error);
@@ -348,9 +349,18 @@ Result<std::shared_ptr<Tensor>> Tensor::from_safetensors_file(std::string const 
 	else if (e.dtype == "BF16") dtype = DType::Bf16;
 	else if (e.dtype == "F32") dtype = DType::F32;
 	else return R::err(ErrPack{TensorOpError::Other, "unsupported dtype " + e.dtype + " in " + path, nullptr});   // dtype.rs:38-50
+	// shape, data_offsets and the file size are checked against each other before anything is allocated
+	size_t want = dtype_bytes(dtype);
+	for (size_t d : e.shape) {
+		if (d != 0 && want > SIZE_MAX / d) return bad("shape overflows usize");
+		want *= d;
+	}
+	if (e.end < e.begin || e.end - e.begin != want) return bad("data_offsets do not match dtype and shape");
+	f.seekg(0, std::ios::end);
+	uint64_t const file_size = uint64_t(f.tellg());
+	if (file_size < 8 + n || file_size - (8 + n) < e.end) return bad("truncated tensor data");
 	auto t = Tensor::new_empty(e.shape, dtype, std::move(device));
 	if (!t.is_ok()) return t;
-	if (e.end < e.begin || e.end - e.begin != (*t.value)->bytes) return bad("data_offsets do not match dtype and shape");
 	std::vector<char> data((*t.value)->bytes);
 	f.seekg(std::streamoff(8 + n + e.begin));
 	if (!data.empty() && !f.read(data.data(), std::streamsize(data.size()))) return bad("truncated tensor data");
@@ -710,6 +720,12 @@ static std::string format_cpp_f64(double v) {   // gemm.rs:257-259
 	return buf;
 }
 
+// A scale's description ends up in a `//` comment of the generated common.h: keep it on that line.
+static std::string one_line(std::string s) {
+	for (char &ch : s) if (ch == '\n' || ch == '\r' || ch == '\\') ch = ' ';
+	return s;
+}
+
 static bool is_pow2(size_t v) { return v != 0 && (v & (v - 1)) == 0; }
 static unsigned ctz(size_t v) { unsigned n = 0; while ((v & 1) == 0) { v >>= 1; ++n; } return n; }
 
@@ -731,7 +747,7 @@ std::unique_ptr<GemmKernel> GemmKernel::create(std::shared_ptr<HipDevice> device
 	size_t const b_rows = *g.b.rows;
 	int const kind = int(e.index());
 	std::ostringstream common;
-	common << "// generated by x17::GemmKernel::create for kernel \"" << kernel_name << "\"\n";
+	common << "// generated by x17::GemmKernel::create for kernel \"" << one_line(kernel_name) << "\"\n";
 	common << "#define X17_A_COLS " << g.a.cols << "\n#define X17_B_ROWS " << b_rows << "\n";
 	common << "#define X17_A_KIND " << kind_of(g.a.dtype) << "\n#define X17_B_KIND " << kind_of(g.b.dtype) << "\n";
 	common << "#define X17_EPILOGUE " << kind << "\n";
@@ -753,20 +769,20 @@ std::unique_ptr<GemmKernel> GemmKernel::create(std::shared_ptr<HipDevice> device
 	if (auto const *c = std::get_if<ScaleConfig>(&e)) {
 		if (g.c_dtype != DType::Int8) { diag.add_error("Scale epilogue requires an i8 output"); return nullptr; }
 		if (!std::isfinite(c->inp_scale.value) || !std::isfinite(c->out_scale.value)) { diag.add_error("invalid Scale epilogue scale values"); return nullptr; }
-		common << "#define X17_INP_SCALE " << format_cpp_f64(c->inp_scale.value) << " // " << c->inp_scale.description << "\n";
-		common << "#define X17_OUT_SCALE " << format_cpp_f64(c->out_scale.value) << " // " << c->out_scale.description << "\n";
+		common << "#define X17_INP_SCALE " << format_cpp_f64(c->inp_scale.value) << " // " << one_line(c->inp_scale.description) << "\n";
+		common << "#define X17_OUT_SCALE " << format_cpp_f64(c->out_scale.value) << " // " << one_line(c->out_scale.description) << "\n";
 	} else if (auto const *c = std::get_if<GeGluConfig>(&e)) {
 		if (g.c_dtype != DType::E4m3 && g.c_dtype != DType::Int8) { diag.add_error("GeGLU epilogue requires an e4m3 or i8 output"); return nullptr; }
 		if (!finite_pos(c->inp_scale.value) || !finite_pos(c->out_scale.value)) { diag.add_error("invalid GeGLU scale values"); return nullptr; }
 		if (b_rows % 2 != 0) { diag.add_error("GeGLU GEMM requires an even raw output column count"); return nullptr; }
-		common << "#define X17_INP_SCALE " << format_cpp_f64(c->inp_scale.value) << " // " << c->inp_scale.description << "\n";
-		common << "#define X17_OUT_SCALE " << format_cpp_f64(c->out_scale.value) << " // " << c->out_scale.description << "\n";
+		common << "#define X17_INP_SCALE " << format_cpp_f64(c->inp_scale.value) << " // " << one_line(c->inp_scale.description) << "\n";
+		common << "#define X17_OUT_SCALE " << format_cpp_f64(c->out_scale.value) << " // " << one_line(c->out_scale.description) << "\n";
 	} else if (auto const *c = std::get_if<ResidualConfig>(&e)) {
 		if (g.c_dtype != DType::E4m3 && g.c_dtype != DType::Int8) { diag.add_error("Residual epilogue requires an e4m3 or i8 output"); return nullptr; }
 		if (!finite_pos(c->inp_scale.value) || !finite_pos(c->out_scale.value)) { diag.add_error("invalid residual GEMM scale values"); return nullptr; }
 		if (b_rows % 2 != 0) { diag.add_error("Residual GEMM requires an even raw output column count"); return nullptr; }
-		common << "#define X17_INP_SCALE " << format_cpp_f64(c->inp_scale.value) << " // " << c->inp_scale.description << "\n";
-		common << "#define X17_OUT_SCALE " << format_cpp_f64(c->out_scale.value) << " // " << c->out_scale.description << "\n";
+		common << "#define X17_INP_SCALE " << format_cpp_f64(c->inp_scale.value) << " // " << one_line(c->inp_scale.description) << "\n";
+		common << "#define X17_OUT_SCALE " << format_cpp_f64(c->out_scale.value) << " // " << one_line(c->out_scale.description) << "\n";
 	} else if (auto const *c = std::get_if<DequantConfig>(&e)) {
 		if (g.c_dtype != DType::Bf16) { diag.add_error("Dequant epilogue requires a bf16 output"); return nullptr; }
 		if (c->geglu && b_rows % 2 != 0) { diag.add_error("Dequant GeGLU GEMM requires an even raw output column count"); return nullptr; }
@@ -790,9 +806,9 @@ std::unique_ptr<GemmKernel> GemmKernel::create(std::shared_ptr<HipDevice> device
 		common << "#define X17_HEAD_DIM " << c->head_dim << "\n#define X17_EPS " << format_cpp_f64(c->eps) << "\n";
 		// gemm.rs:146,152
 		common << "#define X17_HEAD_SCALE " << format_cpp_f64(c->out_scale.value * std::sqrt(double(c->head_dim)))
-		       << " // (" << c->out_scale.description << ") * sqrt(" << c->head_dim << ")\n";
+		       << " // (" << one_line(c->out_scale.description) << ") * sqrt(" << c->head_dim << ")\n";
 		common << "#define X17_SEP_SCALE " << format_cpp_f64(c->inp_scale.value * c->out_scale.value)
-		       << " // (" << c->inp_scale.description << ") * (" << c->out_scale.description << ")\n";
+		       << " // (" << one_line(c->inp_scale.description) << ") * (" << one_line(c->out_scale.description) << ")\n";
 	}
 
 	if (g.a.cols % 128 != 0) { diag.add_error("GEMM K must be a multiple of 128, got " + std::to_string(g.a.cols)); return nullptr; }
@@ -883,6 +899,9 @@ Status GemmKernel::launch(GemmArgs const &args) {
 		s = tensor_check::matrix_shape(op, "rrms", *args.extra, a_rows, rrms_cols, *device, DType::F32, tmp);
 		if (!s.is_ok()) return s;
 	}
+	if (a_rows > 0xFFFFFFFFull || b_rows_v > 0xFFFFFFFFull) {
+		return Status::err(TensorOpError::Other, std::string(op) + " sizes exceed 32 bits (the kernel's row counts are u32)");
+	}
 	size_t grid_x = a_rows >> ctz(metadata.M_PER_BLOCK);
 	size_t grid_y = b_rows_v >> ctz(metadata.N_PER_BLOCK);
 	// 8-byte slots passed by address, exactly as gemm.rs:618-631 does; the kernel's u32 parameters
@@ -952,7 +971,7 @@ std::unique_ptr<AttnKernel> AttnKernel::create(std::shared_ptr<HipDevice> device
 		return nullptr;
 	}
 	std::ostringstream common;
-	common << "// generated by x17::AttnKernel::create for kernel \"" << kernel_name << "\"\n";
+	common << "// generated by x17::AttnKernel::create for kernel \"" << one_line(kernel_name) << "\"\n";
 	common << "#define X17_N_HEADS " << config.n_heads << "\n#define X17_HEAD_DIM " << config.head_dim << "\n";
 	common << "#define X17_Q_STRIDE " << config.q_stride << "\n#define X17_KV_STRIDE " << config.kv_stride << "\n#define X17_O_STRIDE " << config.o_stride << "\n";
 	common << "#define X17_STRICT_MATH " << (strict_math ? 1 : 0) << "\n";
@@ -1064,7 +1083,7 @@ std::unique_ptr<RmsNormKernel> RmsNormKernel::create(std::shared_ptr<HipDevice> 
 	}
 	if (!std::isfinite(config.eps) || config.eps < 0.0) { diag.add_error("invalid rms_norm eps"); return nullptr; }
 	std::ostringstream common;
-	common << "// generated by x17::RmsNormKernel::create for kernel \"" << kernel_name << "\"\n";
+	common << "// generated by x17::RmsNormKernel::create for kernel \"" << one_line(kernel_name) << "\"\n";
 	common << "#define X17_MODEL_DIM " << config.model_dim << "\n#define X17_IN_KIND " << (config.in_dtype == DType::E4m3 ? 1 : 2) << "\n";
 	common << "#define X17_EPS " << format_cpp_f64(config.eps) << "\n";
 	auto built = kernel_build::build(kernel_name, common.str(), "rms_norm.hip", "rms_norm_meta.cpp", diag);
@@ -1124,7 +1143,7 @@ std::unique_ptr<AttnDecodeKernel> AttnDecodeKernel::create(std::shared_ptr<HipDe
 		return nullptr;
 	}
 	std::ostringstream common;
-	common << "// generated by x17::AttnDecodeKernel::create for kernel \"" << kernel_name << "\"\n";
+	common << "// generated by x17::AttnDecodeKernel::create for kernel \"" << one_line(kernel_name) << "\"\n";
 	common << "#define X17_N_HEADS " << config.n_heads << "\n#define X17_HEAD_DIM " << config.head_dim << "\n";
 	common << "#define X17_CACHE_CAPACITY " << config.cache_capacity << "\n";
 	common << "#define X17_STRICT_MATH " << (strict_math ? 1 : 0) << "\n";

@@ -101,11 +101,21 @@ def _specs():
 	for strict in (True, False):                             # the speed builds are bench.py's
 		add(("dequant", 2048, 16384, INT8, INT8, True, strict))
 		add(("dequant", 8192, 2048, INT8, INT8, False, strict))
+	# ---- x17ai_amd.block: benchmark config 4 (bench.py, tests/config4_chain.py) and the reference's own configuration
+	for strict in (True, False):
+		add(("block", 2048, 16, 128, 8192, BF16, strict))
+	add(("block", 2048, 64, 32, 2048, None, True))
+	add(("block", 512, 8, 32, 256, None, True))          # tests/test_gpu_files.py
+	add(("attn_q", 128, 256))
 	return s
 
 
 def _build_one(spec) -> str:
 	kind = spec[0]
+	if kind == "block":
+		from .block import Block, BlockConfig
+		Block(None, BlockConfig(spec[1], spec[2], spec[3], spec[4], 0, 1, spec[5], spec[6]))
+		return f"block-d{spec[1]}-h{spec[2]}x{spec[3]}-f{spec[4]}-{'strict' if spec[6] else 'fast'}"
 	if kind == "attn_q":
 		return recipes.attn_q_kernel(None, spec[1], spec[2]).name
 	if kind == "ffn_f":
