@@ -17,6 +17,7 @@
 #include <atomic>
 #include <bit>
 #include <cassert>
+#include <cstdio>
 #include <cstring>
 #include <exception>
 #include <memory>
@@ -130,6 +131,10 @@ struct Module {
 	int device;
 	hipModule_t module;
 	std::vector<std::unique_ptr<Kernel>> kernels;
+	// The code object as read from the file, alive as long as the module.  The module is created from these bytes and
+	// not from the path: the runtime keeps the file handles of paths it has loaded, so a code object rebuilt under the
+	// same path within one process would be loaded as its previous contents.
+	std::vector<char> image;
 };
 
 // Makes `device` current for the scope, restores the previous device afterwards.
@@ -503,11 +508,31 @@ X17ModuleResult x17ai_hip_load_module(X17HipContextHandle *context, char const *
 			auto result = std::make_unique<Module>();
 			result->device = ctx->device;
 			result->module = nullptr;
-			hipError_t e = hipModuleLoad(&result->module, code_object_path);
+			{
+				std::FILE *f = std::fopen(code_object_path, "rb");
+				if (f == nullptr) [[unlikely]] {
+					return X17_DIAG(
+						"x17ai_hip_load_module(): cannot open the code object.",
+						"x17ai_hip_load_module(): cannot open ", code_object_path
+					);
+				}
+				char buf[65536];
+				size_t got;
+				while ((got = std::fread(buf, 1, sizeof buf, f)) > 0) result->image.insert(result->image.end(), buf, buf + got);
+				bool const failed = std::ferror(f) != 0;
+				std::fclose(f);
+				if (failed || result->image.empty()) [[unlikely]] {
+					return X17_DIAG(
+						"x17ai_hip_load_module(): cannot read the code object.",
+						"x17ai_hip_load_module(): cannot read ", code_object_path
+					);
+				}
+			}
+			hipError_t e = hipModuleLoadData(&result->module, result->image.data());
 			if (e != hipSuccess) [[unlikely]] {
 				return X17_DIAG(
-					"x17ai_hip_load_module(): hipModuleLoad() failed.",
-					"x17ai_hip_load_module(): hipModuleLoad(", code_object_path, ") failed with hip error: ", e
+					"x17ai_hip_load_module(): hipModuleLoadData() failed.",
+					"x17ai_hip_load_module(): hipModuleLoadData(", code_object_path, ") failed with hip error: ", e
 				);
 			}
 			if (result->module == nullptr) [[unlikely]] {
