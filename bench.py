@@ -3,18 +3,22 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] [--only KERNEL] [--copy-probe]
 
-Headline (the JSON line's `value`): benchmark config 2, the int8 FFN GEMM pair
-  ffn_f_fwd   x[8192, 2048] i8 . W1[16384, 2048]^T  -> GeGLU   -> f[8192, 8192] FixedI8
-  ffn_y_fwd   f[8192, 8192] i8 . W2[4096, 8192]^T   -> gated residual with x -> y[8192, 2048] e4m3
-One step = both launches over the 8192-token batch; inputs are resident in HBM before the timed
-region.  value = (2*M*K*N_raw of both GEMMs) * steps / wall time, in TOPS.
+Headline (the JSON line's `value`): benchmark config 4, the full quantized block forward over
+4 sequences x 8192 tokens, d_model 2048, 16 heads x 128, window 512, d_ff 8192:
+  rms_norm (bf16 -> FixedI8 x) -> attn_q, attn_kv -> attn_fwd_i8 -> attn_y ; ffn_f -> ffn_y_f8
+(x17ai_amd.block.Block: stage order and scale recipes of src/main.rs:193-280, 387-675).  One step = the
+seven launches over the 32768-token batch; inputs and weights are resident in HBM before the timed
+region.  value = 32768 * steps / wall time, in tokens per second.
 
-`roofline` is for the dominant kernel (the ffn_f GEMM): algorithmic int8 ops per launch divided by
-its mean launch duration, measured with HIP events on the launching stream inside the timed
-region, against the MI355X dense int8 MFMA peak.  `cpu_baseline` is the CPU oracle (a port of the
-reference's arithmetic) timed on a bounded row sample of the same workload on the host cores.
-`extras` reports the other benchmark configurations (fp8 FFN, block forward, attention prefill,
-decode, rms_norm), each as median-of-launches, next to the roofline that bounds it.
+`roofline` is for the dominant kernel of that block, the e4m3 x int8 ffn_y GEMM (44 % of the block's
+time; both operands are widened exactly to f16 and multiplied on the f16 matrix cores): algorithmic flops
+per launch divided by its mean launch duration, measured with HIP events on the launching stream inside
+the timed region, against the MI355X dense f16 MFMA peak.  `roofline.traffic` is read from the rocprofv3
+summary under profiles/ named in `roofline.traffic_source` (null when that file is absent).
+`cpu_baseline` is the CPU oracle (a port of the reference's arithmetic) timed on a bounded token sample of
+the same block on the host cores.  `extras` reports the other benchmark configurations (int8 and fp8 FFN
+pairs in TOPS, attention prefill, decode, rms_norm), each as median-of-launches next to the roofline that
+bounds it, with a bounded CPU figure per configuration.
 """
 from __future__ import annotations
 
@@ -36,11 +40,23 @@ PEAK_FP8_TFLOPS = 5000.0     # dense fp8
 PEAK_BF16_TFLOPS = 2500.0    # dense bf16
 PEAK_HBM_GBS = 8000.0        # HBM3E
 
-# HBM bytes per ffn_f launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), or None
-FFN_F_TRAFFIC_BYTES = int((198254 * 2.0 + 65536 * 1.0) * 1024)
-# HBM bytes one decode launch of config 5 fetches (profiles/attn_decode_i8_config5.txt): all K rows plus the
-# V rows with a nonzero 8-bit probability -- about half of the 2 GiB cache for the synthetic Gaussian codes
-DECODE_TRAFFIC_BYTES = int(529500 * 2.0 * 1024)
+PEAK_F16_TFLOPS = 2500.0     # dense f16
+# launches per measurement, after the reference's own harnesses (attn_fwd_i8.cu:117-182, ffn_f_fwd_f8.cu:108-161):
+# 50 warm-up launches, 100 timed (attention: 10 timed), median and minimum reported
+GEMM_WARM, GEMM_TIMED = 50, 100
+ATTN_WARM, ATTN_TIMED = 5, 10
+
+
+def profile_traffic(file_name):
+	"""HBM bytes per launch as the rocprofv3 summary under profiles/ records them (the line
+	`roofline.traffic: N bytes per launch`), or None when the file or the line is missing."""
+	import re
+	try:
+		with open(os.path.join(ROOT, "profiles", file_name)) as fh:
+			m = re.search(r"^roofline\.traffic:\s*([0-9]+)\s*bytes per launch", fh.read(), re.M)
+		return int(m.group(1)) if m else None
+	except OSError:
+		return None
 
 
 def _rand_i8(rng, shape):
@@ -66,26 +82,56 @@ def _median_launch(dev, X, fn, iters, warm):
 	return ts[len(ts) // 2], ts[0]
 
 
-def headline(dev, X, recipes, steps, warmup):
-	M, D, F = 8192, 2048, 8192
-	rng = np.random.default_rng(2000)
-	x = X.Tensor.from_numpy(dev, _rand_codes(rng, (M, D)), X.INT8)
-	w1 = X.Tensor.from_numpy(dev, _rand_codes(rng, (2 * F, D)), X.INT8)
-	w2 = X.Tensor.from_numpy(dev, _rand_codes(rng, (2 * D, F)), X.INT8)
-	f = X.Tensor(dev, (M, F), X.INT8)
-	y = X.Tensor(dev, (M, D), X.E4M3)
-	k1 = recipes.ffn_f_kernel(dev, D, 2 * F, False, X.INT8)
-	k2 = recipes.ffn_y_kernel(dev, D, F, False, X.INT8, X.INT8)
-	ops1 = k1.n_ops(x, w1)
-	ops2 = k2.n_ops(f, w2)
+CONFIG4 = dict(T=8192, B=4, D=2048, H=16, HD=128, W=512, F=8192)
+
+
+def config4_inputs(rng, rows):
+	"""Synthetic block inputs of benchmark config 4 for `rows` token rows: the bf16 residual stream and FixedI8
+	weights (N(0,1) codes; the 1/sqrt(fan_in) of the configuration is folded into the kernels' constants exactly as
+	src/main.rs:412-421 folds it)."""
+	c = CONFIG4
+	D, H, HD, F = c["D"], c["H"], c["HD"], c["F"]
+	return {
+		"x_bf16": (rng.standard_normal((rows, D), dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16),
+		"attn_q_weights": _rand_codes(rng, (H * HD, D)),
+		"attn_kv_weights": _rand_codes(rng, (2 * H * HD, D)),
+		"attn_y_weights": _rand_codes(rng, (2 * D, H * HD)),
+		"ffn_f_weights": _rand_codes(rng, (2 * F, D)),
+		"ffn_y_weights": _rand_codes(rng, (2 * D, F)),
+		"sinks_k": _rand_codes(rng, (H, HD)),
+		"sinks_v": _rand_codes(rng, (H, HD)),
+		"attn_temperature": (0.5 + rng.random(H)).astype(np.float32),
+	}
+
+
+def config4_block(dev, X, fused_qkv=False):
+	from x17ai_amd.block import Block, BlockConfig
+	c = CONFIG4
+	cfg = BlockConfig(c["D"], c["H"], c["HD"], c["F"], c["W"], c["B"], X.BF16, False, fused_qkv)
+	block = Block(dev, cfg)
+	rows = c["T"] * c["B"]
+	inp = config4_inputs(np.random.default_rng(4000), rows)
+	w = {k: X.Tensor.from_numpy(dev, v, X.F32 if k == "attn_temperature" else X.INT8) for k, v in inp.items() if k != "x_bf16"}
+	x = X.Tensor.from_numpy(dev, inp["x_bf16"], X.BF16)
+	block.validate(rows, w)
+	out = block.new_outputs(rows)
+	return block, x, w, out, rows
+
+
+def headline(dev, X, steps, warmup, fused_qkv=False):
+	"""`steps` block forwards back to back on the stream; an event pair around the dominant launch of each."""
+	block, x, w, out, rows = config4_block(dev, X, fused_qkv)
+	stages = block.stages(x, w, out)
+	dominant = "ffn_y_f8"
 
 	def step(timer=None):
-		if timer is not None:
-			timer.start()
-		k1.launch(x, w1, f)
-		if timer is not None:
-			timer.stop()
-		k2.launch(f, w2, y, x)
+		for name, launch in stages:
+			if timer is not None and name == dominant:
+				timer.start()
+				launch()
+				timer.stop()
+			else:
+				launch()
 
 	for _ in range(warmup):
 		step()
@@ -95,29 +141,109 @@ def headline(dev, X, recipes, steps, warmup):
 	for t in timers:
 		step(t)
 	dev.synchronize()
-	t1 = time.perf_counter()
-	wall = t1 - t0
-	k1_mean = sum(t.elapsed_seconds() for t in timers) / steps
-	return {
-		"wall_s": wall, "ops_per_step": ops1 + ops2, "k1_ops": ops1, "k1_mean_s": k1_mean,
-		"shapes": {"tokens": M, "d_model": D, "d_ff": F},
-	}
+	wall = time.perf_counter() - t0
+	ops = block.n_ops(rows)
+	return {"wall_s": wall, "rows": rows, "dominant_ops": ops[dominant],
+	        "dominant_mean_s": sum(t.elapsed_seconds() for t in timers) / steps,
+	        "stage_names": [name for name, _ in stages]}
 
 
 def cpu_baseline():
-	"""The CPU oracle on config 2 (all 8192 token rows: about 12 s on 16 host threads)."""
+	"""The CPU oracle over a bounded sample of the config 4 block: the first 1024 tokens of one sequence through all
+	seven stages (attention: all 16 heads over those 1024 positions, window 512).  tokens / CPU seconds."""
 	from oracle import strict as S
-	M, D, F = 8192, 2048, 8192
-	rng = np.random.default_rng(2001)
+	from x17ai_amd import recipes
+	c = CONFIG4
+	D, H, HD, F, W = c["D"], c["H"], c["HD"], c["F"], c["W"]
+	n = 1024
+	inp = config4_inputs(np.random.default_rng(4000), n)
+	inp_scale = 1.0 / math.sqrt(D) / 64.0
+	t0 = time.perf_counter()
+	x = S.rms_norm(inp["x_bf16"], recipes.L2_NORM_EPS, "bf16")
+	q = S.epilogue_scale(S.gemm_i32(x, inp["attn_q_weights"]), inp_scale, 8.0)
+	kv, _ = S.epilogue_l2norm(S.gemm_i32(x, inp["attn_kv_weights"]), HD, recipes.L2_NORM_EPS, inp_scale, 8.0)
+	ao, _ = S.attn_fwd_i8(q, kv, inp["sinks_k"], inp["sinks_v"], inp["attn_temperature"], H, HD, W)
+	S.epilogue_residual(S.gemm_i32(ao, inp["attn_y_weights"]), x, 1.0 / math.sqrt(H * HD) / 64.0, 1.0, S.STORE_E4M3)
+	f = S.epilogue_geglu(S.gemm_i32(x, inp["ffn_f_weights"]), inp_scale, 1.0, S.STORE_E4M3)
+	S.epilogue_residual(S.gemm_f32_seq(f, True, inp["ffn_y_weights"], False), x,
+	                    math.sqrt(recipes.GELU_VAR_FIX_2 / F) / 8.0, 1.0, S.STORE_E4M3)
+	dt = time.perf_counter() - t0
+	return {"value": n / dt, "unit": "tokens/s", "cores": S.num_threads(), "kind": "port",
+	        "sample": f"the first {n} tokens of one sequence of config 4 through all seven stages "
+	                  f"(16 heads, window 512), {dt:.1f} s of CPU time"}
+
+
+def cpu_extras():
+	"""A bounded CPU figure per remaining configuration, in that configuration's unit."""
+	from oracle import strict as S
+	from oracle import dense
+	from x17ai_amd import recipes
+	out = {}
+	rng = np.random.default_rng(5000)
+	# config 1, the reference's CPU-runnable case: dense float64 attention (new_block.py:183-232 semantics), one head
+	# at a time, T=1024, H=8, hd=64, W=256 -- and the strict C port on the same shape
+	T1, H1, HD1, W1 = 1024, 8, 64, 256
+	qc, kvc = _rand_codes(rng, (T1, H1 * HD1)), _rand_codes(rng, (T1, 2 * H1 * HD1))
+	sk, sv = _rand_codes(rng, (H1, HD1)), _rand_codes(rng, (H1, HD1))
+	ops1 = 4.0 * HD1 * H1 * (W1 * (W1 - 1) // 2 + (T1 - W1) * W1)
+	t0 = time.perf_counter()
+	for h in range(H1):
+		kh = kvc[:, 2 * h * HD1:(2 * h + 1) * HD1].astype(np.float64) / 8
+		vh = kvc[:, (2 * h + 1) * HD1:(2 * h + 2) * HD1].astype(np.float64) / 8
+		dense.attn_one_head(qc[:, h * HD1:(h + 1) * HD1].astype(np.float64) / 8, kh, vh, sk[h].astype(np.float64) / 8,
+		                    sv[h].astype(np.float64) / 8, 1.0, W1)
+	dt = time.perf_counter() - t0
+	out["config1_attn_dense_f64"] = {"value": ops1 / dt / 1e12, "unit": "TOPS", "cores": 1, "kind": "port",
+	                                 "sample": f"all of config 1 (numpy float64, dense [T, T+1] scores), {dt:.2f} s"}
+	t0 = time.perf_counter()
+	S.attn_fwd_i8(qc, kvc, sk, sv, np.ones(H1, np.float32), H1, HD1, W1)
+	dt = time.perf_counter() - t0
+	out["config1_attn_strict"] = {"value": ops1 / dt / 1e12, "unit": "TOPS", "cores": S.num_threads(), "kind": "port",
+	                              "sample": f"all of config 1 (strict C port), {dt:.3f} s"}
+	# config 2: the int8 FFN pair, 2048 of the 8192 token rows
+	M, D, F = 2048, 2048, 8192
 	x, w1, w2 = _rand_codes(rng, (M, D)), _rand_codes(rng, (2 * F, D)), _rand_codes(rng, (2 * D, F))
 	t0 = time.perf_counter()
 	f = S.epilogue_geglu(S.gemm_i32(x, w1), 1.0 / math.sqrt(D) / 64.0, 8.0, S.STORE_I8)
-	gelu_var_fix_2 = 1.0 / ((1.0 / 3.0) + (0.5 / math.pi) * (1.0 / math.sqrt(3.0)))
-	S.epilogue_residual(S.gemm_i32(f, w2), x, math.sqrt(gelu_var_fix_2 / F) / 64.0, 1.0, S.STORE_E4M3)
+	S.epilogue_residual(S.gemm_i32(f, w2), x, math.sqrt(recipes.GELU_VAR_FIX_2 / F) / 64.0, 1.0, S.STORE_E4M3)
 	dt = time.perf_counter() - t0
-	ops = 2.0 * M * D * 2 * F + 2.0 * M * F * 2 * D
-	return {"value": ops / dt / 1e12, "unit": "TOPS", "cores": S.num_threads(), "kind": "port",
-	        "sample": f"{M} of 8192 token rows of config 2 (both GEMMs + epilogues), {dt:.1f} s of CPU time"}
+	out["config2_int8_ffn"] = {"value": (2.0 * M * D * 2 * F + 2.0 * M * F * 2 * D) / dt / 1e12, "unit": "TOPS",
+	                           "cores": S.num_threads(), "kind": "port",
+	                           "sample": f"{M} of 8192 token rows, both GEMMs + epilogues, {dt:.1f} s"}
+	del x, w1, w2, f
+	# config 3: the e4m3 FFN pair, 256 of the 16384 token rows (f32 sums in k order)
+	M3, D3, F3 = 256, 4096, 16384
+	x3, w13, w23 = _rand_e4m3(rng, (M3, D3)), _rand_e4m3(rng, (2 * F3, D3)), _rand_e4m3(rng, (2 * D3, F3))
+	r3 = _rand_codes(rng, (M3, D3))
+	t0 = time.perf_counter()
+	f3 = S.epilogue_geglu(S.gemm_f32_seq(x3, True, w13, True), 1.0 / math.sqrt(D3), 1.0, S.STORE_E4M3)
+	S.epilogue_residual(S.gemm_f32_seq(f3, True, w23, True), r3, math.sqrt(recipes.GELU_VAR_FIX_2 / F3), 1.0, S.STORE_E4M3)
+	dt = time.perf_counter() - t0
+	out["config3_fp8_ffn"] = {"value": (2.0 * M3 * D3 * 2 * F3 + 2.0 * M3 * F3 * 2 * D3) / dt / 1e12, "unit": "TFLOP/s",
+	                          "cores": S.num_threads(), "kind": "port",
+	                          "sample": f"{M3} of 16384 token rows, both GEMMs + epilogues, {dt:.1f} s"}
+	del w13
+	del x3, w23, f3
+	# config 5: prefill over the first 8192 positions of 2 of the 32 heads; decode of 2 of the 64 sequences
+	T5, H5, HD5, W5 = 8192, 8, 128, 4096
+	q5, kv5 = _rand_codes(rng, (T5, H5 * HD5)), _rand_codes(rng, (T5, 2 * H5 * HD5))
+	sk5, sv5 = _rand_codes(rng, (H5, HD5)), _rand_codes(rng, (H5, HD5))
+	t0 = time.perf_counter()
+	S.attn_fwd_i8(q5, kv5, sk5, sv5, np.ones(H5, np.float32), H5, HD5, W5, want_l=False)
+	dt = time.perf_counter() - t0
+	ops5 = 4.0 * HD5 * H5 * (W5 * (W5 - 1) // 2 + (T5 - W5) * W5)
+	out["config5_prefill"] = {"value": ops5 / dt / 1e12, "unit": "TOPS", "cores": S.num_threads(), "kind": "port",
+	                          "sample": f"positions 0..{T5 - 1} of {H5} of the 32 heads (window 4096), {dt:.1f} s"}
+	SD, CAP, HDEC = 16, 4096, 32
+	cache = _rand_codes(rng, (SD, CAP, 2 * HDEC * HD5))
+	qd = _rand_codes(rng, (SD, HDEC * HD5))
+	skd, svd = _rand_codes(rng, (HDEC, HD5)), _rand_codes(rng, (HDEC, HD5))
+	t0 = time.perf_counter()
+	S.attn_decode_i8(qd, cache, np.full(SD, CAP, np.uint32), skd, svd, np.ones(HDEC, np.float32), HDEC, HD5, W5)
+	dt = time.perf_counter() - t0
+	out["config5_decode"] = {"value": cache.nbytes / dt / 1e9, "unit": "GB/s of cache", "cores": S.num_threads(), "kind": "port",
+	                         "sample": f"{SD} of the 64 sequences (4096 cached positions x 32 heads each), {dt:.2f} s"}
+	return out
 
 
 def mfma_probe(dev, X):
@@ -152,7 +278,7 @@ def extras(dev, X, recipes):
 	out = {}
 	rng = np.random.default_rng(3000)
 
-	def gemm_entry(kern, a, b, c, extra, peak, iters=20, warm=5):
+	def gemm_entry(kern, a, b, c, extra, peak, iters=GEMM_TIMED, warm=GEMM_WARM):
 		med, mn = _median_launch(dev, X, lambda: kern.launch(a, b, c, extra), iters, warm)
 		ops = kern.n_ops(a, b)
 		return {"median_us": med * 1e6, "min_us": mn * 1e6, "tops": ops / med / 1e12, "frac_of_peak": ops / med / 1e12 / peak}
@@ -169,6 +295,19 @@ def extras(dev, X, recipes):
 		tag = "strict" if strict else "fast"
 		c2[f"ffn_f_{tag}"] = gemm_entry(recipes.ffn_f_kernel(dev, D, 2 * F, strict, X.INT8), x, w1, f, None, PEAK_INT8_TOPS)
 		c2[f"ffn_y_{tag}"] = gemm_entry(recipes.ffn_y_kernel(dev, D, F, strict, X.INT8, X.INT8), f, w2, y, x, PEAK_INT8_TOPS)
+	# both launches back to back, 50 steps after 10 (the headline of earlier versions of this benchmark)
+	kf, ky = recipes.ffn_f_kernel(dev, D, 2 * F, False, X.INT8), recipes.ffn_y_kernel(dev, D, F, False, X.INT8, X.INT8)
+	def pair():
+		kf.launch(x, w1, f)
+		ky.launch(f, w2, y, x)
+	for _ in range(10):
+		pair()
+	dev.synchronize()
+	t0 = time.perf_counter()
+	for _ in range(50):
+		pair()
+	dev.synchronize()
+	c2["pair_back_to_back_tops"] = (kf.n_ops(x, w1) + ky.n_ops(f, w2)) * 50 / (time.perf_counter() - t0) / 1e12
 	# the same pair in the literal form of the config text: per-token / per-output-channel scale vectors
 	# applied in the epilogue, bf16 out (W2 ungated: N_raw = d_model)
 	rs = X.Tensor.from_numpy(dev, (0.01 + 0.01 * rng.random(M)).astype(np.float32), X.F32)
@@ -180,7 +319,7 @@ def extras(dev, X, recipes):
 	kd1 = recipes.dequant_gemm_kernel(dev, D, 2 * F, X.INT8, X.INT8, True, False)
 	kd2 = recipes.dequant_gemm_kernel(dev, F, D, X.INT8, X.INT8, False, False)
 	for name, kern, a_, b_, c_, cs_ in (("dequant_geglu_bf16", kd1, x, w1, hb, cs1), ("dequant_bf16", kd2, f, w2l, yb, cs2)):
-		med, mn = _median_launch(dev, X, lambda: kern.launch_dequant(a_, b_, c_, rs, cs_), 20, 5)
+		med, mn = _median_launch(dev, X, lambda: kern.launch_dequant(a_, b_, c_, rs, cs_), GEMM_TIMED, GEMM_WARM)
 		ops = kern.n_ops(a_, b_)
 		c2[name] = {"median_us": med * 1e6, "min_us": mn * 1e6, "tops": ops / med / 1e12, "frac_of_peak": ops / med / 1e12 / PEAK_INT8_TOPS}
 	out["config2_int8_ffn"] = c2
@@ -194,75 +333,45 @@ def extras(dev, X, recipes):
 	x3 = X.Tensor.from_numpy(dev, e4m3_rand((M3, D3)), X.E4M3)
 	w13 = X.Tensor.from_numpy(dev, e4m3_rand((2 * F3, D3)), X.E4M3)
 	f3 = X.Tensor(dev, (M3, F3), X.E4M3)
-	c3 = {"ffn_f_f8": gemm_entry(recipes.ffn_f_f8_kernel(dev, D3, 2 * F3, False), x3, w13, f3, None, PEAK_FP8_TFLOPS, 10, 3)}
+	c3 = {"ffn_f_f8": gemm_entry(recipes.ffn_f_f8_kernel(dev, D3, 2 * F3, False), x3, w13, f3, None, PEAK_FP8_TFLOPS, 30, 10)}
 	del w13
 	w23 = X.Tensor.from_numpy(dev, e4m3_rand((2 * D3, F3)), X.E4M3)
 	r3 = X.Tensor.from_numpy(dev, _rand_codes(rng, (M3, D3)), X.INT8)
 	y3 = X.Tensor(dev, (M3, D3), X.E4M3)
-	c3["ffn_y_f8"] = gemm_entry(recipes.ffn_y_kernel(dev, D3, F3, False, X.E4M3, X.E4M3), f3, w23, y3, r3, PEAK_FP8_TFLOPS, 10, 3)
+	c3["ffn_y_f8"] = gemm_entry(recipes.ffn_y_kernel(dev, D3, F3, False, X.E4M3, X.E4M3), f3, w23, y3, r3, PEAK_FP8_TFLOPS, 30, 10)
 	out["config3_fp8_ffn"] = c3
 	del x3, w23, f3, r3, y3
 
-	# ---- config 4: block forward, 4 x 8192 tokens, d_model 2048, 16 heads x 128, window 512, d_ff 8192
-	T, B, H, HD, W = 8192, 4, 16, 128, 512
-	rows = T * B
-	xb = X.Tensor.from_numpy(dev, (rng.standard_normal((rows, D), dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16), X.BF16)
-	xi = X.Tensor(dev, (rows, D), X.INT8)
-	wq = X.Tensor.from_numpy(dev, _rand_codes(rng, (H * HD, D)), X.INT8)
-	wkv = X.Tensor.from_numpy(dev, _rand_codes(rng, (2 * H * HD, D)), X.INT8)
-	wy = X.Tensor.from_numpy(dev, _rand_codes(rng, (2 * D, H * HD)), X.INT8)
-	wf = X.Tensor.from_numpy(dev, _rand_codes(rng, (2 * F, D)), X.INT8)
-	wfy = X.Tensor.from_numpy(dev, _rand_codes(rng, (2 * D, F)), X.INT8)
-	sk = X.Tensor.from_numpy(dev, _rand_codes(rng, (H, HD)), X.INT8)
-	sv = X.Tensor.from_numpy(dev, _rand_codes(rng, (H, HD)), X.INT8)
-	temp = X.Tensor.from_numpy(dev, (0.5 + rng.random(H)).astype(np.float32), X.F32)
-	q = X.Tensor(dev, (rows, H * HD), X.INT8)
-	kv = X.Tensor(dev, (rows, 2 * H * HD), X.INT8)
-	rrms = X.Tensor(dev, (rows, H), X.F32)
-	ao = X.Tensor(dev, (rows, H * HD), X.INT8)
-	al = X.Tensor(dev, (H, rows), X.F32)
-	ay = X.Tensor(dev, (rows, D), X.E4M3)
-	ff = X.Tensor(dev, (rows, F), X.E4M3)
-	fy = X.Tensor(dev, (rows, D), X.E4M3)
-	k_rms = recipes.rms_norm_kernel(dev, D, X.BF16)
-	k_q = recipes.attn_q_kernel(dev, D, H * HD)
-	k_kv = recipes.attn_kv_kernel(dev, D, 2 * H * HD, HD)
-	k_at = recipes.attn_kernel(dev, H, HD, False)
-	k_ay = recipes.attn_y_kernel(dev, D, H * HD, False)
-	k_ff = recipes.ffn_f_kernel(dev, D, 2 * F, False)
-	k_fy = recipes.ffn_y_kernel(dev, D, F, False)
-	stages = [
-		("rms_norm", lambda: k_rms.launch(xb, xi)),
-		("attn_q", lambda: k_q.launch(xi, wq, q)),
-		("attn_kv", lambda: k_kv.launch(xi, wkv, kv, rrms)),
-		("attn_fwd_i8", lambda: k_at.launch(q, kv, sk, sv, temp, ao, al, W, B)),
-		("attn_y", lambda: k_ay.launch(ao, wy, ay, xi)),
-		("ffn_f", lambda: k_ff.launch(xi, wf, ff)),
-		("ffn_y_f8", lambda: k_fy.launch(ff, wfy, fy, xi)),
-	]
+	# ---- config 4 per stage (the headline's block): median of each stage launched alone, both projection forms
+	c = CONFIG4
+	T, B, H, HD, W, F4 = c["T"], c["B"], c["H"], c["HD"], c["W"], c["F"]
 	c4 = {}
-	total = 0.0
-	for name, fn in stages:
-		med, mn = _median_launch(dev, X, fn, 10, 3)
-		c4[name + "_us"] = med * 1e6
-		total += med
+	for fused in (False, True) if hasattr(recipes, "attn_qkv_kernel") else (False,):
+		block, xb, wts, outs, rows = config4_block(dev, X, fused)
+		ops = block.n_ops(rows)
+		total = 0.0
+		for name, fn in block.stages(xb, wts, outs):
+			if fused and name != "attn_qkv":
+				continue
+			iters, warm = (ATTN_TIMED, ATTN_WARM) if name == "attn_fwd_i8" else (30, 10)
+			med, mn = _median_launch(dev, X, fn, iters, warm)
+			c4[name + "_us"] = med * 1e6
+			if name in ops:
+				c4[name + "_tops"] = ops[name] / med / 1e12
+			total += med
+		if not fused:
+			c4["sum_of_stage_medians_us"] = total * 1e6
+		del block, xb, wts, outs
 	pairs = W * (W - 1) // 2 + (T - W) * W
-	attn_ops = 4.0 * HD * H * B * pairs
-	c4["attn_tops"] = attn_ops / (c4["attn_fwd_i8_us"] * 1e-6) / 1e12
-	c4["attn_frac_of_int8_peak"] = c4["attn_tops"] / PEAK_INT8_TOPS
+	c4["attn_fwd_i8_tops"] = 4.0 * HD * H * B * pairs / (c4["attn_fwd_i8_us"] * 1e-6) / 1e12     # visible (query, key) pairs only
+	c4["attn_frac_of_int8_peak"] = c4["attn_fwd_i8_tops"] / PEAK_INT8_TOPS
 	c4["rms_norm_gbs"] = rows * D * 3 / (c4["rms_norm_us"] * 1e-6) / 1e9
 	c4["rms_norm_frac_of_hbm"] = c4["rms_norm_gbs"] / PEAK_HBM_GBS
-	c4["ffn_y_f8_tflops"] = 2.0 * rows * F * 2 * D / (c4["ffn_y_f8_us"] * 1e-6) / 1e12
-	c4["block_tokens_per_s"] = rows / total
-	# end to end, back to back on the stream
-	def block():
-		for _, fn in stages:
-			fn()
-	med, _ = _median_launch(dev, X, block, 5, 2)
-	c4["block_back_to_back_us"] = med * 1e6
-	c4["block_tokens_per_s_back_to_back"] = rows / med
-	out["config4_block"] = c4
-	del xb, xi, wq, wkv, wy, wf, wfy, q, kv, rrms, ao, al, ay, ff, fy
+	for name in ("attn_q", "attn_kv", "attn_qkv", "attn_y", "ffn_f"):
+		if name + "_tops" in c4:
+			c4[name + "_frac_of_int8_peak"] = c4[name + "_tops"] / PEAK_INT8_TOPS
+	c4["ffn_y_f8_frac_of_f16_peak"] = c4["ffn_y_f8_tops"] / PEAK_F16_TFLOPS
+	out["config4_block_stages"] = c4
 
 	# ---- config 1: attention T=1024, H=8, hd=64, W=256
 	T1, H1, HD1, W1 = 1024, 8, 64, 256
@@ -273,7 +382,7 @@ def extras(dev, X, recipes):
 	tp1 = X.Tensor.from_numpy(dev, np.ones(H1, np.float32), X.F32)
 	o1 = X.Tensor(dev, (T1, H1 * HD1), X.INT8)
 	k1 = recipes.attn_kernel(dev, H1, HD1, False)
-	med, _ = _median_launch(dev, X, lambda: k1.launch(q1, kv1, sk1, sv1, tp1, o1, None, W1), 20, 5)
+	med, _ = _median_launch(dev, X, lambda: k1.launch(q1, kv1, sk1, sv1, tp1, o1, None, W1), 100, 50)
 	p1 = W1 * (W1 - 1) // 2 + (T1 - W1) * W1
 	out["config1_attn"] = {"median_us": med * 1e6, "gops": 4.0 * HD1 * H1 * p1 / 1e9, "tops": 4.0 * HD1 * H1 * p1 / med / 1e12}
 
@@ -286,7 +395,7 @@ def extras(dev, X, recipes):
 	rs1 = row_scale_tensors(T1, H1)
 	ob1 = X.Tensor(dev, (T1, H1 * HD1), X.BF16)
 	k1r = recipes.attn_row_scaled_kernel(dev, H1, HD1, X.BF16, False)
-	med, _ = _median_launch(dev, X, lambda: k1r.launch_row_scaled(q1, kv1, sk1, sv1, tp1, ob1, None, W1, *rs1), 20, 5)
+	med, _ = _median_launch(dev, X, lambda: k1r.launch_row_scaled(q1, kv1, sk1, sv1, tp1, ob1, None, W1, *rs1), 100, 50)
 	out["config1_attn_row_scaled_bf16"] = {"median_us": med * 1e6, "tops": 4.0 * HD1 * H1 * p1 / med / 1e12}
 
 	# ---- config 5: prefill T=65536, H=32, hd=128, W=4096; decode 64 sequences x 4096 cached positions
@@ -300,7 +409,7 @@ def extras(dev, X, recipes):
 	c5 = {}
 	for strict in (False, True):
 		k5 = recipes.attn_kernel(dev, H5, HD5, strict)
-		med, _ = _median_launch(dev, X, lambda: k5.launch(q5, kv5, sk5, sv5, tp5, o5, None, W5), 3, 1)
+		med, _ = _median_launch(dev, X, lambda: k5.launch(q5, kv5, sk5, sv5, tp5, o5, None, W5), ATTN_TIMED, 3)
 		p5 = W5 * (W5 - 1) // 2 + (T5 - W5) * W5
 		tag = "strict" if strict else "fast"
 		c5[f"prefill_{tag}_ms"] = med * 1e3
@@ -309,7 +418,7 @@ def extras(dev, X, recipes):
 	rs5 = row_scale_tensors(T5, H5)
 	ob5 = X.Tensor(dev, (T5, H5 * HD5), X.BF16)
 	k5r = recipes.attn_row_scaled_kernel(dev, H5, HD5, X.BF16, False)
-	med, _ = _median_launch(dev, X, lambda: k5r.launch_row_scaled(q5, kv5, sk5, sv5, tp5, ob5, None, W5, *rs5), 3, 1)
+	med, _ = _median_launch(dev, X, lambda: k5r.launch_row_scaled(q5, kv5, sk5, sv5, tp5, ob5, None, W5, *rs5), ATTN_TIMED, 3)
 	c5["prefill_row_scaled_bf16_ms"] = med * 1e3
 	c5["prefill_row_scaled_bf16_tops"] = 4.0 * HD5 * H5 * p5 / med / 1e12
 	del q5, kv5, o5, ob5, rs5
@@ -319,15 +428,22 @@ def extras(dev, X, recipes):
 	qd = X.Tensor.from_numpy(dev, _rand_codes(rng, (S5, H5 * HD5)), X.INT8)
 	lens = X.Tensor.from_numpy(dev, np.full(S5, CAP, np.uint32).view(np.float32), X.F32)
 	od = X.Tensor(dev, (S5, H5 * HD5), X.INT8)
+	nbytes = S5 * CAP * 2 * H5 * HD5                  # the whole cache: what the recurrence reads when no probability rounds to 0
+	q_flat = X.Tensor.from_numpy(dev, np.zeros((S5, H5 * HD5), np.int8), X.INT8)
 	for strict in (False, True):
 		kd = recipes.attn_decode_kernel(dev, H5, HD5, CAP, strict)
-		med, _ = _median_launch(dev, X, lambda: kd.launch(qd, cache, lens, sk5, sv5, tp5, od, None, W5), 10, 3)
-		nbytes = S5 * CAP * 2 * H5 * HD5
 		tag = "strict" if strict else "fast"
-		c5[f"decode_{tag}_us"] = med * 1e6
-		c5[f"decode_{tag}_cache_gbs"] = nbytes / med / 1e9            # whole cache / time: counts the V rows skipped
-		c5[f"decode_{tag}_hbm_gbs"] = DECODE_TRAFFIC_BYTES / med / 1e9  # bytes actually fetched (rocprofv3) / time
-		c5[f"decode_{tag}_frac_of_hbm"] = DECODE_TRAFFIC_BYTES / med / 1e9 / PEAK_HBM_GBS
+		# dense case: an all-zero query gives every key the same score, so every 8-bit probability is 255 and every
+		# K and V row of the window is read -- the roofline figure of the kernel
+		med, _ = _median_launch(dev, X, lambda: kd.launch(q_flat, cache, lens, sk5, sv5, tp5, od, None, W5), 30, 10)
+		c5[f"decode_dense_{tag}_us"] = med * 1e6
+		c5[f"decode_dense_{tag}_gbs"] = nbytes / med / 1e9
+		c5[f"decode_dense_{tag}_frac_of_hbm"] = nbytes / med / 1e9 / PEAK_HBM_GBS
+		# Gaussian queries and cache: about 99 % of the 8-bit probabilities are 0 and their V rows are not fetched.
+		# The rate below divides the WHOLE cache by the time: work avoided, not bandwidth (it can exceed the HBM peak).
+		med, _ = _median_launch(dev, X, lambda: kd.launch(qd, cache, lens, sk5, sv5, tp5, od, None, W5), 30, 10)
+		c5[f"decode_gaussian_{tag}_us"] = med * 1e6
+		c5[f"decode_gaussian_{tag}_cache_gbs_work_avoided"] = nbytes / med / 1e9
 	# the cache as a row-scaled prefill leaves it: one scale per (row, head) of k and v, bf16 output
 	kd_rows = recipes.attn_decode_row_scaled_kernel(dev, H5, HD5, CAP, X.BF16, False)
 	scale_one = [(0.125 * (0.75 + 0.5 * rng.random((1, H5, CAP)))).astype(np.float32) for _ in range(2)]
@@ -335,7 +451,7 @@ def extras(dev, X, recipes):
 	f32t = lambda a: X.Tensor.from_numpy(dev, np.ascontiguousarray(a, dtype=np.float32), X.F32)
 	rsd = [f32t(0.125 * (0.75 + 0.5 * rng.random((S5, H5)))), f32t(np.broadcast_to(scale_one[0], (S5, H5, CAP))), f32t(vw5), f32t(sw5), f32t(os5)]
 	odb = X.Tensor(dev, (S5, H5 * HD5), X.BF16)
-	med, _ = _median_launch(dev, X, lambda: kd_rows.launch_row_scaled(qd, cache, lens, sk5, sv5, tp5, odb, None, W5, *rsd), 10, 3)
+	med, _ = _median_launch(dev, X, lambda: kd_rows.launch_row_scaled(qd, cache, lens, sk5, sv5, tp5, odb, None, W5, *rsd), 30, 10)
 	c5["decode_row_scaled_bf16_us"] = med * 1e6
 	out["config5_long_context"] = c5
 	# what the matrix cores sustain with no memory traffic at all, beside the nominal peaks used above
@@ -425,6 +541,7 @@ def main():
 	ap.add_argument("--warmup", type=int, default=10)
 	ap.add_argument("--no-extras", action="store_true")
 	ap.add_argument("--no-cpu", action="store_true")
+	ap.add_argument("--fused-qkv", action="store_true", help="headline block with the q and kv projections as one launch")
 	ap.add_argument("--copy-probe", action="store_true",
 	                help="only run a 1 GiB device-to-device copy kernel (calibrates the HBM traffic counters)")
 	ap.add_argument("--mfma-probe", action="store_true",
@@ -458,26 +575,35 @@ def main():
 	if args.only:
 		single(dev, X, recipes, args.only, args.steps)
 		return
-	h = headline(dev, X, recipes, args.steps, args.warmup)
-	value = h["ops_per_step"] * args.steps / h["wall_s"] / 1e12
-	achieved = h["k1_ops"] / h["k1_mean_s"] / 1e12
+	h = headline(dev, X, args.steps, args.warmup, args.fused_qkv)
+	value = h["rows"] * args.steps / h["wall_s"]
+	achieved = h["dominant_ops"] / h["dominant_mean_s"] / 1e12
+	traffic_file = "gemm_b8_ffn_y_f8_config4.txt"
+	traffic = profile_traffic(traffic_file)
+	c = CONFIG4
 	line = {
-		"metric": "int8 TOPS at 1 MI355X (config 2: FFN GEMM pair ffn_f_fwd + ffn_y_fwd_i8); fp8 TOPS, block-fwd tokens/sec and % of MFMA/HBM roofline under extras",
-		"value": value, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+		"metric": "block-fwd tokens/sec at 1 MI355X (config 4: full quantized block forward); int8/fp8 TOPS and % of "
+		          "MFMA/HBM roofline per kernel under extras",
+		"value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
 		"ms_per_step": h["wall_s"] / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
 		"vs_baseline": None, "dtype": "int8", "data": "synthetic",
-		"config": {"workload": "config 2: int8 FFN GEMM pair, tokens=8192, d_model=2048, d_ff=8192 (gated layout: "
-		                       "W1 [16384, 2048] GeGLU -> FixedI8, W2 [4096, 8192] gated residual -> e4m3)",
-		           "math": "hardware transcendentals in the epilogues (strict build reported under extras)"},
-		"roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
-		             "frac": achieved / PEAK_INT8_TOPS, "traffic": FFN_F_TRAFFIC_BYTES,
-		             "kernel": "gemm_b8 (ffn_f_fwd: M=8192, K=2048, N_raw=16384, GeGLU epilogue)",
-		             "mean_launch_us": h["k1_mean_s"] * 1e6},
+		"config": {"workload": f"config 4: full quantized block forward, batch {c['B']} x seq {c['T']} tokens, d_model {c['D']}, "
+		                       f"{c['H']} heads x {c['HD']}, window {c['W']}, d_ff {c['F']}; stages " + " -> ".join(h["stage_names"]),
+		           "operands": "bf16 residual stream in; FixedI8 x, q, kv, attention out; int8 weights; e4m3 attn_y, ffn_f, ffn_y "
+		                       "(int8 x int8 -> int32 on the int8 matrix cores; ffn_y e4m3 x int8 -> f32 on the f16 matrix cores)",
+		           "math": "hardware transcendentals in the epilogues and the softmax (the bit-exact strict builds are the tests')"},
+		"roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
+		             "frac": achieved / PEAK_F16_TFLOPS, "traffic": traffic,
+		             "traffic_source": "profiles/" + traffic_file if traffic is not None else None,
+		             "kernel": "gemm_b8 (ffn_y_fwd_f8: M=32768, K=8192, N_raw=4096, e4m3 x int8 widened to f16, gated-residual epilogue)",
+		             "mean_launch_us": h["dominant_mean_s"] * 1e6},
 	}
 	if not args.no_cpu:
 		line["cpu_baseline"] = cpu_baseline()
 	if not args.no_extras:
 		line["extras"] = extras(dev, X, recipes)
+		if not args.no_cpu:
+			line["extras"]["cpu_baselines"] = cpu_extras()
 	dev.synchronize()
 	print(json.dumps(line))
 
