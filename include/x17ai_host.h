@@ -34,7 +34,12 @@ enum { X17H_E4M3 = 0, X17H_INT8 = 1, X17H_BF16 = 2, X17H_F32 = 3 };
 /* epilogues, src/device/cuda/gemm.rs:322-349 */
 enum { X17H_EPI_SCALE = 0, X17H_EPI_GEGLU = 1, X17H_EPI_RESIDUAL = 2, X17H_EPI_RMSNORM = 3,
        /* no counterpart in gemm.rs: run-time per-row x per-column f32 scales, bf16 output */
-       X17H_EPI_DEQUANT = 4 };
+       X17H_EPI_DEQUANT = 4,
+       /* the older Q writer with a learned bf16 scale per column, cuda/qkvg_fwd_i8.cuh:145-219 (launch: extra =
+        * q_norm_scales bf16 [b_rows]; head_dim, eps and out_scale as for RMSNorm, no V halves) */
+       X17H_EPI_QNORM = 5,
+       /* no counterpart in gemm.rs: the q (Scale) and kv (RMSNorm) projections as one launch, x17h_gemm_kernel_launch_qkv */
+       X17H_EPI_QKV = 6 };
 enum { X17H_ACT_NONE = 0, X17H_ACT_GEGLU = 1 };
 
 char const *x17h_last_error(void);
@@ -87,6 +92,11 @@ typedef struct X17hGemmConfig {
 	size_t sep_dim;          /* RMSNorm only */
 	int strict_math;         /* 1: deterministic transcendentals (parity build), 0: hardware ones */
 	int activation;          /* Dequant only: X17H_ACT_* */
+	/* X17H_EPI_QKV only: raw columns [0, q_cols) are the q projection (Scale writer with q_inp_scale * q_out_scale),
+	 * the other b_rows - q_cols the kv projection (RMSNorm writer with inp_scale, out_scale, eps, head_dim, sep_dim) */
+	size_t q_cols;
+	double q_inp_scale;
+	double q_out_scale;
 } X17hGemmConfig;
 
 /* GemmKernel::<E>::new, gemm.rs:368-437.  dev == NULL: generate and compile only. */
@@ -98,6 +108,11 @@ int x17h_gemm_kernel_launch(X17hGemmKernel *k, X17hTensor *a, X17hTensor *b, X17
  * row_scale f32 [M], col_scale f32 [N_raw].  No counterpart in the reference (its scales are constants). */
 int x17h_gemm_kernel_launch_dequant(X17hGemmKernel *k, X17hTensor *a, X17hTensor *b, X17hTensor *c,
                                     X17hTensor *row_scale, X17hTensor *col_scale);
+/* X17H_EPI_QKV: the q projection (src/main.rs:387-438) and the kv projection (:440-493) as one launch that reads x
+ * once.  x i8 [M, K]; q_weights i8 [q_cols, K]; kv_weights i8 [b_rows - q_cols, K]; q i8 [M, q_cols];
+ * kv i8 [M, b_rows - q_cols]; rrms f32 [M, heads].  Outputs equal those of the two separate kernels bit for bit. */
+int x17h_gemm_kernel_launch_qkv(X17hGemmKernel *k, X17hTensor *x, X17hTensor *q_weights, X17hTensor *kv_weights,
+                                X17hTensor *q, X17hTensor *kv, X17hTensor *rrms);
 /* GemmKernel::n_ops, gemm.rs:445-449 */
 double x17h_gemm_kernel_n_ops(X17hGemmKernel *k, X17hTensor *a, X17hTensor *b);
 /* launch geometry read back from meta.json: THREADS_PER_BLOCK, SMEM_BYTES, M_PER_BLOCK, N_PER_BLOCK */

@@ -411,6 +411,45 @@ X17_EXPORT void x17o_epilogue_l2norm(const int32_t *acc, int8_t *C, float *rrms,
 	}
 }
 
+/* The learned-scale Q writer: QMatrixWriter, cuda/qkvg_fwd_i8.cuh:145-219, whose l2_norm<USE_DYN_SCALE = true>
+ * (:16-85) survives in the live header as kv_helpers::l2_norm (cuda/gemm_b8.cuh:761-824).  Every `hd` raw columns
+ * of a row are one head (no V halves): partial sums and total as in x17o_epilogue_l2norm,
+ * scale = rsq(S + eps) * f32(head_scale), and column c is stored as
+ *   fixedi8( (x[c] * scale) * f32(dyn[c]) )         -- two multiplies in that order (gemm_b8.cuh:819-820)
+ * with dyn a bf16 vector of N_raw learned scales (given as bf16 bit patterns).  The old writer adds no eps
+ * (qkvg_fwd_i8.cuh:56) and takes head_scale = sqrt(hd) * 8 (:205); the live hook adds EPS (gemm_b8.cuh:808).
+ * rrms (may be NULL) receives scale per (row, head).
+ * Parity note: the old writer's final store goes through a base class (b8::FixedI8MatrixWriter) that no longer
+ * exists in the reference tree; the FixedI8 conversion of the live writers (clamp to +-127, round to nearest even)
+ * is assumed for it. */
+X17_EXPORT void x17o_epilogue_qnorm(const int32_t *acc, int8_t *C, float *rrms, const uint16_t *dyn_bf16,
+                                    size_t M, size_t N_raw, size_t hd, double eps, double head_scale) {
+	size_t heads = N_raw / hd;
+	float feps = (float)eps, fhs = (float)head_scale;
+	#pragma omp parallel for schedule(static)
+	for (size_t m = 0; m < M; ++m) {
+		for (size_t h = 0; h < heads; ++h) {
+			const int32_t *a = acc + m * N_raw + h * hd;
+			int8_t *c = C + m * N_raw + h * hd;
+			float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+			for (size_t d = 0; d < hd; ++d) {
+				float x = (float)a[d];
+				size_t q = (d % 8) / 2;
+				s[q] = fmaf(x, x, s[q]);
+			}
+			float S = (s[0] + s[1]) + (s[2] + s[3]);
+			float scale = sfu_rsq(S + feps) * fhs;
+			for (size_t d = 0; d < hd; ++d) {
+				uint32_t bits = (uint32_t)dyn_bf16[h * hd + d] << 16;
+				float dyn;
+				memcpy(&dyn, &bits, 4);
+				c[d] = fixedi8(((float)a[d] * scale) * dyn);
+			}
+			if (rrms != NULL) rrms[m * heads + h] = scale;
+		}
+	}
+}
+
 /* ------------------------------------------------------------------ attention
  * AttnForward::run cuda/attn_fwd_i8.cuh:368-619 restated per (head, query):
  *   window rounded up to a multiple of 16 (:409-412); query i sees keys

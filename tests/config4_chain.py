@@ -66,6 +66,18 @@ def run_strict(dev, inp, fused_qkv: bool = False):
 	return {k: t.download() for k, t in out.items()}
 
 
+def run_fused_qkv(dev, got, strict: bool = True):
+	"""q, kv and rrms of the fused projection kernel on the FixedI8 x of `got` (run_strict's result)."""
+	inp = inputs()
+	k = recipes.attn_qkv_kernel(dev, D, H * HD, 2 * H * HD, HD, strict)
+	q = X.Tensor(dev, (ROWS, H * HD), X.INT8)
+	kv = X.Tensor(dev, (ROWS, 2 * H * HD), X.INT8)
+	rr = X.Tensor(dev, (ROWS, H), X.F32)
+	k.launch_qkv(X.Tensor.from_numpy(dev, got["x"], X.INT8), X.Tensor.from_numpy(dev, inp["attn_q_weights"], X.INT8),
+	             X.Tensor.from_numpy(dev, inp["attn_kv_weights"], X.INT8), q, kv, rr)
+	return {"q": q.download(), "kv": kv.download(), "k_rrms": rr.download()}
+
+
 def sample_rows(rng, count=96):
 	# first / last rows, rows either side of 256-row tile edges and of sequence edges, random ones
 	fixed = [0, 1, 255, 256, 257, T - 1, T, T + 1, 2 * T - 257, ROWS - 256, ROWS - 1]

@@ -336,3 +336,8 @@ def test_config4_block_chain(dev):
 	for name in ("attn_y", "ffn_f", "ffn_y_f8"):
 		r = rep[name]
 		assert r["frac_mismatched"] < 5e-3 and r["frac_beyond_one_code"] == 0.0, (name, r)
+	# the q and kv projections as one launch (24 column tiles, the first 8 through the Scale writer): the same bytes
+	fused = C.run_fused_qkv(dev, got)
+	for name in ("q", "kv"):
+		assert np.array_equal(fused[name], got[name]), name
+	assert np.array_equal(fused["k_rrms"].view(np.uint32), got["k_rrms"].view(np.uint32))

@@ -90,6 +90,84 @@ def test_l2norm_epilogue_bit_exact(dev, hd, m, k):
 	assert np.array_equal(rrms.download().view(np.uint32), want_r.view(np.uint32))
 
 
+@pytest.mark.parametrize("hd", [64, 128])
+def test_l2norm_epilogue_on_a_walk_of_more_tiles_than_workgroups(dev, hd):
+	"""2048 tokens x 2048 raw columns = 512 output tiles over the 256 persistent workgroups: every workgroup writes two
+	tiles with the next tile's loads and the rrms stores in flight; heads of 64 and 128 columns."""
+	m, k, n = 2048, 256, 2048
+	rng = rng_for("l2-walk", hd)
+	a, b = i8_codes(rng, (m, k)), i8_codes(rng, (n, k))
+	kern = recipes.attn_kv_kernel(dev, k, n, hd)
+	c = X.Tensor(dev, (m, n), X.INT8)
+	rrms = X.Tensor(dev, (m, n // (2 * hd)), X.F32)
+	kern.launch(_up(dev, a, X.INT8), _up(dev, b, X.INT8), c, rrms)
+	want_c, want_r = S.epilogue_l2norm(S.gemm_i32(a, b), hd, recipes.L2_NORM_EPS, 1.0 / math.sqrt(k) / 64.0, 8.0)
+	assert np.array_equal(c.download(), want_c)
+	assert np.array_equal(rrms.download().view(np.uint32), want_r.view(np.uint32))
+
+
+def _bf16_bits(x: np.ndarray) -> np.ndarray:
+	u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+	return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+@pytest.mark.parametrize("hd", [32, 64, 128])
+def test_learned_scale_q_writer_bit_exact(dev, hd):
+	"""cuda/qkvg_fwd_i8.cuh:145-219: every head L2-normalised, then a bf16 scale per column."""
+	m, k, n = 512, 512, 512
+	rng = rng_for("qnorm", hd)
+	a, b = i8_codes(rng, (m, k)), i8_codes(rng, (n, k))
+	dyn = _bf16_bits(0.25 + 1.5 * rng.random(n))
+	kern = recipes.attn_q_norm_kernel(dev, k, n, hd, 0.0)
+	c = X.Tensor(dev, (m, n), X.INT8)
+	kern.launch(_up(dev, a, X.INT8), _up(dev, b, X.INT8), c, _up(dev, dyn, X.BF16))
+	want = S.epilogue_qnorm(S.gemm_i32(a, b), hd, 0.0, 8.0, dyn)
+	got = c.download()
+	assert np.array_equal(got, want)
+	assert len(np.unique(got)) > 50                       # (not a constant, not saturated)
+	# the learned scales are column-wise: wrong scale vector, wrong answer
+	assert not np.array_equal(S.epilogue_qnorm(S.gemm_i32(a, b), hd, 0.0, 8.0, np.roll(dyn, 1)), want)
+
+
+def test_learned_scale_q_writer_with_eps_at_a_full_width(dev):
+	"""The hook that survives in the live header adds EPS (cuda/gemm_b8.cuh:808); 1024 columns = four column tiles."""
+	m, k, n, hd = 512, 2048, 1024, 128
+	rng = rng_for("qnorm-eps")
+	a, b = i8_codes(rng, (m, k)), i8_codes(rng, (n, k))
+	a[7] = 0                                                   # an all-zero token row: sum of squares 0, rsq(eps)
+	dyn = _bf16_bits(0.5 + rng.random(n))
+	kern = recipes.attn_q_norm_kernel(dev, k, n, hd, recipes.L2_NORM_EPS)
+	c = X.Tensor(dev, (m, n), X.INT8)
+	kern.launch(_up(dev, a, X.INT8), _up(dev, b, X.INT8), c, _up(dev, dyn, X.BF16))
+	want = S.epilogue_qnorm(S.gemm_i32(a, b), hd, recipes.L2_NORM_EPS, 8.0, dyn)
+	assert np.array_equal(c.download(), want)
+	assert not c.download()[7].any()
+
+
+@pytest.mark.parametrize("hd", [32, 64, 128])
+def test_fused_q_kv_projection_equals_the_two_kernels(dev, hd):
+	"""One launch for src/main.rs:387-493's two: q, kv and rrms bit for bit those of the oracle (and so of the separate
+	kernels)."""
+	m, k, nq, nkv = 512, 512, 256, 512
+	rng = rng_for("qkv", hd)
+	x, wq, wkv = i8_codes(rng, (m, k)), i8_codes(rng, (nq, k)), i8_codes(rng, (nkv, k))
+	kern = recipes.attn_qkv_kernel(dev, k, nq, nkv, hd)
+	q, kv = X.Tensor(dev, (m, nq), X.INT8), X.Tensor(dev, (m, nkv), X.INT8)
+	rrms = X.Tensor(dev, (m, nkv // (2 * hd)), X.F32)
+	kern.launch_qkv(_up(dev, x, X.INT8), _up(dev, wq, X.INT8), _up(dev, wkv, X.INT8), q, kv, rrms)
+	inp = 1.0 / math.sqrt(k) / 64.0
+	want_q = S.epilogue_scale(S.gemm_i32(x, wq), inp, 8.0)
+	want_kv, want_r = S.epilogue_l2norm(S.gemm_i32(x, wkv), hd, recipes.L2_NORM_EPS, inp, 8.0)
+	assert np.array_equal(q.download(), want_q)
+	assert np.array_equal(kv.download(), want_kv)
+	assert np.array_equal(rrms.download().view(np.uint32), want_r.view(np.uint32))
+	# shape checks of the launcher
+	with pytest.raises(X.X17Error):
+		kern.launch_qkv(_up(dev, x, X.INT8), _up(dev, wkv, X.INT8), _up(dev, wq, X.INT8), q, kv, rrms)
+	with pytest.raises(X.X17Error):
+		kern.launch(_up(dev, x, X.INT8), _up(dev, wq, X.INT8), q, rrms)
+
+
 @pytest.mark.parametrize("store", [X.E4M3, X.INT8])
 @pytest.mark.parametrize("m,k,n", SHAPES)
 def test_geglu_epilogue(dev, m, k, n, store):

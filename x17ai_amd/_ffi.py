@@ -37,6 +37,9 @@ class GemmConfigC(ctypes.Structure):
 		("sep_dim", ctypes.c_size_t),
 		("strict_math", ctypes.c_int),
 		("activation", ctypes.c_int),
+		("q_cols", ctypes.c_size_t),
+		("q_inp_scale", ctypes.c_double),
+		("q_out_scale", ctypes.c_double),
 	]
 
 
@@ -98,6 +101,7 @@ def host() -> ctypes.CDLL:
 	h.x17h_gemm_kernel_free.restype = None
 	h.x17h_gemm_kernel_launch.argtypes = [P, P, P, P, P]
 	h.x17h_gemm_kernel_launch_dequant.argtypes = [P, P, P, P, P, P]
+	h.x17h_gemm_kernel_launch_qkv.argtypes = [P, P, P, P, P, P, P]
 	h.x17h_gemm_kernel_n_ops.argtypes = [P, P, P]
 	h.x17h_gemm_kernel_n_ops.restype = ctypes.c_double
 	h.x17h_gemm_kernel_metadata.argtypes = [P, ctypes.POINTER(SZ)]

@@ -227,7 +227,40 @@ class DequantConfig:
 	kind = 4
 
 
-EpilogueConfig = Union[ScaleConfig, GeGluConfig, ResidualConfig, RMSNormConfig, DequantConfig]
+@dataclasses.dataclass
+class QNormConfig:
+	"""The reference's older Q writer (cuda/qkvg_fwd_i8.cuh:145-219; hook cuda/gemm_b8.cuh:761-824): every head_dim
+	raw columns are one L2-normalised head, times a learned bf16 scale per column passed at launch."""
+	eps: float
+	head_dim: int
+	out_scale: float
+	inp_scale: float = 1.0
+	kind = 5
+
+
+@dataclasses.dataclass
+class QkvConfig:
+	"""No counterpart in gemm.rs: the q projection (Scale writer) and the kv projection (RMSNorm writer) of
+	src/main.rs:387-493 as one launch over the same token rows.  Raw columns [0, q_cols) are q."""
+	q_cols: int
+	q: ScaleConfig
+	kv: RMSNormConfig
+	kind = 6
+
+	# the fields the flat configuration reads for the kv part
+	@property
+	def inp_scale(self): return self.kv.inp_scale
+	@property
+	def out_scale(self): return self.kv.out_scale
+	@property
+	def eps(self): return self.kv.eps
+	@property
+	def head_dim(self): return self.kv.head_dim
+	@property
+	def sep_dim(self): return self.kv.sep_dim
+
+
+EpilogueConfig = Union[ScaleConfig, GeGluConfig, ResidualConfig, RMSNormConfig, DequantConfig, QNormConfig, QkvConfig]
 
 
 def _attrs_dict(raw) -> dict:
@@ -257,6 +290,8 @@ class GemmKernel:
 		c.sep_dim = getattr(epilogue_config, "sep_dim", 0)
 		c.strict_math = int(strict_math)
 		c.activation = int(bool(getattr(epilogue_config, "geglu", False)))
+		if isinstance(epilogue_config, QkvConfig):
+			c.q_cols, c.q_inp_scale, c.q_out_scale = epilogue_config.q_cols, epilogue_config.q.inp_scale, epilogue_config.q.out_scale
 		self.device = device
 		self.name = kernel_name
 		self.epilogue_kind = epilogue_config.kind
@@ -270,6 +305,10 @@ class GemmKernel:
 
 	def launch_dequant(self, a: Tensor, b: Tensor, c: Tensor, row_scale: Tensor, col_scale: Tensor) -> None:
 		check(_ffi.host().x17h_gemm_kernel_launch_dequant(self._h, a._h, b._h, c._h, row_scale._h, col_scale._h))
+
+	def launch_qkv(self, x: Tensor, q_weights: Tensor, kv_weights: Tensor, q: Tensor, kv: Tensor, rrms: Tensor) -> None:
+		"""QkvConfig kernels: q = Scale(x . Wq^T), kv, rrms = RMSNorm(x . Wkv^T) in one launch."""
+		check(_ffi.host().x17h_gemm_kernel_launch_qkv(self._h, x._h, q_weights._h, kv_weights._h, q._h, kv._h, rrms._h))
 
 	def n_ops(self, a: Tensor, b: Tensor) -> float:
 		return float(_ffi.host().x17h_gemm_kernel_n_ops(self._h, a._h, b._h))

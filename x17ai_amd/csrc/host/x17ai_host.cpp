@@ -811,6 +811,49 @@ std::unique_ptr<GemmKernel> GemmKernel::create(std::shared_ptr<HipDevice> device
 		       << " // (" << one_line(c->inp_scale.description) << ") * (" << one_line(c->out_scale.description) << ")\n";
 	}
 
+	size_t q_cols = 0;
+	auto rmsnorm_defines = [&](RMSNormConfig const &c, size_t kv_rows) -> bool {
+		if (!std::isfinite(c.eps) || c.eps < 0.0 || !std::isfinite(c.inp_scale.value) || !std::isfinite(c.out_scale.value)) {
+			diag.add_error("invalid RMSNorm epilogue values"); return false;
+		}
+		if (c.head_dim != c.sep_dim || (c.head_dim != 32 && c.head_dim != 64 && c.head_dim != 128)) {
+			diag.add_error("RMSNorm GEMM epilogue requires head_dim == sep_dim in {32, 64, 128}"); return false;
+		}
+		if (kv_rows == 0 || kv_rows % (c.head_dim + c.sep_dim) != 0) { diag.add_error("RMSNorm GEMM raw output columns must be whole K|V heads"); return false; }
+		common << "#define X17_HEAD_DIM " << c.head_dim << "\n#define X17_EPS " << format_cpp_f64(c.eps) << "\n";
+		common << "#define X17_HEAD_SCALE " << format_cpp_f64(c.out_scale.value * std::sqrt(double(c.head_dim)))
+		       << " // (" << one_line(c.out_scale.description) << ") * sqrt(" << c.head_dim << ")\n";
+		common << "#define X17_SEP_SCALE " << format_cpp_f64(c.inp_scale.value * c.out_scale.value)
+		       << " // (" << one_line(c.inp_scale.description) << ") * (" << one_line(c.out_scale.description) << ")\n";
+		return true;
+	};
+	if (auto const *c = std::get_if<QNormConfig>(&e)) {
+		if (g.c_dtype != DType::Int8 || g.a.dtype != DType::Int8 || g.b.dtype != DType::Int8) { diag.add_error("QNorm epilogue requires i8 inputs and an i8 output"); return nullptr; }
+		if (!std::isfinite(c->eps) || c->eps < 0.0 || !finite_pos(c->out_scale.value)) { diag.add_error("invalid QNorm epilogue values"); return nullptr; }
+		if (c->head_dim != 32 && c->head_dim != 64 && c->head_dim != 128) { diag.add_error("QNorm GEMM epilogue requires head_dim in {32, 64, 128}"); return nullptr; }
+		if (b_rows % c->head_dim != 0) { diag.add_error("QNorm GEMM raw output columns must be whole heads"); return nullptr; }
+		head_dim = c->head_dim;
+		common << "#define X17_INP_SCALE 1.0\n#define X17_OUT_SCALE " << format_cpp_f64(c->out_scale.value) << "\n";
+		common << "#define X17_HEAD_DIM " << c->head_dim << "\n#define X17_EPS " << format_cpp_f64(c->eps) << "\n";
+		// cuda/qkvg_fwd_i8.cuh:205
+		common << "#define X17_HEAD_SCALE " << format_cpp_f64(c->out_scale.value * std::sqrt(double(c->head_dim)))
+		       << " // (" << one_line(c->out_scale.description) << ") * sqrt(" << c->head_dim << ")\n";
+	} else if (auto const *c = std::get_if<QkvConfig>(&e)) {
+		if (g.c_dtype != DType::Int8 || g.a.dtype != DType::Int8 || g.b.dtype != DType::Int8) { diag.add_error("fused q + kv GEMM requires i8 inputs and i8 outputs"); return nullptr; }
+		if (c->q_cols == 0 || c->q_cols >= b_rows || c->q_cols % 256 != 0) {
+			diag.add_error("fused q + kv GEMM: q_cols must be a multiple of 256 below the raw output column count"); return nullptr;
+		}
+		if (!std::isfinite(c->q.inp_scale.value) || !std::isfinite(c->q.out_scale.value)) { diag.add_error("invalid Scale epilogue scale values"); return nullptr; }
+		common << "#define X17_INP_SCALE " << format_cpp_f64(c->kv.inp_scale.value) << "\n#define X17_OUT_SCALE " << format_cpp_f64(c->kv.out_scale.value) << "\n";
+		common << "#define X17_Q_COLS " << c->q_cols << "\n";
+		common << "#define X17_Q_SCALE (" << format_cpp_f64(c->q.inp_scale.value) << " * " << format_cpp_f64(c->q.out_scale.value) << ")"
+		       << " // (" << one_line(c->q.inp_scale.description) << ") * (" << one_line(c->q.out_scale.description) << ")\n";
+		if (!rmsnorm_defines(c->kv, b_rows - c->q_cols)) return nullptr;
+		head_dim = c->kv.head_dim;
+		sep_dim = c->kv.sep_dim;
+		q_cols = c->q_cols;
+	}
+
 	if (g.a.cols % 128 != 0) { diag.add_error("GEMM K must be a multiple of 128, got " + std::to_string(g.a.cols)); return nullptr; }
 
 	auto built = kernel_build::build(kernel_name, common.str(), "gemm_b8.hip", "gemm_meta.cpp", diag);
@@ -841,6 +884,7 @@ std::unique_ptr<GemmKernel> GemmKernel::create(std::shared_ptr<HipDevice> device
 	out->c_dtype = g.c_dtype;
 	out->head_dim = head_dim;
 	out->sep_dim = sep_dim;
+	out->q_cols = q_cols;
 	if (auto const *c = std::get_if<DequantConfig>(&e)) out->dequant_geglu = c->geglu;
 	if (device) {
 		out->kernel = kernel_build::load_kernel(*device->stream, built->code_object_path, "kernel", out->metadata.SMEM_BYTES, diag);
@@ -862,6 +906,7 @@ Status GemmKernel::launch(GemmArgs const &args) {
 	size_t a_shape[2], b_shape[2], c_shape[2], tmp[2];
 	Status s = tensor_check::matrix_shape(op, "a", *args.a, std::nullopt, a_cols, *device, a_dtype, a_shape);
 	if (!s.is_ok()) return s;
+	if (epilogue_kind == 6) return launch_qkv(args, a_shape[0]);
 	s = tensor_check::matrix_shape(op, "b", *args.b, b_rows, a_cols, *device, b_dtype, b_shape);
 	if (!s.is_ok()) return s;
 	size_t const a_rows = a_shape[0], b_rows_v = b_shape[0];
@@ -892,6 +937,11 @@ Status GemmKernel::launch(GemmArgs const &args) {
 		s = tensor_check::vector_shape(op, "col_scale", *args.extra2, b_rows_v, *device, DType::F32);
 		if (!s.is_ok()) return s;
 	}
+	if (epilogue_kind == 5) {
+		if (args.extra == nullptr) return Status::err(TensorOpError::Other, "QNorm GEMM needs a q_norm_scales tensor");
+		s = tensor_check::vector_shape(op, "q_norm_scales", *args.extra, b_rows_v, *device, DType::Bf16);
+		if (!s.is_ok()) return s;
+	}
 	if (epilogue_kind == 3) {
 		if (args.extra == nullptr) return Status::err(TensorOpError::Other, "RMSNorm GEMM needs an rrms tensor");
 		size_t chunk = head_dim + sep_dim;
@@ -920,6 +970,44 @@ Status GemmKernel::launch(GemmArgs const &args) {
 		grid[0] = metadata.MAX_BLOCKS;
 		grid[1] = 1;
 	}
+	size_t block[3] = {metadata.THREADS_PER_BLOCK, 1, 1};
+	return kernel->launch(*device->stream, grid, block, metadata.SMEM_BYTES, raw_args);
+}
+
+// The fused q + kv launch: the checks of gemm.rs:591-641 for the q part and of :860-918 for the kv part.
+Status GemmKernel::launch_qkv(GemmArgs const &args, size_t a_rows) {
+	char const *op = "fused q + kv GEMM";
+	if (args.b == nullptr || args.c == nullptr || args.b2 == nullptr || args.c2 == nullptr || args.extra == nullptr) {
+		return Status::err(TensorOpError::Other, "fused q + kv GEMM needs x, the q and kv weights, the q and kv outputs and an rrms tensor");
+	}
+	size_t const kv_cols = *b_rows - q_cols;
+	size_t tmp[2];
+	Status s = tensor_check::matrix_shape(op, "q weights", *args.b, q_cols, a_cols, *device, b_dtype, tmp);
+	if (!s.is_ok()) return s;
+	s = tensor_check::matrix_shape(op, "kv weights", *args.b2, kv_cols, a_cols, *device, b_dtype, tmp);
+	if (!s.is_ok()) return s;
+	s = tensor_check::matrix_shape(op, "q", *args.c, a_rows, q_cols, *device, c_dtype, tmp);
+	if (!s.is_ok()) return s;
+	s = tensor_check::matrix_shape(op, "kv", *args.c2, a_rows, kv_cols, *device, c_dtype, tmp);
+	if (!s.is_ok()) return s;
+	s = tensor_check::matrix_shape(op, "rrms", *args.extra, a_rows, kv_cols >> ctz(head_dim + sep_dim), *device, DType::F32, tmp);
+	if (!s.is_ok()) return s;
+	if ((a_rows & (metadata.M_PER_BLOCK - 1)) != 0) {
+		return Status::err(TensorOpError::Other, std::string(op) + " token rows (" + std::to_string(a_rows) + ") must be divisible by the tile height "
+			+ std::to_string(metadata.M_PER_BLOCK));
+	}
+	if (a_rows > 0xFFFFFFFFull) return Status::err(TensorOpError::Other, std::string(op) + " sizes exceed 32 bits (the kernel's row counts are u32)");
+	void *a_ptr = args.a->ptr;
+	size_t a_rows_arg = a_rows;
+	void *b_ptr = args.b->ptr;
+	size_t b_rows_arg = *b_rows;
+	void *c_ptr = args.c->ptr;
+	void *rrms_ptr = args.extra->ptr;
+	void *b2_ptr = args.b2->ptr;
+	void *c2_ptr = args.c2->ptr;
+	void *raw_args[8] = {&a_ptr, &a_rows_arg, &b_ptr, &b_rows_arg, &c_ptr, &rrms_ptr, &b2_ptr, &c2_ptr};
+	size_t tiles = (a_rows >> ctz(metadata.M_PER_BLOCK)) * (*b_rows >> ctz(metadata.N_PER_BLOCK));
+	size_t grid[3] = {metadata.MAX_BLOCKS != 0 && tiles > metadata.MAX_BLOCKS ? metadata.MAX_BLOCKS : tiles, 1, 1};
 	size_t block[3] = {metadata.THREADS_PER_BLOCK, 1, 1};
 	return kernel->launch(*device->stream, grid, block, metadata.SMEM_BYTES, raw_args);
 }
@@ -1397,6 +1485,11 @@ int x17h_gemm_kernel_new(X17hDevice *dev, char const *kernel_name, X17hGemmConfi
 			case X17H_EPI_RESIDUAL: e = ResidualConfig{inp, outs}; break;
 			case X17H_EPI_RMSNORM: e = RMSNormConfig{c->eps, c->head_dim, c->sep_dim, inp, outs}; break;
 			case X17H_EPI_DEQUANT: e = DequantConfig{c->activation == X17H_ACT_GEGLU}; break;
+			case X17H_EPI_QNORM: e = QNormConfig{c->eps, c->head_dim, outs}; break;
+			case X17H_EPI_QKV:
+				e = QkvConfig{c->q_cols, ScaleConfig{Scale{c->q_inp_scale, "q inp_scale"}, Scale{c->q_out_scale, "q out_scale"}},
+				              RMSNormConfig{c->eps, c->head_dim, c->sep_dim, inp, outs}};
+				break;
 			default: return fail("unknown epilogue");
 		}
 		Diagnostics diag;
@@ -1419,6 +1512,14 @@ int x17h_gemm_kernel_launch_dequant(X17hGemmKernel *k, X17hTensor *a, X17hTensor
 		return fail("dequant GEMM launch needs a, b, c, row_scale and col_scale");
 	}
 	GemmArgs args{a->t.get(), b->t.get(), c->t.get(), row_scale->t.get(), col_scale->t.get()};
+	return from_status(k->k->launch(args));
+}
+int x17h_gemm_kernel_launch_qkv(X17hGemmKernel *k, X17hTensor *x, X17hTensor *q_weights, X17hTensor *kv_weights,
+                                X17hTensor *q, X17hTensor *kv, X17hTensor *rrms) {
+	if (x == nullptr || q_weights == nullptr || kv_weights == nullptr || q == nullptr || kv == nullptr || rrms == nullptr) {
+		return fail("fused q + kv GEMM launch needs x, both weight matrices, both outputs and rrms");
+	}
+	GemmArgs args{x->t.get(), q_weights->t.get(), q->t.get(), rrms->t.get(), nullptr, kv_weights->t.get(), kv->t.get()};
 	return from_status(k->k->launch(args));
 }
 double x17h_gemm_kernel_n_ops(X17hGemmKernel *k, X17hTensor *a, X17hTensor *b) { return k->k->n_ops(*a->t, *b->t); }

@@ -195,7 +195,14 @@ struct GeGluConfig { Scale inp_scale, out_scale; };
 // Run-time per-row and per-column dequantisation scales, bf16 output, optional GeGLU over column pairs
 // (no counterpart in gemm.rs: the superset for symmetric per-row / per-channel int8 quantisation).
 struct DequantConfig { bool geglu; };
-using EpilogueConfig = std::variant<ScaleConfig, GeGluConfig, ResidualConfig, RMSNormConfig, DequantConfig>;   // index = X17_EPILOGUE
+// The reference's older Q writer (cuda/qkvg_fwd_i8.cuh:145-219; hook cuda/gemm_b8.cuh:761-824): every head_dim raw
+// columns are one L2-normalised head, multiplied by a learned bf16 scale per column given at launch.
+struct QNormConfig { double eps; size_t head_dim; Scale out_scale; };
+// The q and the kv projection of src/main.rs:387-493 as ONE launch over the same token rows (no counterpart in
+// gemm.rs, which launches them one after the other): raw columns [0, q_cols) come from the q weights and go through
+// the Scale writer `q`, the remaining b.rows - q_cols come from the kv weights and go through the RMSNorm writer `kv`.
+struct QkvConfig { size_t q_cols; ScaleConfig q; RMSNormConfig kv; };
+using EpilogueConfig = std::variant<ScaleConfig, GeGluConfig, ResidualConfig, RMSNormConfig, DequantConfig, QNormConfig, QkvConfig>;   // index = X17_EPILOGUE
 
 struct GemmInputConfig { DType dtype; size_t cols; std::optional<size_t> rows; bool trans; };
 struct GemmConfig { GemmInputConfig a, b; DType c_dtype; };
@@ -205,14 +212,18 @@ struct GemmLauncherMetadata { size_t THREADS_PER_BLOCK, SMEM_BYTES, M_PER_BLOCK,
 
 struct GemmArgs {
 	Tensor const *a; Tensor const *b; Tensor const *c;
-	Tensor const *extra;     // rrms (RMSNorm epilogue), residual (Residual epilogue) or row scales (Dequant), else null
+	Tensor const *extra;     // rrms (RMSNorm, Qkv), residual (Residual), row scales (Dequant), q_norm_scales (QNorm), else null
 	Tensor const *extra2 = nullptr;   // column scales (Dequant epilogue)
+	// Qkv only: a = x, b = q weights, c = q, extra = rrms, and the kv weights and the kv output:
+	Tensor const *b2 = nullptr;
+	Tensor const *c2 = nullptr;
 };
 
 struct GemmKernel {
 	std::string name;
 	kernel_build::BuiltKernel files;
-	int epilogue_kind = 0;                // 0 scale, 1 geglu, 2 residual, 3 rmsnorm
+	int epilogue_kind = 0;                // 0 scale, 1 geglu, 2 residual, 3 rmsnorm, 4 dequant, 5 qnorm, 6 fused q + kv
+	size_t q_cols = 0;                    // fused q + kv: raw columns that belong to q
 	size_t a_cols = 0;
 	std::optional<size_t> b_rows;
 	DType a_dtype, b_dtype, c_dtype;
@@ -227,6 +238,7 @@ struct GemmKernel {
 	                                           GemmConfig const &gemm_config, EpilogueConfig const &epilogue_config,
 	                                           bool strict_math, Diagnostics &diag);
 	Status launch(GemmArgs const &args);
+	Status launch_qkv(GemmArgs const &args, size_t a_rows);   // epilogue_kind 6, reached through launch()
 	double n_ops(Tensor const &a, Tensor const &b) const;     // 2*M*K*N_raw, gemm.rs:445-449
 };
 

@@ -29,10 +29,18 @@
 //
 // common.h (generated per kernel by the host-side kernel builder) provides:
 //   X17_A_COLS (K), X17_B_ROWS (N_raw), X17_A_KIND / X17_B_KIND (0 = int8, 1 = e4m3),
-//   X17_EPILOGUE (0 scale, 1 geglu, 2 residual, 3 l2norm, 4 dequant), X17_STORE (0 FixedI8, 1 e4m3; dequant
-//   always stores bf16), X17_DEQ_GEGLU (dequant only: 0 plain, 1 GeGLU over column pairs),
-//   X17_INP_SCALE, X17_OUT_SCALE, and for l2norm X17_HEAD_DIM, X17_EPS, X17_HEAD_SCALE,
-//   X17_SEP_SCALE (doubles), X17_STRICT_MATH.
+//   X17_EPILOGUE (0 scale, 1 geglu, 2 residual, 3 l2norm, 4 dequant, 5 qnorm, 6 fused q + kv), X17_STORE
+//   (0 FixedI8, 1 e4m3; dequant always stores bf16), X17_DEQ_GEGLU (dequant only: 0 plain, 1 GeGLU over column
+//   pairs), X17_INP_SCALE, X17_OUT_SCALE, for l2norm / qnorm / fused X17_HEAD_DIM, X17_EPS, X17_HEAD_SCALE,
+//   X17_SEP_SCALE (doubles), for fused X17_Q_COLS (the first raw columns belong to q) and X17_Q_SCALE,
+//   X17_STRICT_MATH.
+//
+// Epilogue 5 (qnorm) is the reference's older Q writer with learned scales (cuda/qkvg_fwd_i8.cuh:145-219; the
+// hook is still in the live header: kv_helpers::l2_norm<USE_DYN_SCALE>, cuda/gemm_b8.cuh:761-824): every head_dim
+// raw columns are L2-normalised like the K halves of epilogue 3 and multiplied by a bf16 scale per column.
+// Epilogue 6 computes the q and the kv projection of src/main.rs:387-493 in ONE launch over the same token tiles
+// (raw columns [0, X17_Q_COLS) from the q weights through the Scale writer into q, the rest from the kv weights
+// through the L2-norm writer into kv and rrms): the writer is chosen per output tile, x is read once.
 
 #include "common.h"
 #include "x17_device.h"
@@ -56,6 +64,13 @@ constexpr u32 N_RAW = X17_B_ROWS;
 constexpr int A_KIND = X17_A_KIND;
 constexpr int B_KIND = X17_B_KIND;
 constexpr int STORE = X17_STORE;
+
+// The writers that normalise whole heads (and the fused q + kv kernel, which contains one) keep the weight rows in
+// their natural order: a lane then owns, of every 32-column block, the columns whose (column % 8) / 4 equals
+// lane / 32 -- exactly two of the reference's four partial sums of squares (cuda/gemm_b8.cuh:789-801), so a head's
+// sum needs one exchange between the lanes of a pair whatever its width.  Every other writer takes 64 consecutive
+// columns per lane (pairs and 16-byte output vectors stay inside a lane).
+constexpr bool NATURAL_COLS = X17_EPILOGUE == 3 || X17_EPILOGUE == 5 || X17_EPILOGUE == 6;
 
 // 0: int8 MFMA, 1: fp8 MFMA, 2: f16 MFMA after widening
 constexpr int MMA = (A_KIND == 0 && B_KIND == 0) ? 0 : ((A_KIND == 1 && B_KIND == 1) ? 1 : 2);
@@ -253,11 +268,129 @@ struct DequantEpilogue {
 };
 #endif
 
-// The l2norm epilogue needs more than one lane for head_dim > 64 and is handled in the kernel body.
-#if X17_EPILOGUE == 3
-static_assert(LANE_COLS == 64, "the l2norm writer is written for 128-column waves");
+// ---- writers over the natural column order (l2norm, qnorm and the fused q + kv kernel).
+// For ONE token row a lane holds x[16 * b + r] = raw column 32 * b + 8 * (r / 4) + 4 * (lane / 32) + r % 4 of its
+// wave's 128 columns (b = 32-column block, r = accumulator register).
+#if X17_EPILOGUE == 3 || X17_EPILOGUE == 5 || X17_EPILOGUE == 6
+static_assert(LANE_COLS == 64, "the head-normalising writers are written for 128-column waves");
 constexpr u32 HEAD_DIM = X17_HEAD_DIM;
 static_assert(HEAD_DIM == 32 || HEAD_DIM == 64 || HEAD_DIM == 128, "head_dim must be 32, 64 or 128");
+struct NaturalWriters {
+	static constexpr f32 EPS = f32(f64(X17_EPS));
+	static constexpr f32 HEAD_SCALE = f32(f64(X17_HEAD_SCALE));
+	static constexpr int HB = HEAD_DIM / 32;                    // 32-column blocks per head
+
+	// value of lane ^ 32
+	X17_DEV static f32 partner(f32 v, u32 half) {
+		u32 const u = f2u(v);
+		auto const r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+		return u2f(half == 0 ? r[1] : r[0]);
+	}
+	// The lane pair (lane, lane + 32) holds the 32 output bytes of a block interleaved word by word (word g of a lane
+	// = columns 8 g + 4 half .. + 3); two cross-half swaps give the lower lane bytes 0..15 and the upper lane bytes
+	// 16..31, so that each lane writes one 16-byte vector.
+	X17_DEV static void store_block(u8 *block, u32 const (&w)[4], u32 half) {
+		auto const a = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
+		auto const b = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
+		*reinterpret_cast<v4u *>(block + 16 * half) = v4u{a[0], a[1], b[0], b[1]};
+	}
+	// kv_helpers::l2_norm, cuda/gemm_b8.cuh:767-830: the sum of squares of the head made of blocks [B0, B0 + HB).
+	// The reference's partial sum q owns the columns with (column % 8) / 2 == q in increasing order; the lower lane
+	// of a pair runs the chains of q = 0 and 1, the upper lane those of 2 and 3, total (s0 + s1) + (s2 + s3).
+	template <int B0>
+	X17_DEV static f32 head_scale(f32 const (&x)[64], u32 half) {
+		f32 p0 = 0.0f, p1 = 0.0f;
+		X17_UNROLL for (int b = B0; b < B0 + HB; ++b) {
+			X17_UNROLL for (int g = 0; g < 4; ++g) {
+				p0 = fmaf32(x[16 * b + 4 * g], x[16 * b + 4 * g], p0);
+				p0 = fmaf32(x[16 * b + 4 * g + 1], x[16 * b + 4 * g + 1], p0);
+				p1 = fmaf32(x[16 * b + 4 * g + 2], x[16 * b + 4 * g + 2], p1);
+				p1 = fmaf32(x[16 * b + 4 * g + 3], x[16 * b + 4 * g + 3], p1);
+			}
+		}
+		f32 const mine = p0 + p1;
+		f32 const other = partner(mine, half);
+		f32 const total = half == 0 ? mine + other : other + mine;
+		return strict::rsq(total + EPS) * HEAD_SCALE;
+	}
+	// block b of the row times `scale` (and, with learned scales, times the bf16 scale of each column, in that order:
+	// cuda/gemm_b8.cuh:819-820) -> FixedI8, 16 bytes per lane.  `dst` and `dyn` point at the wave's first column.
+	template <bool DYN>
+	X17_DEV static void emit_block(f32 const (&x)[64], int b, f32 scale, u8 *dst, u16 const *dyn, u32 half) {
+		u32 w[4];
+		X17_UNROLL for (int g = 0; g < 4; ++g) {
+			f32 y[4];
+			X17_UNROLL for (int e = 0; e < 4; ++e) y[e] = x[16 * b + 4 * g + e] * scale;
+			if constexpr (DYN) {
+				v2u const d = *reinterpret_cast<v2u const *>(dyn + 32 * b + 8 * g + 4 * half);
+				y[0] = y[0] * u2f(d[0] << 16);
+				y[1] = y[1] * u2f(d[0] & 0xFFFF0000u);
+				y[2] = y[2] * u2f(d[1] << 16);
+				y[3] = y[3] * u2f(d[1] & 0xFFFF0000u);
+			}
+			w[g] = pack4_fixedi8(y[0], y[1], y[2], y[3]);
+		}
+		store_block(dst + 32 * b, w, half);
+	}
+#if X17_EPILOGUE == 3 || X17_EPILOGUE == 6
+	// L2NormMatrixWriter, cuda/gemm_b8.cuh:861-949: per head the columns are [K (hd) | V (hd)]; K is normalised,
+	// V only scaled, rrms[row, head] = the K scale.  `col0` = the wave's first raw column of the kv matrix.
+	static constexpr f32 SEP_SCALE = f32(f64(X17_SEP_SCALE));
+	X17_DEV static void l2norm_row(f32 const (&x)[64], u8 *c, f32 *rrms, u32 row, u32 col0, u32 kv_cols, u32 half) {
+		u8 *dst = c + (size_t)row * kv_cols + col0;
+		f32 *rr = rrms + (size_t)row * (kv_cols / (2 * HEAD_DIM));
+		if constexpr (HEAD_DIM == 32) {
+			f32 const scale0 = head_scale<0>(x, half);
+			emit_block<false>(x, 0, scale0, dst, nullptr, half);
+			emit_block<false>(x, 1, SEP_SCALE, dst, nullptr, half);
+			f32 const scale1 = head_scale<2>(x, half);
+			emit_block<false>(x, 2, scale1, dst, nullptr, half);
+			emit_block<false>(x, 3, SEP_SCALE, dst, nullptr, half);
+			if (half == 0) {
+				rr[col0 / 64] = scale0;
+				rr[col0 / 64 + 1] = scale1;
+			}
+		} else if constexpr (HEAD_DIM == 64) {
+			f32 const scale = head_scale<0>(x, half);
+			emit_block<false>(x, 0, scale, dst, nullptr, half);
+			emit_block<false>(x, 1, scale, dst, nullptr, half);
+			emit_block<false>(x, 2, SEP_SCALE, dst, nullptr, half);
+			emit_block<false>(x, 3, SEP_SCALE, dst, nullptr, half);
+			if (half == 0) rr[col0 / 128] = scale;
+		} else {
+			// the wave's 128 columns are the K half or the V half of one head
+			if ((col0 / 128) % 2 == 0) {
+				f32 const scale = head_scale<0>(x, half);
+				X17_UNROLL for (int b = 0; b < 4; ++b) emit_block<false>(x, b, scale, dst, nullptr, half);
+				if (half == 0) rr[col0 / 256] = scale;
+			} else {
+				X17_UNROLL for (int b = 0; b < 4; ++b) emit_block<false>(x, b, SEP_SCALE, dst, nullptr, half);
+			}
+		}
+	}
+#endif
+#if X17_EPILOGUE == 5
+	// QMatrixWriter, cuda/qkvg_fwd_i8.cuh:145-219: every head_dim columns are one normalised head
+	template <int B0>
+	X17_DEV static void qnorm_heads(f32 const (&x)[64], u8 *dst, u16 const *dyn, u32 half) {
+		if constexpr (B0 < 4) {
+			f32 const scale = head_scale<B0>(x, half);
+			X17_UNROLL for (int b = B0; b < B0 + HB; ++b) emit_block<true>(x, b, scale, dst, dyn, half);
+			qnorm_heads<B0 + HB>(x, dst, dyn, half);
+		}
+	}
+	X17_DEV static void qnorm_row(f32 const (&x)[64], u8 *c, u16 const *dyn, u32 row, u32 col0, u32 half) {
+		qnorm_heads<0>(x, c + (size_t)row * N_RAW + col0, dyn + col0, half);
+	}
+#endif
+#if X17_EPILOGUE == 6
+	// ScaledMatrixWriter (cuda/gemm_b8.cuh:291-339) over the natural column order, for the q columns
+	X17_DEV static void scale_row(f32 const (&x)[64], u8 *c, u32 row, u32 col0, u32 q_cols, u32 half) {
+		u8 *dst = c + (size_t)row * q_cols + col0;
+		X17_UNROLL for (int b = 0; b < 4; ++b) emit_block<false>(x, b, f32(f64(X17_Q_SCALE)), dst, nullptr, half);
+	}
+#endif
+};
 #endif
 
 // ------------------------------------------------------------------ tile loads
@@ -287,6 +420,9 @@ constexpr bool LANE_UNIT_OFFSETS = gt::WAVES_PER_SIMD == 1;
 constexpr u32 X_OFFSETS = LANE_UNIT_OFFSETS ? X_UNITS : 2;
 constexpr u32 W_OFFSETS = LANE_UNIT_OFFSETS ? W_UNITS : 2;
 X17_DEV constexpr u32 w_unit_row(u32 r0) {   // weight row that LDS weight row r0 (a multiple of the unit) starts from
+	if (NATURAL_COLS) {
+		return r0;
+	}
 	return gt::WAVE_N * (r0 / gt::WAVE_N) + 16 * ((r0 % gt::WAVE_N) / 32) + 4 * ((r0 % 32) / 8);
 }
 struct LaneOffsets {
@@ -661,6 +797,11 @@ void kernel(
 	, i8 const *residual
 #elif X17_EPILOGUE == 4
 	, f32 const *row_scale, f32 const *col_scale
+#elif X17_EPILOGUE == 5
+	, u16 const *q_norm_scales          // bf16 [N_raw]
+#elif X17_EPILOGUE == 6
+	// a, b = q weights [X17_Q_COLS, K], c = q [M, X17_Q_COLS]; then:
+	, f32 *rrms, u8 const *b_kv /* [N_raw - X17_Q_COLS, K] */, u8 *c_kv /* [M, N_raw - X17_Q_COLS] */
 #endif
 ) {
 	extern __shared__ __attribute__((aligned(1024))) u8 smem[];
@@ -710,7 +851,7 @@ void kernel(
 			u32 key = ((odd * UNIT_ROWS + j) >> SWZ_SHIFT) & (CHUNKS - 1);
 			u32 chunk = p ^ key;
 			even_odd_x[odd] = j * K_TOTAL + 16 * chunk;
-			even_odd_w[odd] = ((gt::WAVE_N / 2) * ((j >> 2) & 1) + 4 * (j >> 3) + (j & 3)) * K_TOTAL + 16 * chunk;
+			even_odd_w[odd] = (NATURAL_COLS ? j : (gt::WAVE_N / 2) * ((j >> 2) & 1) + 4 * (j >> 3) + (j & 3)) * K_TOTAL + 16 * chunk;
 		}
 		if constexpr (LANE_UNIT_OFFSETS) {
 			u32 const w_first = wave * W_UNITS * UNIT_ROWS;
@@ -749,10 +890,19 @@ void kernel(
 	u32 const x_off = wm * gt::WAVE_M * ROW_BYTES + lo.frag_row;
 	u32 const w_off = W_RING_OFFSET + wn * gt::WAVE_N * ROW_BYTES + lo.frag_row;
 
+	// the weight rows of column tile t: one matrix, or (fused q + kv) the q weights followed by the kv weights
+	auto weight_tile = [&](u32 t) -> u8 const * {
+#if X17_EPILOGUE == 6
+		constexpr u32 Q_TILES = X17_Q_COLS / gt::N_PER_BLOCK;
+		return t < Q_TILES ? b + (size_t)(t * gt::N_PER_BLOCK) * K_TOTAL : b_kv + (size_t)((t - Q_TILES) * gt::N_PER_BLOCK) * K_TOTAL;
+#else
+		return b + (size_t)(t * gt::N_PER_BLOCK) * K_TOTAL;
+#endif
+	};
 	u32 tile_m, tile_n;
 	tile_coords(group, tile_m, tile_n);
 	u8 const *a_tile = a + (size_t)(tile_m * gt::M_PER_BLOCK) * K_TOTAL;
-	u8 const *b_tile = b + (size_t)(tile_n * gt::N_PER_BLOCK) * K_TOTAL;
+	u8 const *b_tile = weight_tile(tile_n);
 	// the first steps of a tile nobody prefetched, in the order the waits of the main loop assume
 	// (token tile s, weight tile s, ..., then the extra token tile of a deeper token ring)
 	auto prologue = [&]() __attribute__((always_inline)) {
@@ -780,7 +930,7 @@ void kernel(
 			tile_coords(lin + n_groups, next_m, next_n);
 		}
 		u8 const *a_next = a + (size_t)(next_m * gt::M_PER_BLOCK) * K_TOTAL;
-		u8 const *b_next = b + (size_t)(next_n * gt::N_PER_BLOCK) * K_TOTAL;
+		u8 const *b_next = weight_tile(next_n);
 		if constexpr (!CROSS_TILE) {
 			if (!first_tile) {
 				__builtin_amdgcn_s_waitcnt(0xC07F);        // lgkmcnt(0)
@@ -981,76 +1131,18 @@ void kernel(
 		ResidualEpilogue::run(x, c, row, n0, residual);
 #elif X17_EPILOGUE == 4
 		DequantEpilogue::run(x, c, row, n0, row_scale, col_scale);
+#elif X17_EPILOGUE == 3
+		NaturalWriters::l2norm_row(x, c, rrms, row, tile_n * gt::N_PER_BLOCK + wn * gt::WAVE_N, N_RAW, lo.half);
+#elif X17_EPILOGUE == 5
+		NaturalWriters::qnorm_row(x, c, q_norm_scales, row, tile_n * gt::N_PER_BLOCK + wn * gt::WAVE_N, lo.half);
 #else
-		// L2NormMatrixWriter, cuda/gemm_b8.cuh:861-949 with kv_helpers::l2_norm :767-830.
-		// Per head the columns are [K (hd) | V (hd)].  Sum of squares of the K half: four partial
-		// sums, partial q owns columns with (col % 8) / 2 == q in increasing column order, total
-		// (s0+s1)+(s2+s3).  A lane holds 64 consecutive columns, so a 128-wide K half is summed by
-		// the lower-half lane first and continued by lane+32.
-		constexpr f32 EPS = f32(f64(X17_EPS));
-		constexpr f32 HEAD_SCALE = f32(f64(X17_HEAD_SCALE));
-		constexpr f32 SEP_SCALE = f32(f64(X17_SEP_SCALE));
-		constexpr u32 HEADS_TOTAL = N_RAW / (2 * HEAD_DIM);
-		u8 *dst = c + (size_t)row * N_RAW + n0;
-		auto sumsq = [&](int first, int count, f32 (&s)[4]) {
-			X17_UNROLL for (int d = 0; d < count; ++d) {
-				int q = (d % 8) / 2;
-				s[q] = fmaf32(x[first + d], x[first + d], s[q]);
-			}
-		};
-		auto emit = [&](int first, int count, f32 scale, bool dyn) {
-			(void)dyn;
-			X17_UNROLL for (int v = 0; v < count / 16; ++v) {
-				v4u pack;
-				X17_UNROLL for (int w = 0; w < 4; ++w) {
-					int d = first + 16 * v + 4 * w;
-					pack[w] = pack4_fixedi8(x[d] * scale, x[d + 1] * scale, x[d + 2] * scale, x[d + 3] * scale);
-				}
-				*reinterpret_cast<v4u *>(dst + first + 16 * v) = pack;
-			}
-		};
-		if constexpr (HEAD_DIM == 32) {
-			// a lane holds one whole head: K = x[0..32), V = x[32..64)
-			f32 s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-			sumsq(0, 32, s);
-			f32 scale = strict::rsq(((s[0] + s[1]) + (s[2] + s[3])) + EPS) * HEAD_SCALE;
-			emit(0, 32, scale, true);
-			emit(32, 32, SEP_SCALE, false);
-			rrms[(size_t)row * HEADS_TOTAL + n0 / 64] = scale;
-		} else if constexpr (HEAD_DIM == 64) {
-			// lower-half lanes hold K, upper-half lanes hold V of the same head
-			f32 s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-			sumsq(0, 64, s);
-			f32 scale = strict::rsq(((s[0] + s[1]) + (s[2] + s[3])) + EPS) * HEAD_SCALE;
-			if (lo.half == 0) {
-				emit(0, 64, scale, true);
-				rrms[(size_t)row * HEADS_TOTAL + n0 / 128] = scale;
+		{
+			constexpr u32 Q_COLS = X17_Q_COLS;
+			u32 const col0 = tile_n * gt::N_PER_BLOCK + wn * gt::WAVE_N;
+			if (col0 < Q_COLS) {
+				NaturalWriters::scale_row(x, c, row, col0, Q_COLS, lo.half);
 			} else {
-				emit(0, 64, SEP_SCALE, false);
-			}
-		} else {
-			// a wave's 128 columns are the K half (even wn) or the V half (odd wn) of one head
-			f32 s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-			if (wn % 2 == 0) {
-				f32 t[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-				sumsq(0, 64, t);                                   // columns 0..63 (valid in lower lanes)
-				X17_UNROLL for (int q = 0; q < 4; ++q) {
-					f32 from_low = __shfl(t[q], lane % 32, 64);     // lower lane's partial sums
-					s[q] = lo.half == 0 ? 0.0f : from_low;
-				}
-				if (lo.half != 0) {
-					sumsq(0, 64, s);                               // continue with columns 64..127
-				}
-				X17_UNROLL for (int q = 0; q < 4; ++q) {
-					s[q] = __shfl(s[q], 32 + lane % 32, 64);       // the finished sums live in the upper lanes
-				}
-				f32 scale = strict::rsq(((s[0] + s[1]) + (s[2] + s[3])) + EPS) * HEAD_SCALE;
-				emit(0, 64, scale, true);
-				if (lo.half == 0) {
-					rrms[(size_t)row * HEADS_TOTAL + (tile_n * gt::N_PER_BLOCK + wn * 128) / 256] = scale;
-				}
-			} else {
-				emit(0, 64, SEP_SCALE, false);
+				NaturalWriters::l2norm_row(x, c_kv, rrms, row, col0 - Q_COLS, N_RAW - Q_COLS, lo.half);
 			}
 		}
 #endif

@@ -38,6 +38,12 @@ def _specs():
 		add(("ffn_y", n // 2, k, True, E4M3, INT8))
 	for k, n in ((512, 256), (4096, 512)):
 		add(("ffn_f_f8", k, n, True))
+	for hd in (32, 64, 128):             # learned-scale Q writer; fused q + kv
+		add(("attn_q_norm", 512, 512, hd, 0.0))
+		add(("attn_qkv", 512, 256, 512, hd, True))
+	add(("attn_q_norm", 2048, 1024, 128, recipes.L2_NORM_EPS))
+	for hd in (64, 128):                 # L2-norm writer on a walk of more tiles than workgroups
+		add(("attn_kv", 256, 2048, hd))
 	add(("attn_q", 384, 1024))           # the shortest K with the deeper token ring, more tiles than workgroups
 	add(("ffn_f_f8", 384, 512, True))
 	# ---- tests/test_gpu_attn.py
@@ -104,6 +110,7 @@ def _specs():
 	# ---- x17ai_amd.block: benchmark config 4 (bench.py, tests/config4_chain.py) and the reference's own configuration
 	for strict in (True, False):
 		add(("block", 2048, 16, 128, 8192, BF16, strict))
+		add(("attn_qkv", 2048, 2048, 4096, 128, strict))
 	add(("block", 2048, 64, 32, 2048, None, True))
 	add(("block", 512, 8, 32, 256, None, True))          # tests/test_gpu_files.py
 	add(("attn_q", 128, 256))
@@ -118,6 +125,10 @@ def _build_one(spec) -> str:
 		return f"block-d{spec[1]}-h{spec[2]}x{spec[3]}-f{spec[4]}-{'strict' if spec[6] else 'fast'}"
 	if kind == "attn_q":
 		return recipes.attn_q_kernel(None, spec[1], spec[2]).name
+	if kind == "attn_q_norm":
+		return recipes.attn_q_norm_kernel(None, spec[1], spec[2], spec[3], spec[4]).name
+	if kind == "attn_qkv":
+		return recipes.attn_qkv_kernel(None, spec[1], spec[2], spec[3], spec[4], spec[5]).name
 	if kind == "ffn_f":
 		return recipes.ffn_f_kernel(None, spec[1], spec[2], spec[3], spec[4]).name
 	if kind == "attn_y":

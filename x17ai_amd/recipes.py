@@ -12,7 +12,7 @@ from typing import Optional
 from .api import (
 	BF16, E4M3, INT8,
 	AttnDecodeKernel, AttnKernel, AttnKernelConfig, Device, DequantConfig, GeGluConfig, GemmConfig, GemmInputConfig, GemmKernel,
-	ResidualConfig, RMSNormConfig, RmsNormKernel, ScaleConfig,
+	QkvConfig, QNormConfig, ResidualConfig, RMSNormConfig, RmsNormKernel, ScaleConfig,
 )
 
 FIXED_I8_SCALE = 8.0                     # src/main.rs:33
@@ -47,6 +47,29 @@ def attn_kv_kernel(device: Optional[Device], model_dim: int, kv_proj_outputs: in
 	                    _inv_sqrt(model_dim) / (FIXED_I8_SCALE * FIXED_I8_SCALE), FIXED_I8_SCALE)
 	return GemmKernel(device, f"attn_kv_fwd-k{model_dim}-n{kv_proj_outputs}-hd{head_dim}-{_mode(strict)}",
 	                  _gemm(INT8, INT8, INT8, model_dim, kv_proj_outputs), cfg, strict)
+
+
+def attn_qkv_kernel(device: Optional[Device], model_dim: int, q_proj_outputs: int, kv_proj_outputs: int, head_dim: int,
+                    strict: bool = True) -> GemmKernel:
+	"""attn_q_kernel and attn_kv_kernel (src/main.rs:387-493) as one launch that reads x once: the first
+	q_proj_outputs raw columns go through the Scale writer into q, the rest through the L2-norm writer into kv and
+	rrms.  Launch with GemmKernel.launch_qkv; the outputs equal those of the two kernels bit for bit."""
+	inp = _inv_sqrt(model_dim) / (FIXED_I8_SCALE * FIXED_I8_SCALE)
+	cfg = QkvConfig(q_proj_outputs, ScaleConfig(inp, FIXED_I8_SCALE),
+	                RMSNormConfig(L2_NORM_EPS, head_dim, head_dim, inp, FIXED_I8_SCALE))
+	return GemmKernel(device, f"attn_qkv_fwd-k{model_dim}-q{q_proj_outputs}-kv{kv_proj_outputs}-hd{head_dim}-{_mode(strict)}",
+	                  _gemm(INT8, INT8, INT8, model_dim, q_proj_outputs + kv_proj_outputs), cfg, strict)
+
+
+def attn_q_norm_kernel(device: Optional[Device], model_dim: int, q_proj_outputs: int, head_dim: int,
+                       eps: float = 0.0, strict: bool = True) -> GemmKernel:
+	"""The reference's older Q projection with learned scales (attn_q_fwd_i8.cu:30-34 loads q_norm_scales.bin for
+	it; writer cuda/qkvg_fwd_i8.cuh:145-219): x[i8] . Wq[i8]^T, every head L2-normalised to sqrt(head_dim) * 8 and
+	multiplied by a bf16 scale per column (launch(x, wq, q, q_norm_scales)).  eps = 0 is the old writer; the hook
+	that survives in cuda/gemm_b8.cuh:761-824 adds L2_NORM_EPS."""
+	cfg = QNormConfig(eps, head_dim, FIXED_I8_SCALE)
+	return GemmKernel(device, f"attn_q_norm_fwd-k{model_dim}-n{q_proj_outputs}-hd{head_dim}-{_mode(strict)}",
+	                  _gemm(INT8, INT8, INT8, model_dim, q_proj_outputs), cfg, strict)
 
 
 def attn_kernel(device: Optional[Device], n_heads: int, head_dim: int, strict: bool = True) -> AttnKernel:
