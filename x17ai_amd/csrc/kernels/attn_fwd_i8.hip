@@ -78,7 +78,7 @@ static_assert(N_HEADS % HPK == 0, "n_heads must be divisible by heads_per_kernel
 
 constexpr f32 PROB_SCALE = 255.0f;                                  // cuda/attn_fwd_i8.cuh:206
 constexpr f32 LOG2_PROB_SCALE = 7.9943534368588578f;                // lg2(255)
-constexpr f32 MAX_LIFT = 64.0f;                                     // 255 * 64 stays far inside f16
+constexpr f32 MAX_LIFT = 32.0f;                                     // (1024 + 255) * 32 stays inside f16
 constexpr f32 BASE_TEMPERATURE = ROW_SCALES ? f32(constexpr_inv_sqrt(f64(HD)))
                                             : f32(constexpr_inv_sqrt(f64(HD)) / 64.0);   // :47, :447-449
 
@@ -118,6 +118,19 @@ X17_DEV u32 pack_f16(f32 lo, f32 hi) {
 	// both values are integers below 2048: exact in f16 whatever the rounding mode
 	return __builtin_bit_cast(u32, __builtin_amdgcn_cvt_pkrtz(lo, hi));
 }
+
+// One 16-byte-per-lane direct-to-LDS load: LDS destination in M0 (wave-uniform; lane l lands 16 * l bytes further),
+// global source = a uniform 64-bit base in scalar registers + a 32-bit offset per lane (the compiler's own selection
+// forms a 64-bit address per lane with a 64-bit vector add in front of every load).
+X17_DEV void load_to_lds_16(u8 *lds_uniform, i8 const *src_uniform, u32 lane_offset) {
+	asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+	             :: "s"((u32)(size_t)X17_LDS_PTR(lds_uniform)), "v"(lane_offset), "s"(src_uniform) : "memory", "m0");
+}
+
+// Speed build: p + PACK_MAGIC rounds p in [0, 256) to the nearest integer P (ties to even, as rintf) and leaves
+// the f16 bit pattern of 1024 + P in the low half of the sum: 12582912 = 1.5 * 2^23 has an ulp of 1 and the bits
+// 0x4B400000; adding 0x6400 = 25600 puts the f16 exponent of 1024 above the eight integer bits.
+constexpr f32 PACK_MAGIC = 12582912.0f + 25600.0f;
 
 } // namespace
 
@@ -191,7 +204,7 @@ void kernel(
 			stage_v_src = (tid / CPR) * KV_STRIDE + HD + (tid % CPR) * 16;
 			widen_dst = v_granule_offset(tid / CPR, tid % CPR);
 		}
-		u32 const stage_lds = (tid / 64) * 1024;          // wave-uniform part of the direct-to-LDS address
+		u32 const stage_lds = wave * 1024;                // wave-uniform part of the direct-to-LDS address
 		auto issue_kv_load = [&](u32 kb, u32 slot) {
 			if (stager) {
 				i8 const *src = kv_head + (size_t)(kb * at::KV_PER_STEP) * KV_STRIDE;
@@ -295,8 +308,163 @@ void kernel(
 		}
 #endif
 
-		// ---- pipeline prologue
 		u32 const n_steps = kb_end - kb_begin;
+		bool handled = false;
+		if constexpr (!STRICT && !ROW_SCALES) {
+		if (positive_temperature) {
+			// ---- speed build, positive temperature.  The same recurrence with the bookkeeping taken out of the key
+			// loop: a wave's steps fall into runs -- nothing to do, masked (the window's edge), fully visible, the
+			// diagonal, nothing to do -- and each run is its own loop; every step requests a tile (past the end the last
+			// one again, into a slot nobody reads any more), so the waits are constants; the tile requests take a
+			// scalar base and a lane offset; the 8-bit probabilities are rounded and turned into f16 by one addition
+			// and one byte shuffle per pair (PACK_MAGIC), the lift and the removal of the 1024 are one packed fma; the
+			// partial sums are kept at the scale of O (the maximum m_ref), so a moving maximum costs one exponential.
+			handled = true;
+			v2h neg_bias2 = {(_Float16)-1024.0f, (_Float16)-1024.0f};      // -1024 * lift2
+			u32 const first_active = wave_kb_first - kb_begin;
+			u32 const diagonal = wave_kb_last - kb_begin;
+			// first block that lies inside the window of all 32 queries: q_wave0 + 31 - 32 kb <= wr
+			u32 const inside_kb = q_wave0 + 31 > wr ? (q_wave0 + 62 - wr) / 32 : 0;
+			u32 const inside_clamped = inside_kb < wave_kb_first ? wave_kb_first : (inside_kb > wave_kb_last ? wave_kb_last : inside_kb);
+			u32 const first_full = inside_clamped - kb_begin;
+
+			i8 const *load_src = kv_head + (size_t)(kb_begin * at::KV_PER_STEP) * KV_STRIDE;
+			u32 next_step = 0;
+			auto request_tiles = [&]() {
+				u32 const slot = next_step % at::RING;
+				if (CPR == 8 || stager) {
+					load_to_lds_16(smem + at::K_RING_OFFSET + slot * at::K_TILE_BYTES + stage_lds, load_src, stage_k_src);
+					load_to_lds_16(smem + at::RAW_V_RING_OFFSET + slot * at::RAW_V_TILE_BYTES + stage_lds, load_src, stage_v_src);
+				}
+				++next_step;
+				if (next_step < n_steps) {
+					load_src += (size_t)at::KV_PER_STEP * KV_STRIDE;
+				}
+			};
+			// K tile i and raw V tile i + 1 have landed once at most the two requests of step i + 2 are in flight
+			auto stage = [&](u32 i) {
+				__builtin_amdgcn_s_waitcnt(0x0F72);          // vmcnt(2)
+				__builtin_amdgcn_s_waitcnt(0xC07F);          // lgkmcnt(0): own LDS traffic of step i-1 is complete
+				__builtin_amdgcn_s_barrier();                // ... and so is everybody else's: tiles i are visible
+				request_tiles();                             // step i + 3 into the slot step i - 1 used
+			};
+			auto widen_next = [&](u32 i) { widen_v((i + 1) % at::RING, (i + 1) & 1); };
+			// maximum of a lane pair's two values, in both lanes
+			auto pair_max_i32 = [](i32 x) {
+				auto const r = __builtin_amdgcn_permlane32_swap((u32)x, (u32)x, false, false);
+				return (i32)r[0] > (i32)r[1] ? (i32)r[0] : (i32)r[1];
+			};
+
+			auto compute = [&]<bool MASKED>(u32 i) __attribute__((always_inline)) {
+				u32 const kb = kb_begin + i;
+				u8 const *k_tile = smem + at::K_RING_OFFSET + (i % at::RING) * at::K_TILE_BYTES;
+				u8 const *v_tile = smem + at::V_TILES_OFFSET + (i & 1) * at::V_TILE_BYTES;
+				v16i s_acc = {0};
+				X17_UNROLL for (u32 sl = 0; sl < K_SLICES; ++sl) {
+					v4i kf = *reinterpret_cast<v4i const *>(k_tile + k_chunk_offset(qlane, 2 * sl + half));
+					s_acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[sl], s_acc, 0, 0, 0);
+				}
+				widen_next(i);                                // (behind the matrix instructions, whose results are not ready yet)
+				u32 const key0 = kb * at::KV_PER_STEP;
+				X17_UNROLL for (u32 tile = 0; tile < 2; ++tile) {
+					f32 sc[8];
+					f32 tmax;
+					if constexpr (!MASKED) {
+						// the row maximum over the integer dots (the scaling is monotone), scaled once
+						i32 const *a = reinterpret_cast<i32 const *>(&s_acc) + 8 * tile;
+						auto mx = [](i32 x, i32 y) { return x > y ? x : y; };
+						i32 const imax = mx(mx(mx(a[0], a[1]), mx(a[2], a[3])), mx(mx(a[4], a[5]), mx(a[6], a[7])));
+						tmax = f32(pair_max_i32(imax)) * temperature;
+					} else {
+						X17_UNROLL for (u32 r = 0; r < 8; ++r) sc[r] = f32(s_acc[8 * tile + r]) * temperature;
+						u32 const first = qi - 1 - (key0 + 16 * tile + 4 * half);
+						X17_UNROLL for (u32 r = 0; r < 8; ++r) {
+							u32 const distance = first - (8 * (r / 4) + (r % 4));
+							sc[r] = distance <= vis_bound ? sc[r] : -__builtin_inff();
+						}
+						f32 const lmax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fmaxf(sc[0], sc[1]), __builtin_fmaxf(sc[2], sc[3])),
+						                                 __builtin_fmaxf(__builtin_fmaxf(sc[4], sc[5]), __builtin_fmaxf(sc[6], sc[7])));
+						tmax = __builtin_fmaxf(lmax, partner_f32(lmax, half));
+					}
+					if (__any(tmax > m)) {
+						m = tmax > m ? tmax : m;
+						lift = hw::ex2(m - m_ref);
+						if (__any(lift > MAX_LIFT)) {
+							// O and the partial sums come down to the scale of the new maximum
+							f32 const down = hw::rcp(lift);
+							X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
+								X17_UNROLL for (int r = 0; r < 16; ++r) o_acc[db][r] = o_acc[db][r] * down;
+							}
+							sum_lo = sum_lo * down;
+							sum_hi = sum_hi * down;
+							m_ref = m;
+							lift = 1.0f;
+						}
+						lift2 = v2h{(_Float16)lift, (_Float16)lift};      // round to nearest
+						neg_bias2 = lift2 * v2h{(_Float16)-1024.0f, (_Float16)-1024.0f};     // exact
+					}
+					f32 const shift = m - LOG2_PROB_SCALE;        // 255 * 2^(s - m) = 2^(s - (m - lg2 255))
+					f32 p[8];
+					if constexpr (!MASKED) {
+						X17_UNROLL for (u32 r = 0; r < 8; ++r) p[r] = hw::ex2(fmaf32(f32(s_acc[8 * tile + r]), temperature, -shift));
+					} else {
+						X17_UNROLL for (u32 r = 0; r < 8; ++r) p[r] = hw::ex2(sc[r] - shift);
+					}
+					sum_lo = fmaf32((p[0] + p[1]) + (p[2] + p[3]), lift, sum_lo);
+					sum_hi = fmaf32((p[4] + p[5]) + (p[6] + p[7]), lift, sum_hi);
+					v4u pp;
+					X17_UNROLL for (int w = 0; w < 4; ++w) {
+						u32 const lo16 = f2u(p[2 * w] + PACK_MAGIC), hi16 = f2u(p[2 * w + 1] + PACK_MAGIC);
+						u32 const pair = __builtin_amdgcn_perm(hi16, lo16, 0x05040100u);           // f16 (1024 + P) twice
+						pp[w] = __builtin_bit_cast(u32, __builtin_elementwise_fma(__builtin_bit_cast(v2h, pair), lift2, neg_bias2));
+					}
+					v8h const pfrag = __builtin_bit_cast(v8h, pp);
+					X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
+						u32 const t = lane % 16;
+						u32 const dh = (lane / 16) % 2;
+						u32 const key = 16 * tile + 4 * half + (t >> 2);
+						u8 const *p0 = v_tile + v_granule_offset(key, 2 * db + dh) + 8 * (t & 3);
+						u8 const *p1 = v_tile + v_granule_offset(key + 8, 2 * db + dh) + 8 * (t & 3);
+						v4s const lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3))) *)p0);
+						v4s const hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3))) *)p1);
+						typedef short v8s __attribute__((ext_vector_type(8)));
+						v8s const both = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+						o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, both), pfrag, o_acc[db], 0, 0, 0);
+					}
+				}
+			};
+
+			__syncthreads();                      // previous head's tiles are no longer read
+			X17_UNROLL for (u32 j = 0; j < at::PREFETCH; ++j) request_tiles();
+			__builtin_amdgcn_s_waitcnt(0x0F74);   // vmcnt(4): step 0 has landed
+			widen_v(0, 0);
+			u32 i = 0;
+			for (; i < first_active; ++i) {
+				stage(i);
+				widen_next(i);
+			}
+			for (; i < first_full; ++i) {
+				stage(i);
+				compute.template operator()<true>(i);
+			}
+			for (; i < diagonal; ++i) {
+				stage(i);
+				compute.template operator()<false>(i);
+			}
+			stage(i);
+			compute.template operator()<true>(i);
+			for (++i; i < n_steps; ++i) {
+				stage(i);
+				widen_next(i);
+			}
+			__builtin_amdgcn_s_waitcnt(0x0F70);   // the last requests write LDS: they land before the tiles are reused
+			// the partial sums are at the scale of m_ref: the common ending below takes them as if that were the maximum
+			m = m_ref;
+			lift = 1.0f;
+		}
+		}
+		if (!handled) {
+		// ---- pipeline prologue
 		__syncthreads();                      // previous head's tiles are no longer read
 		X17_UNROLL for (u32 j = 0; j < at::PREFETCH; ++j) {
 			if (j < n_steps) issue_kv_load(kb_begin + j, j);
@@ -470,6 +638,7 @@ void kernel(
 				}
 			}
 
+		}
 		}
 
 		// ---- finish (cuda/attn_fwd_i8.cuh:293-351): the lane pair holds partial sums (s0, s2) and (s1, s3)
