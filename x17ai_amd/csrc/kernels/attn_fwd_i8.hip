@@ -309,24 +309,23 @@ void kernel(
 #endif
 
 		u32 const n_steps = kb_end - kb_begin;
-		bool handled = false;
 		if constexpr (!STRICT && !ROW_SCALES) {
-		if (positive_temperature) {
-			// ---- speed build, positive temperature.  The same recurrence with the bookkeeping taken out of the key
+			// ---- speed build.  The same recurrence with the bookkeeping taken out of the key
 			// loop: a wave's steps fall into runs -- nothing to do, masked (the window's edge), fully visible, the
 			// diagonal, nothing to do -- and each run is its own loop; every step requests a tile (past the end the last
 			// one again, into a slot nobody reads any more), so the waits are constants; the tile requests take a
 			// scalar base and a lane offset; the 8-bit probabilities are rounded and turned into f16 by one addition
 			// and one byte shuffle per pair (PACK_MAGIC), the lift and the removal of the 1024 are one packed fma; the
 			// partial sums are kept at the scale of O (the maximum m_ref), so a moving maximum costs one exponential.
-			handled = true;
 			v2h neg_bias2 = {(_Float16)-1024.0f, (_Float16)-1024.0f};      // -1024 * lift2
 			u32 const first_active = wave_kb_first - kb_begin;
 			u32 const diagonal = wave_kb_last - kb_begin;
 			// first block that lies inside the window of all 32 queries: q_wave0 + 31 - 32 kb <= wr
 			u32 const inside_kb = q_wave0 + 31 > wr ? (q_wave0 + 62 - wr) / 32 : 0;
 			u32 const inside_clamped = inside_kb < wave_kb_first ? wave_kb_first : (inside_kb > wave_kb_last ? wave_kb_last : inside_kb);
-			u32 const first_full = inside_clamped - kb_begin;
+			// (the fully visible steps take the row maximum over the integer dots, which needs a positive temperature;
+			// with any other temperature every step goes the way of the masked ones, which compare the scaled scores)
+			u32 const first_full = (positive_temperature ? inside_clamped : wave_kb_last) - kb_begin;
 
 			i8 const *load_src = kv_head + (size_t)(kb_begin * at::KV_PER_STEP) * KV_STRIDE;
 			u32 next_step = 0;
@@ -461,9 +460,7 @@ void kernel(
 			// the partial sums are at the scale of m_ref: the common ending below takes them as if that were the maximum
 			m = m_ref;
 			lift = 1.0f;
-		}
-		}
-		if (!handled) {
+		} else {
 		// ---- pipeline prologue
 		__syncthreads();                      // previous head's tiles are no longer read
 		X17_UNROLL for (u32 j = 0; j < at::PREFETCH; ++j) {

@@ -28,7 +28,7 @@ constexpr unsigned RING = PREFETCH + 1;
 // Register budget: this many wavefronts (= workgroups) share a SIMD, so that one workgroup's waits for
 // its K/V tiles and its barrier are covered by the others' arithmetic.
 #ifndef X17_ATTN_WAVES_PER_SIMD
-#define X17_ATTN_WAVES_PER_SIMD 2
+#define X17_ATTN_WAVES_PER_SIMD (X17_STRICT_MATH ? 2 : 3)   // the deterministic transcendentals need more registers
 #endif
 constexpr unsigned WAVES_PER_SIMD = X17_ATTN_WAVES_PER_SIMD;
 
