@@ -163,15 +163,30 @@ void kernel(
 	u32 const half = lane / 32;
 	u32 const qlane = lane % 32;
 
-	u32 const seq = blockIdx.z;
-	size_t const row_base = (size_t)seq * seq_len;          // first row of this sequence
-	// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  When the number of query
-	// blocks is a multiple of 8, XCD k gets a contiguous eighth of the sequence, so that the query blocks
-	// resident on one XCD at a time are neighbours and share their K/V windows in its L2.
+	// Which (sequence, head group, query block) this workgroup takes.  The hardware starts workgroups in the order of
+	// their linear index and deals them round-robin to the 8 XCDs (each with its own L2).  When the (sequence, head
+	// group) pairs divide evenly among the XCDs, each XCD walks its pairs one after the other and the query blocks of
+	// a pair from the last to the first: the workgroups resident on an XCD at one time are neighbouring blocks of one
+	// or two heads, whose key/value windows overlap and stay in its L2, and the blocks with the shortest windows (the
+	// first of each sequence) run last, where they fill the tail of the launch.
+	u32 seq = blockIdx.z;
+	u32 head_group = blockIdx.y;
 	u32 q_block_index = blockIdx.x;
-	if (gridDim.x % 8 == 0) {
-		q_block_index = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
+	{
+		u32 const pairs = gridDim.y * gridDim.z;
+		if (pairs % 8 == 0) {
+			u32 const lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+			u32 const xcd = lin % 8, j = lin / 8;
+			u32 const pair = xcd * (pairs / 8) + j / gridDim.x;
+			q_block_index = gridDim.x - 1 - j % gridDim.x;
+			head_group = pair % gridDim.y;
+			seq = pair / gridDim.y;
+		} else if (gridDim.x % 8 == 0) {
+			// otherwise XCD k gets a contiguous eighth of every sequence
+			q_block_index = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
+		}
 	}
+	size_t const row_base = (size_t)seq * seq_len;          // first row of this sequence
 	u32 const q_block0 = q_block_index * at::Q_PER_BLOCK;   // position of the block's first query
 	u32 const q_wave0 = q_block0 + wave * at::Q_PER_WAVE;
 	u32 const qi = q_wave0 + qlane;                         // this lane's query position
@@ -187,7 +202,7 @@ void kernel(
 	u32 const wave_kb_last = q_wave0 / at::KV_PER_STEP;                      // inclusive
 
 	for (u32 hh = 0; hh < HPK; ++hh) {
-		u32 const head = blockIdx.y * HPK + hh;
+		u32 const head = head_group * HPK + hh;
 		i8 const *q_head = q + row_base * Q_STRIDE + (size_t)head * HD;
 		i8 const *kv_head = kv + row_base * KV_STRIDE + (size_t)head * 2 * HD;
 
@@ -224,7 +239,7 @@ void kernel(
 #endif
 		};
 		auto widen_v = [&](u32 slot, u32 tile) {
-			if (stager) {
+			if (CPR == 8 || stager) {          // (head_dim 128: every thread stages)
 				v4u raw = *reinterpret_cast<v4u const *>(smem + at::RAW_V_RING_OFFSET + slot * at::RAW_V_TILE_BYTES + tid * 16);
 				// int8 -> f16: b + 128 as an unsigned byte u, 0x6400 | u == 1024 + u, minus 1152
 				v2h const bias = {(_Float16)-1152.0f, (_Float16)-1152.0f};
@@ -354,6 +369,20 @@ void kernel(
 				return (i32)r[0] > (i32)r[1] ? (i32)r[0] : (i32)r[1];
 			};
 
+			// V^T operand of the 32 dims of block db: lane = dim 32 * db + lane % 32, slots = keys 16 * tile + {4 * half .. + 3,
+			// 8 + 4 * half .. + 3}.  The lane's part of the address is the same for both tiles and both key groups
+			// (they differ by whole 256-byte lines: 4096 bytes per tile, 2048 per group of 8 keys).
+			// A key's granules fill CPR * 32 bytes; 16 keys further is always a whole number of 4-line groups further
+			// (the swizzle key repeats), 8 keys further is one only when a key row has at least four granules.
+			u32 v_lane_off[D_BLOCKS];
+			[[maybe_unused]] u32 v_lane_off8[D_BLOCKS];
+			{
+				u32 const t = lane % 16, dh = (lane / 16) % 2;
+				X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
+					v_lane_off[db] = v_granule_offset(4 * half + (t >> 2), 2 * db + dh) + 8 * (t & 3);
+					v_lane_off8[db] = v_granule_offset(8 + 4 * half + (t >> 2), 2 * db + dh) + 8 * (t & 3);
+				}
+			}
 			auto compute = [&]<bool MASKED>(u32 i) __attribute__((always_inline)) {
 				u32 const kb = kb_begin + i;
 				u8 const *k_tile = smem + at::K_RING_OFFSET + (i % at::RING) * at::K_TILE_BYTES;
@@ -372,7 +401,7 @@ void kernel(
 						// the row maximum over the integer dots (the scaling is monotone), scaled once
 						i32 const *a = reinterpret_cast<i32 const *>(&s_acc) + 8 * tile;
 						auto mx = [](i32 x, i32 y) { return x > y ? x : y; };
-						i32 const imax = mx(mx(mx(a[0], a[1]), mx(a[2], a[3])), mx(mx(a[4], a[5]), mx(a[6], a[7])));
+						i32 const imax = mx(mx(mx(mx(mx(mx(mx(a[0], a[1]), a[2]), a[3]), a[4]), a[5]), a[6]), a[7]);     // four max3-type operations
 						tmax = f32(pair_max_i32(imax)) * temperature;
 					} else {
 						X17_UNROLL for (u32 r = 0; r < 8; ++r) sc[r] = f32(s_acc[8 * tile + r]) * temperature;
@@ -419,11 +448,9 @@ void kernel(
 					}
 					v8h const pfrag = __builtin_bit_cast(v8h, pp);
 					X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
-						u32 const t = lane % 16;
-						u32 const dh = (lane / 16) % 2;
-						u32 const key = 16 * tile + 4 * half + (t >> 2);
-						u8 const *p0 = v_tile + v_granule_offset(key, 2 * db + dh) + 8 * (t & 3);
-						u8 const *p1 = v_tile + v_granule_offset(key + 8, 2 * db + dh) + 8 * (t & 3);
+						// (a key's granules fill whole lines of CPR * 32 bytes: 16 keys = one tile further, 8 keys = the other group)
+						u8 const *p0 = v_tile + v_lane_off[db] + tile * (16 * CPR * 32);
+						u8 const *p1 = CPR >= 4 ? p0 + 8 * CPR * 32 : v_tile + v_lane_off8[db] + tile * (16 * CPR * 32);
 						v4s const lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3))) *)p0);
 						v4s const hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3))) *)p1);
 						typedef short v8s __attribute__((ext_vector_type(8)));
