@@ -332,7 +332,20 @@ void kernel(
 			// scalar base and a lane offset; the 8-bit probabilities are rounded and turned into f16 by one addition
 			// and one byte shuffle per pair (PACK_MAGIC), the lift and the removal of the 1024 are one packed fma; the
 			// partial sums are kept at the scale of O (the maximum m_ref), so a moving maximum costs one exponential.
-			v2h neg_bias2 = {(_Float16)-1024.0f, (_Float16)-1024.0f};      // -1024 * lift2
+			// O and the partial sums live at the scale of a reference maximum m_ref that is kept HEADROOM above the
+			// running maximum whenever it is set: the lift 2^(m - m_ref) of new probabilities then starts at 2^-12
+			// (8-bit integers times it are still exact f16 values) and O has to be brought down only after the
+			// maximum has grown by 17 (Gaussian scores move it by that much a few times per query block, not per tile).
+			constexpr f32 HEADROOM = 12.0f, LIFT0 = 1.0f / 4096.0f;
+			m_ref = m + HEADROOM;
+			lift = LIFT0;
+			lift2 = v2h{(_Float16)LIFT0, (_Float16)LIFT0};
+			v2h neg_bias2 = {(_Float16)(-1024.0f * LIFT0), (_Float16)(-1024.0f * LIFT0)};      // -1024 * lift2
+			sum_lo = sum_lo * LIFT0;
+			sum_hi = sum_hi * LIFT0;
+			X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
+				X17_UNROLL for (int r = 0; r < 16; ++r) o_acc[db][r] = o_acc[db][r] * LIFT0;
+			}
 			u32 const first_active = wave_kb_first - kb_begin;
 			u32 const diagonal = wave_kb_last - kb_begin;
 			// first block that lies inside the window of all 32 queries: q_wave0 + 31 - 32 kb <= wr
@@ -419,14 +432,14 @@ void kernel(
 						lift = hw::ex2(m - m_ref);
 						if (__any(lift > MAX_LIFT)) {
 							// O and the partial sums come down to the scale of the new maximum
-							f32 const down = hw::rcp(lift);
+							f32 const down = hw::rcp(lift) * LIFT0;
 							X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
 								X17_UNROLL for (int r = 0; r < 16; ++r) o_acc[db][r] = o_acc[db][r] * down;
 							}
 							sum_lo = sum_lo * down;
 							sum_hi = sum_hi * down;
-							m_ref = m;
-							lift = 1.0f;
+							m_ref = m + HEADROOM;
+							lift = LIFT0;
 						}
 						lift2 = v2h{(_Float16)lift, (_Float16)lift};      // round to nearest
 						neg_bias2 = lift2 * v2h{(_Float16)-1024.0f, (_Float16)-1024.0f};     // exact
