@@ -164,28 +164,19 @@ void kernel(
 	u32 const qlane = lane % 32;
 
 	// Which (sequence, head group, query block) this workgroup takes.  The hardware starts workgroups in the order of
-	// their linear index and deals them round-robin to the 8 XCDs (each with its own L2).  When the (sequence, head
-	// group) pairs divide evenly among the XCDs, each XCD walks its pairs one after the other and the query blocks of
-	// a pair from the last to the first: the workgroups resident on an XCD at one time are neighbouring blocks of one
-	// or two heads, whose key/value windows overlap and stay in its L2, and the blocks with the shortest windows (the
-	// first of each sequence) run last, where they fill the tail of the launch.
-	u32 seq = blockIdx.z;
-	u32 head_group = blockIdx.y;
-	u32 q_block_index = blockIdx.x;
-	{
-		u32 const pairs = gridDim.y * gridDim.z;
-		if (pairs % 8 == 0) {
-			u32 const lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-			u32 const xcd = lin % 8, j = lin / 8;
-			u32 const pair = xcd * (pairs / 8) + j / gridDim.x;
-			q_block_index = gridDim.x - 1 - j % gridDim.x;
-			head_group = pair % gridDim.y;
-			seq = pair / gridDim.y;
-		} else if (gridDim.x % 8 == 0) {
-			// otherwise XCD k gets a contiguous eighth of every sequence
-			q_block_index = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
-		}
-	}
+	// their linear index (and deals them round-robin to the 8 XCDs).  The query block is the slowest index of that
+	// order and runs from the last block to the first: the workgroups in flight at one time are the same few query
+	// blocks of every (sequence, head group) pair -- neighbouring blocks of a pair share most of their key/value
+	// window in the L2 of the XCD the pair keeps landing on when the pairs are a multiple of 8 -- and the blocks with
+	// the shortest windows (the first of each sequence) come last, where they fill the tail of the launch.
+	// Measured against the other orders on both long workloads: 2-4 % faster than query blocks fastest
+	// (4 x 8192 tokens, window 512), 7 % faster on 65536 tokens with a window of 4096.
+	u32 const pairs = gridDim.y * gridDim.z;
+	u32 const lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+	u32 const pair = lin % pairs;
+	u32 const q_block_index = gridDim.x - 1 - lin / pairs;
+	u32 const head_group = pair % gridDim.y;
+	u32 const seq = pair / gridDim.y;
 	size_t const row_base = (size_t)seq * seq_len;          // first row of this sequence
 	u32 const q_block0 = q_block_index * at::Q_PER_BLOCK;   // position of the block's first query
 	u32 const q_wave0 = q_block0 + wave * at::Q_PER_WAVE;
