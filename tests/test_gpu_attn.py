@@ -77,6 +77,31 @@ def test_attn_fast_within_one_code(dev, t, h, hd, w):
 	assert np.max(np.abs(got_l - want_l)) < 1e-4
 
 
+@pytest.mark.parametrize("t,h,hd,w,strict", [(448, 2, 64, 128, True), (192, 4, 32, 0, True), (1088, 2, 128, 256, True),
+                                             (1088, 2, 128, 256, False), (16384 + 64, 2, 128, 512, False)])
+def test_attn_sequence_lengths_that_are_multiples_of_64_only(dev, t, h, hd, w, strict):
+	"""src/device/cuda/attn.rs:398-404 accepts seq_len % 64 == 0; the query block here holds 128 queries.  The last
+	block of such a sequence starts 64 queries early: every output against the oracle (strict builds bit for bit)."""
+	rng = rng_for("attn-t64", t, h, hd, w)
+	q, kv, sk, sv, temp = _attn_inputs(rng, t, h, hd)
+	kern = recipes.attn_kernel(dev, h, hd, strict)
+	got, got_l = _run_attn(dev, kern, q, kv, sk, sv, temp, w)
+	want, want_l = S.attn_fwd_i8(q, kv, sk, sv, temp, h, hd, w)
+	if strict:
+		assert np.array_equal(got, want)
+		assert np.array_equal(got_l.view(np.uint32), want_l.view(np.uint32))
+	else:
+		d = np.abs(got.astype(np.int32) - want.astype(np.int32))
+		assert d.max() <= 1 and np.mean(d > 0) < 0.02, (d.max(), np.mean(d > 0))
+		assert np.max(np.abs(got_l - want_l)) < 1e-4
+	# two stacked sequences of such a length: the second one's rows start at an odd multiple of 64
+	if t == 448:
+		q2, kv2 = np.concatenate((q, q[::-1])), np.concatenate((kv, kv[::-1]))
+		got2, _ = _run_attn(dev, kern, q2, kv2, sk, sv, temp, w, batch=2)
+		assert np.array_equal(got2[:t], want)
+		assert np.array_equal(got2[t:], S.attn_fwd_i8(q[::-1], kv[::-1], sk, sv, temp, h, hd, w)[0])
+
+
 def test_attn_batched_sequences_and_no_l(dev):
 	"""gridDim.z extension: stacked sequences are independent; L may be omitted (attn.rs:396)."""
 	t, h, hd, w, b = 256, 2, 64, 64, 3
@@ -123,7 +148,7 @@ def test_attn_launch_rejects_bad_arguments(dev):
 	q, kv, sk, sv, temp = _attn_inputs(rng, 256, h, hd)
 	with pytest.raises(X.X17Error, match="window_size must be zero or divisible by 16"):
 		_run_attn(dev, kern, q, kv, sk, sv, temp, 24)
-	with pytest.raises(X.X17Error, match="seq_len must be divisible by 128"):
+	with pytest.raises(X.X17Error, match="seq_len must be divisible by 64 and at least 128"):
 		_run_attn(dev, kern, q[:64], kv[:64], sk, sv, temp, 0)
 	with pytest.raises(X.X17Error, match="kv has 128 rows, but should have 256"):
 		_run_attn(dev, kern, q, kv[:128], sk, sv, temp, 0)

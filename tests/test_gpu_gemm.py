@@ -168,6 +168,47 @@ def test_fused_q_kv_projection_equals_the_two_kernels(dev, hd):
 		kern.launch(_up(dev, x, X.INT8), _up(dev, wq, X.INT8), q, rrms)
 
 
+def test_shapes_of_the_reference_that_are_not_whole_tiles(dev):
+	"""src/device/cuda/gemm.rs:605-614 accepts rows % 64 == 0 and raw columns % 128 == 0; the tile here is 256 x 256.
+	320 token rows x 384 raw columns (one full tile and an overhanging one in each direction) through every writer,
+	against the oracle over the whole output; below one tile and off the 64 / 128 grid are errors."""
+	m, k, n = 320, 512, 384
+	rng = rng_for("tails")
+	a, b = i8_codes(rng, (m, k)), i8_codes(rng, (n, k))
+	acc = S.gemm_i32(a, b)
+	inp = 1.0 / math.sqrt(k) / 64.0
+	ta, tb = _up(dev, a, X.INT8), _up(dev, b, X.INT8)
+	c = X.Tensor(dev, (m, n), X.INT8)
+	recipes.attn_q_kernel(dev, k, n).launch(ta, tb, c)
+	assert np.array_equal(c.download(), S.epilogue_scale(acc, inp, 8.0))
+	ch = X.Tensor(dev, (m, n // 2), X.E4M3)
+	recipes.ffn_f_kernel(dev, k, n, True, X.E4M3).launch(ta, tb, ch)
+	assert np.array_equal(ch.download(), S.epilogue_geglu(acc, inp, 1.0, S.STORE_E4M3))
+	res = i8_codes(rng, (m, n // 2))
+	recipes.attn_y_kernel(dev, n // 2, k, True).launch(ta, tb, ch, _up(dev, res, X.INT8))
+	assert np.array_equal(ch.download(), S.epilogue_residual(acc, res, inp, 1.0, S.STORE_E4M3))
+	for hd in (32, 64):
+		rrms = X.Tensor(dev, (m, n // (2 * hd)), X.F32)
+		recipes.attn_kv_kernel(dev, k, n, hd).launch(ta, tb, c, rrms)
+		want_c, want_r = S.epilogue_l2norm(acc, hd, recipes.L2_NORM_EPS, inp, 8.0)
+		assert np.array_equal(c.download(), want_c)
+		assert np.array_equal(rrms.download().view(np.uint32), want_r.view(np.uint32))
+	# e4m3 activations x int8 weights (the four-wave form)
+	ae = e4m3_bytes(rng, (m, k))
+	recipes.mixed_gemm_kernel(dev, k, n, False).launch(_up(dev, ae, X.E4M3), tb, c)
+	want = S.epilogue_scale(S.gemm_f32_seq(ae, True, b, False), 1.0 / math.sqrt(k) / 8.0, 8.0)
+	assert np.abs(c.download().astype(np.int32) - want.astype(np.int32)).max() <= 1
+	# what the reference rejects is rejected here too, and so is less than one tile
+	kern = recipes.attn_q_kernel(dev, k, n)
+	for rows in (288, 192):
+		with pytest.raises(X.X17Error, match="divisible by \\[64, 128\\]"):
+			kern.launch(_up(dev, a[:rows], X.INT8), tb, X.Tensor(dev, (rows, n), X.INT8))
+	with pytest.raises(X.X17Error, match="multiple of 128"):
+		recipes.attn_q_kernel(dev, k, 320)
+	with pytest.raises(X.X17Error, match="at least one tile"):
+		recipes.attn_q_kernel(dev, k, 128)
+
+
 @pytest.mark.parametrize("store", [X.E4M3, X.INT8])
 @pytest.mark.parametrize("m,k,n", SHAPES)
 def test_geglu_epilogue(dev, m, k, n, store):
@@ -400,7 +441,7 @@ def test_launch_rejects_bad_arguments(dev):
 		kern.launch(X.Tensor(dev, (256, 2 * k), X.INT8), b, c)
 	with pytest.raises(X.X17Error, match="must be 2D"):
 		kern.launch(X.Tensor(dev, (256, k, 1), X.INT8), b, c)
-	with pytest.raises(X.X17Error, match="must be divisible by tile shape"):
+	with pytest.raises(X.X17Error, match="at least one tile"):
 		kern.launch(X.Tensor(dev, (64, k), X.INT8), b, X.Tensor(dev, (64, n), X.INT8))
 	with pytest.raises(X.X17Error, match="is not on device"):
 		kern.launch(X.Tensor(None, (256, k), X.INT8), b, c)

@@ -85,7 +85,12 @@ def _gemm(a, b, c, k=256, n=256, trans_a=False, trans_b=True, rows=True):
 	(_gemm(X.INT8, X.INT8, X.INT8), X.RMSNormConfig(1e-9, 48, 48, 1.0, 1.0), "multiples of 32"),
 	(_gemm(X.INT8, X.INT8, X.INT8), X.RMSNormConfig(1e-9, 32, 64, 1.0, 1.0), "head_dim == sep_dim"),
 	(_gemm(X.INT8, X.INT8, X.INT8, k=200), X.ScaleConfig(1.0, 1.0), "multiple of 128"),
-	(_gemm(X.INT8, X.INT8, X.INT8, n=192), X.ScaleConfig(1.0, 1.0), "raw output columns must be a multiple of 256"),
+	(_gemm(X.INT8, X.INT8, X.INT8, n=192), X.ScaleConfig(1.0, 1.0), "raw output columns must be a multiple of 128"),
+	(_gemm(X.INT8, X.INT8, X.INT8, n=128), X.ScaleConfig(1.0, 1.0), "at least one tile"),
+	(_gemm(X.INT8, X.INT8, X.INT8), X.QNormConfig(0.0, 48, 8.0), "head_dim in"),
+	(_gemm(X.INT8, X.INT8, X.E4M3), X.QNormConfig(0.0, 64, 8.0), "QNorm epilogue requires i8"),
+	(_gemm(X.INT8, X.INT8, X.INT8, n=768), X.QkvConfig(128, X.ScaleConfig(1.0, 8.0), X.RMSNormConfig(1e-9, 64, 64, 1.0, 8.0)), "q_cols must be a multiple of 256"),
+	(_gemm(X.INT8, X.INT8, X.INT8, n=768), X.QkvConfig(256, X.ScaleConfig(1.0, 8.0), X.RMSNormConfig(1e-9, 64, 32, 1.0, 8.0)), "head_dim == sep_dim"),
 ])
 def test_gemm_kernel_config_validation(cfg, epi, msg):
 	with pytest.raises(X.X17Error, match=msg):

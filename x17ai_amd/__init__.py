@@ -11,11 +11,12 @@ from ._ffi import X17Error, lib_paths
 from .api import (
 	BF16, E4M3, F32, INT8,
 	AttnDecodeKernel, AttnKernel, AttnKernelConfig, DequantConfig, Device, GeGluConfig, GemmConfig, GemmInputConfig,
-	GemmKernel, ResidualConfig, RMSNormConfig, RmsNormKernel, ScaleConfig, Tensor, Timer,
+	GemmKernel, QkvConfig, QNormConfig, ResidualConfig, RMSNormConfig, RmsNormKernel, ScaleConfig, Tensor, Timer,
 )
 
 __all__ = [
 	"X17Error", "lib_paths", "BF16", "E4M3", "F32", "INT8", "AttnDecodeKernel", "AttnKernel", "AttnKernelConfig",
-	"DequantConfig", "Device", "GeGluConfig", "GemmConfig", "GemmInputConfig", "GemmKernel", "ResidualConfig", "RMSNormConfig",
+	"DequantConfig", "Device", "GeGluConfig", "GemmConfig", "GemmInputConfig", "GemmKernel", "QkvConfig", "QNormConfig",
+	"ResidualConfig", "RMSNormConfig",
 	"RmsNormKernel", "ScaleConfig", "Tensor", "Timer",
 ]

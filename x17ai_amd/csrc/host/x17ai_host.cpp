@@ -855,6 +855,9 @@ std::unique_ptr<GemmKernel> GemmKernel::create(std::shared_ptr<HipDevice> device
 	}
 
 	if (g.a.cols % 128 != 0) { diag.add_error("GEMM K must be a multiple of 128, got " + std::to_string(g.a.cols)); return nullptr; }
+	// gemm.rs:607-614 (N_PER_BLOCK of the reference's tile)
+	if (b_rows % 128 != 0) { diag.add_error("GEMM raw output columns must be a multiple of 128, got " + std::to_string(b_rows)); return nullptr; }
+	if (b_rows < 256) { diag.add_error("GEMM raw output columns must be at least one tile (256), got " + std::to_string(b_rows)); return nullptr; }
 
 	auto built = kernel_build::build(kernel_name, common.str(), "gemm_b8.hip", "gemm_meta.cpp", diag);
 	if (!built) return nullptr;
@@ -869,8 +872,10 @@ std::unique_ptr<GemmKernel> GemmKernel::create(std::shared_ptr<HipDevice> device
 		diag.add_error("Invalid JSON metadata in " + built->meta_json_path);
 		return nullptr;
 	}
-	if (b_rows % out->metadata.N_PER_BLOCK != 0) {
-		diag.add_error("GEMM raw output columns (" + std::to_string(b_rows) + ") must be divisible by the tile width "
+	// gemm.rs:607-614 accepts raw columns % 128 == 0 (its tile is 64 x 128).  The tile here is wider; a last tile that
+	// would overhang is moved back to end at the matrix edge, so the same shapes are accepted from one tile upwards.
+	if (b_rows % 128 != 0 || b_rows < out->metadata.N_PER_BLOCK) {
+		diag.add_error("GEMM raw output columns (" + std::to_string(b_rows) + ") must be a multiple of 128 and at least the tile width "
 			+ std::to_string(out->metadata.N_PER_BLOCK));
 		return nullptr;
 	}
@@ -923,9 +928,10 @@ Status GemmKernel::launch(GemmArgs const &args) {
 		s = tensor_check::matrix_shape(op, "residual", *args.extra, a_rows, out_cols, *device, DType::Int8, tmp);
 		if (!s.is_ok()) return s;
 	}
-	if ((a_rows & (metadata.M_PER_BLOCK - 1)) != 0 || (b_rows_v & (metadata.N_PER_BLOCK - 1)) != 0) {
+	// gemm.rs:607-614: rows % 64 == 0, raw columns % 128 == 0 (the reference's tile shape); here from one tile upwards
+	if (a_rows % 64 != 0 || b_rows_v % 128 != 0 || a_rows < metadata.M_PER_BLOCK || b_rows_v < metadata.N_PER_BLOCK) {
 		return Status::err(TensorOpError::Other, std::string(op) + " raw output shape [" + std::to_string(a_rows) + ", "
-			+ std::to_string(b_rows_v) + "] must be divisible by tile shape [" + std::to_string(metadata.M_PER_BLOCK) + ", "
+			+ std::to_string(b_rows_v) + "] must be divisible by [64, 128] and at least one tile [" + std::to_string(metadata.M_PER_BLOCK) + ", "
 			+ std::to_string(metadata.N_PER_BLOCK) + "]");
 	}
 	if (epilogue_kind == 4) {
@@ -952,8 +958,8 @@ Status GemmKernel::launch(GemmArgs const &args) {
 	if (a_rows > 0xFFFFFFFFull || b_rows_v > 0xFFFFFFFFull) {
 		return Status::err(TensorOpError::Other, std::string(op) + " sizes exceed 32 bits (the kernel's row counts are u32)");
 	}
-	size_t grid_x = a_rows >> ctz(metadata.M_PER_BLOCK);
-	size_t grid_y = b_rows_v >> ctz(metadata.N_PER_BLOCK);
+	size_t grid_x = (a_rows + metadata.M_PER_BLOCK - 1) >> ctz(metadata.M_PER_BLOCK);
+	size_t grid_y = (b_rows_v + metadata.N_PER_BLOCK - 1) >> ctz(metadata.N_PER_BLOCK);
 	// 8-byte slots passed by address, exactly as gemm.rs:618-631 does; the kernel's u32 parameters
 	// read the low halves.
 	void *a_ptr = args.a->ptr;
@@ -992,8 +998,8 @@ Status GemmKernel::launch_qkv(GemmArgs const &args, size_t a_rows) {
 	if (!s.is_ok()) return s;
 	s = tensor_check::matrix_shape(op, "rrms", *args.extra, a_rows, kv_cols >> ctz(head_dim + sep_dim), *device, DType::F32, tmp);
 	if (!s.is_ok()) return s;
-	if ((a_rows & (metadata.M_PER_BLOCK - 1)) != 0) {
-		return Status::err(TensorOpError::Other, std::string(op) + " token rows (" + std::to_string(a_rows) + ") must be divisible by the tile height "
+	if (a_rows % 64 != 0 || a_rows < metadata.M_PER_BLOCK) {
+		return Status::err(TensorOpError::Other, std::string(op) + " token rows (" + std::to_string(a_rows) + ") must be a multiple of 64 and at least the tile height "
 			+ std::to_string(metadata.M_PER_BLOCK));
 	}
 	if (a_rows > 0xFFFFFFFFull) return Status::err(TensorOpError::Other, std::string(op) + " sizes exceed 32 bits (the kernel's row counts are u32)");
@@ -1006,7 +1012,7 @@ Status GemmKernel::launch_qkv(GemmArgs const &args, size_t a_rows) {
 	void *b2_ptr = args.b2->ptr;
 	void *c2_ptr = args.c2->ptr;
 	void *raw_args[8] = {&a_ptr, &a_rows_arg, &b_ptr, &b_rows_arg, &c_ptr, &rrms_ptr, &b2_ptr, &c2_ptr};
-	size_t tiles = (a_rows >> ctz(metadata.M_PER_BLOCK)) * (*b_rows >> ctz(metadata.N_PER_BLOCK));
+	size_t tiles = ((a_rows + metadata.M_PER_BLOCK - 1) >> ctz(metadata.M_PER_BLOCK)) * ((*b_rows + metadata.N_PER_BLOCK - 1) >> ctz(metadata.N_PER_BLOCK));
 	size_t grid[3] = {metadata.MAX_BLOCKS != 0 && tiles > metadata.MAX_BLOCKS ? metadata.MAX_BLOCKS : tiles, 1, 1};
 	size_t block[3] = {metadata.THREADS_PER_BLOCK, 1, 1};
 	return kernel->launch(*device->stream, grid, block, metadata.SMEM_BYTES, raw_args);
@@ -1132,8 +1138,11 @@ Status AttnKernel::launch(AttnKernelArgs const &a) {
 		return Status::err(TensorOpError::Other, "attention rows (" + std::to_string(rows) + ") must be divisible by batch (" + std::to_string(a.batch) + ")");
 	}
 	size_t const seq_len = rows / a.batch;
-	if ((seq_len & (metadata.Q_PER_BLOCK - 1)) != 0) {
-		return Status::err(TensorOpError::Other, "attention seq_len must be divisible by " + std::to_string(metadata.Q_PER_BLOCK)
+	// attn.rs:398-404: seq_len % 64 == 0 (the reference's query block).  The query block here is larger; a last block
+	// that would overhang starts earlier instead (it recomputes some of its neighbour's queries and stores the same
+	// bytes), so the same lengths are accepted from one block upwards.
+	if (seq_len % 64 != 0 || seq_len < metadata.Q_PER_BLOCK) {
+		return Status::err(TensorOpError::Other, "attention seq_len must be divisible by 64 and at least " + std::to_string(metadata.Q_PER_BLOCK)
 			+ ", got " + std::to_string(seq_len));
 	}
 	if (a.window_size > 0 && a.window_size % 16 != 0) {
@@ -1155,7 +1164,7 @@ Status AttnKernel::launch(AttnKernelArgs const &a) {
 	// the plain kernel takes the first nine arguments only
 	void *raw_args[14] = {&seq_len_arg, &q_ptr, &kv_ptr, &sk, &sv, &tp, &out_ptr, &l_ptr, &window_arg,
 	                      &scale_ptrs[0], &scale_ptrs[1], &scale_ptrs[2], &scale_ptrs[3], &scale_ptrs[4]};
-	size_t grid[3] = {seq_len / metadata.Q_PER_BLOCK, config.head_group_cnt(), a.batch};
+	size_t grid[3] = {(seq_len + metadata.Q_PER_BLOCK - 1) / metadata.Q_PER_BLOCK, config.head_group_cnt(), a.batch};
 	size_t block[3] = {metadata.THREADS_PER_BLOCK, 1, 1};
 	return kernel->launch(*device->stream, grid, block, metadata.SMEM_BYTES, raw_args);
 }

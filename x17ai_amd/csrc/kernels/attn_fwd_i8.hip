@@ -178,7 +178,9 @@ void kernel(
 	u32 const head_group = pair % gridDim.y;
 	u32 const seq = pair / gridDim.y;
 	size_t const row_base = (size_t)seq * seq_len;          // first row of this sequence
-	u32 const q_block0 = q_block_index * at::Q_PER_BLOCK;   // position of the block's first query
+	// position of the block's first query; a last block that would overhang the sequence (lengths are multiples of 64,
+	// src/device/cuda/attn.rs:398-404) starts earlier and recomputes some of its neighbour's queries
+	u32 const q_block0 = q_block_index * at::Q_PER_BLOCK + at::Q_PER_BLOCK > seq_len ? seq_len - at::Q_PER_BLOCK : q_block_index * at::Q_PER_BLOCK;
 	u32 const q_wave0 = q_block0 + wave * at::Q_PER_WAVE;
 	u32 const qi = q_wave0 + qlane;                         // this lane's query position
 

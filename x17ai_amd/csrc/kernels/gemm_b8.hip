@@ -77,7 +77,7 @@ constexpr int MMA = (A_KIND == 0 && B_KIND == 0) ? 0 : ((A_KIND == 1 && B_KIND =
 constexpr bool ACC_F32 = MMA != 0;
 
 static_assert(K_TOTAL % gt::K_STEP == 0, "K must be a multiple of 128");
-static_assert(N_RAW % gt::N_PER_BLOCK == 0, "raw output columns must be a multiple of 256");
+static_assert(N_RAW % 128 == 0 && N_RAW >= gt::N_PER_BLOCK, "raw output columns: a multiple of 128, at least one tile");
 
 constexpr u32 ROW_BYTES = gt::K_STEP;                       // one LDS row = one step of K
 constexpr u32 X_TILE_BYTES = gt::M_PER_BLOCK * ROW_BYTES;   // tokens
@@ -812,8 +812,12 @@ void kernel(
 	// workgroup runs the loop once).  The linear tile id is remapped so that each XCD (own L2) gets a
 	// compact block of tiles -- the hardware deals workgroups round-robin to the 8 XCDs -- and tiles
 	// are walked in bands of token-tiles so that co-resident tiles share weight and token panels.
-	u32 const tiles_m = a_rows / gt::M_PER_BLOCK;
-	constexpr u32 tiles_n = N_RAW / gt::N_PER_BLOCK;
+	// A shape that is not a whole number of tiles (src/device/cuda/gemm.rs:605-614 accepts rows % 64 == 0 and raw
+	// columns % 128 == 0) is covered by moving the last tile of a row or column of tiles back until it ends at the
+	// matrix edge: it recomputes a few rows or columns of its neighbour and stores the same bytes again, and nothing
+	// in the kernel needs a predicate.  (tile_coords hands out a tile's first row and first raw column.)
+	u32 const tiles_m = (a_rows + gt::M_PER_BLOCK - 1) / gt::M_PER_BLOCK;
+	constexpr u32 tiles_n = (N_RAW + gt::N_PER_BLOCK - 1) / gt::N_PER_BLOCK;
 	u32 const total = tiles_m * tiles_n;
 	u32 const n_groups = gridDim.x * gridDim.y * gridDim.z;
 	u32 const group = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
@@ -830,8 +834,10 @@ void kernel(
 		u32 band = lin / band_tiles;
 		u32 in_band = lin % band_tiles;
 		u32 rows_in_band = (tiles_m - band * BAND) < BAND ? (tiles_m - band * BAND) : BAND;
-		tile_m = band * BAND + in_band % rows_in_band;
-		tile_n = in_band / rows_in_band;
+		tile_m = (band * BAND + in_band % rows_in_band) * gt::M_PER_BLOCK;
+		tile_n = (in_band / rows_in_band) * gt::N_PER_BLOCK;
+		tile_m = tile_m + gt::M_PER_BLOCK > a_rows ? a_rows - gt::M_PER_BLOCK : tile_m;
+		tile_n = tile_n + gt::N_PER_BLOCK > N_RAW ? N_RAW - gt::N_PER_BLOCK : tile_n;
 	};
 	if (group >= total) {
 		return;
@@ -890,18 +896,19 @@ void kernel(
 	u32 const x_off = wm * gt::WAVE_M * ROW_BYTES + lo.frag_row;
 	u32 const w_off = W_RING_OFFSET + wn * gt::WAVE_N * ROW_BYTES + lo.frag_row;
 
-	// the weight rows of column tile t: one matrix, or (fused q + kv) the q weights followed by the kv weights
-	auto weight_tile = [&](u32 t) -> u8 const * {
+	// the weight rows of the tile whose first raw column is `col`: one matrix, or (fused q + kv) the q weights
+	// followed by the kv weights
+	auto weight_tile = [&](u32 col) -> u8 const * {
 #if X17_EPILOGUE == 6
-		constexpr u32 Q_TILES = X17_Q_COLS / gt::N_PER_BLOCK;
-		return t < Q_TILES ? b + (size_t)(t * gt::N_PER_BLOCK) * K_TOTAL : b_kv + (size_t)((t - Q_TILES) * gt::N_PER_BLOCK) * K_TOTAL;
+		static_assert(X17_Q_COLS % gt::N_PER_BLOCK == 0 && N_RAW - X17_Q_COLS >= gt::N_PER_BLOCK, "q and kv parts are whole tiles / at least a tile");
+		return col < X17_Q_COLS ? b + (size_t)col * K_TOTAL : b_kv + (size_t)(col - X17_Q_COLS) * K_TOTAL;
 #else
-		return b + (size_t)(t * gt::N_PER_BLOCK) * K_TOTAL;
+		return b + (size_t)col * K_TOTAL;
 #endif
 	};
 	u32 tile_m, tile_n;
 	tile_coords(group, tile_m, tile_n);
-	u8 const *a_tile = a + (size_t)(tile_m * gt::M_PER_BLOCK) * K_TOTAL;
+	u8 const *a_tile = a + (size_t)tile_m * K_TOTAL;
 	u8 const *b_tile = weight_tile(tile_n);
 	// the first steps of a tile nobody prefetched, in the order the waits of the main loop assume
 	// (token tile s, weight tile s, ..., then the extra token tile of a deeper token ring)
@@ -929,7 +936,7 @@ void kernel(
 		if (more_tiles) {
 			tile_coords(lin + n_groups, next_m, next_n);
 		}
-		u8 const *a_next = a + (size_t)(next_m * gt::M_PER_BLOCK) * K_TOTAL;
+		u8 const *a_next = a + (size_t)next_m * K_TOTAL;
 		u8 const *b_next = weight_tile(next_n);
 		if constexpr (!CROSS_TILE) {
 			if (!first_tile) {
@@ -1098,8 +1105,8 @@ void kernel(
 
 	// ---- epilogue.  Lane owns token (32*bm + lane%32) of its wave and raw columns
 	// LANE_COLS*(lane/32) + 16*bn + r of its wave, r = accumulator register index.
-	u32 const row0 = tile_m * gt::M_PER_BLOCK + wm * gt::WAVE_M + lane % 32;
-	u32 const n0 = tile_n * gt::N_PER_BLOCK + wn * gt::WAVE_N + LANE_COLS * lo.half;
+	u32 const row0 = tile_m + wm * gt::WAVE_M + lane % 32;
+	u32 const n0 = tile_n + wn * gt::WAVE_N + LANE_COLS * lo.half;
 
 	X17_UNROLL for (int bm = 0; bm < BM; ++bm) {
 		if constexpr (gt::WAVES_PER_SIMD == 1) {
@@ -1132,13 +1139,13 @@ void kernel(
 #elif X17_EPILOGUE == 4
 		DequantEpilogue::run(x, c, row, n0, row_scale, col_scale);
 #elif X17_EPILOGUE == 3
-		NaturalWriters::l2norm_row(x, c, rrms, row, tile_n * gt::N_PER_BLOCK + wn * gt::WAVE_N, N_RAW, lo.half);
+		NaturalWriters::l2norm_row(x, c, rrms, row, tile_n + wn * gt::WAVE_N, N_RAW, lo.half);
 #elif X17_EPILOGUE == 5
-		NaturalWriters::qnorm_row(x, c, q_norm_scales, row, tile_n * gt::N_PER_BLOCK + wn * gt::WAVE_N, lo.half);
+		NaturalWriters::qnorm_row(x, c, q_norm_scales, row, tile_n + wn * gt::WAVE_N, lo.half);
 #else
 		{
 			constexpr u32 Q_COLS = X17_Q_COLS;
-			u32 const col0 = tile_n * gt::N_PER_BLOCK + wn * gt::WAVE_N;
+			u32 const col0 = tile_n + wn * gt::WAVE_N;
 			if (col0 < Q_COLS) {
 				NaturalWriters::scale_row(x, c, row, col0, Q_COLS, lo.half);
 			} else {

@@ -44,6 +44,13 @@ def _specs():
 	add(("attn_q_norm", 2048, 1024, 128, recipes.L2_NORM_EPS))
 	for hd in (64, 128):                 # L2-norm writer on a walk of more tiles than workgroups
 		add(("attn_kv", 256, 2048, hd))
+	# shapes off the 256-grid (rows % 64, raw columns % 128 as the reference accepts them)
+	add(("attn_q", 512, 384))
+	add(("ffn_f", 512, 384, True, E4M3))
+	add(("attn_y", 192, 512, True, E4M3))
+	for hd in (32, 64):
+		add(("attn_kv", 512, 384, hd))
+	add(("mixed", 512, 384, False))
 	add(("attn_q", 384, 1024))           # the shortest K with the deeper token ring, more tiles than workgroups
 	add(("ffn_f_f8", 384, 512, True))
 	# ---- tests/test_gpu_attn.py
