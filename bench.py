@@ -249,7 +249,7 @@ def cpu_extras():
 def mfma_probe(dev, X):
 	"""Loops of nothing but MFMAs on register operands, all-zero and Gaussian data: what the matrix cores of this
 	machine sustain (the clock under dense MFMA load depends on how much the operands toggle)."""
-	from x17ai_amd.api import MfmaProbe
+	from x17ai_amd.probes import MfmaProbe
 	rng = np.random.default_rng(7)
 	out = X.Tensor(dev, (256 * 512,), X.F32)
 	result = {}
@@ -271,6 +271,27 @@ def mfma_probe(dev, X):
 			med, mn = _median_launch(dev, X, fn, 10, 3)
 			result[f"{name}_{data_name}"] = {"median_us": med * 1e6, "tops": ops[0] / med / 1e12,
 			                                 "frac_of_nominal_peak": ops[0] / med / 1e12 / peak}
+	return result
+
+
+def valu_probe(dev, X):
+	"""Issue rate of single vector instructions, in nanoseconds of SIMD time per wavefront-instruction, with 1, 2, 3,
+	4 and 8 wavefronts on every SIMD of the chip."""
+	from x17ai_amd.probes import ValuProbe, valu_probe_ops
+	src = X.Tensor.from_numpy(dev, np.zeros(256, np.float32), X.F32)
+	out = X.Tensor(dev, (1024 * 8 * 64,), X.F32)
+	result = {}
+	for op, name in enumerate(valu_probe_ops()):
+		probe = ValuProbe(dev, op)
+		row = {}
+		for waves in (1, 2, 3, 4, 8):
+			n = [0.0]
+
+			def fn():
+				n[0] = probe.launch(src, out, waves, 1024)
+			med, mn = _median_launch(dev, X, fn, 5, 2)
+			row[f"waves_{waves}"] = mn * 1e9 / n[0]
+		result[name] = row
 	return result
 
 
@@ -547,6 +568,9 @@ def main():
 	ap.add_argument("--mfma-probe", action="store_true",
 	                help="only run loops of nothing but MFMAs on register operands (all-zero and Gaussian data; int8, "
 	                     "e4m3, f16): what the matrix cores of this machine sustain, beside the nominal peaks")
+	ap.add_argument("--valu-probe", action="store_true",
+	                help="only run loops of one vector instruction each (issue rate per instruction and wavefronts per SIMD: "
+	                     "what bounds the attention kernel's softmax)")
 	ap.add_argument("--only", choices=ONLY_TARGETS,
 	                help="launch one kernel of one workload --steps times and print its median (used for the profiles)")
 	args = ap.parse_args()
@@ -559,7 +583,7 @@ def main():
 
 	dev = X.Device(0)
 	if args.copy_probe:
-		from x17ai_amd.api import CopyProbe
+		from x17ai_amd.probes import CopyProbe
 		n = 1 << 30
 		src = X.Tensor.from_numpy(dev, np.zeros(n, np.int8), X.INT8)
 		dst = X.Tensor(dev, (n,), X.INT8)
@@ -571,6 +595,9 @@ def main():
 		return
 	if args.mfma_probe:
 		print(json.dumps({"mfma_probe": mfma_probe(dev, X)}))
+		return
+	if args.valu_probe:
+		print(json.dumps({"valu_probe_ns_per_wave_instruction_per_simd": valu_probe(dev, X)}))
 		return
 	if args.only:
 		single(dev, X, recipes, args.only, args.steps)

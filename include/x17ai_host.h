@@ -176,20 +176,6 @@ int x17h_decode_kernel_launch_row_scaled(X17hDecodeKernel *k, X17hTensor *q, X17
                                          X17hTensor *q_scale, X17hTensor *k_scale, X17hTensor *v_weight,
                                          X17hTensor *sink_v_weight, X17hTensor *out_scale);
 
-/* Measurement aid with no reference counterpart: a plain device-to-device copy kernel of known
- * size, against which HBM-traffic counters are calibrated (src and dst: equal sizes, multiple of 16). */
-typedef struct X17hMfmaProbe X17hMfmaProbe;
-/* Measurement aid with no reference counterpart: a loop of nothing but matrix-core instructions on register
- * operands taken from `operands` (at least 98304 bytes; what the machine sustains depends on their values).
- * kind: 0 int8, 1 e4m3, 2 f16.  `out` takes 4 bytes per thread (256 x 512); *ops receives the operations launched. */
-int x17h_mfma_probe_new(X17hDevice *dev, int kind, X17hMfmaProbe **out);
-void x17h_mfma_probe_free(X17hMfmaProbe *p);
-int x17h_mfma_probe_launch(X17hMfmaProbe *p, X17hTensor *operands, X17hTensor *out, size_t iterations, double *ops);
-typedef struct X17hCopyProbe X17hCopyProbe;
-int x17h_copy_probe_new(X17hDevice *dev, X17hCopyProbe **out);
-void x17h_copy_probe_free(X17hCopyProbe *p);
-int x17h_copy_probe_launch(X17hCopyProbe *p, X17hTensor *src, X17hTensor *dst);
-
 #ifdef __cplusplus
 }
 #endif

@@ -18,7 +18,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def _declared(header):
 	text = open(os.path.join(ROOT, "include", header)).read()
 	text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-	return sorted(set(re.findall(r"\b(x17(?:ai|h)_[a-z0-9_]+)\s*\(", text)))
+	return sorted(set(re.findall(r"\b(x17(?:ai|h|p)_[a-z0-9_]+)\s*\(", text)))
 
 
 def _exported(lib):
@@ -37,6 +37,16 @@ def test_host_library_exports_every_declared_entry_point():
 	declared = _declared("x17ai_host.h")
 	exported = set(_exported(_ffi.lib_paths()["host"]))
 	assert declared and not [s for s in declared if s not in exported]
+
+
+def test_probe_library_exports_its_header_and_the_product_header_names_no_probe():
+	"""The benchmark's measurement aids live in their own header and library."""
+	declared = _declared("x17ai_probe.h")
+	path = os.path.join(os.path.dirname(_ffi.lib_paths()["host"]), "libx17ai_probe.so")
+	exported = set(_exported(path))
+	assert declared and not [s for s in declared if s not in exported]
+	assert not [s for s in _declared("x17ai_host.h") if "probe" in s]
+	assert not [s for s in _exported(_ffi.lib_paths()["host"]) if "probe" in s and s.startswith("x17h_")]
 
 
 def test_struct_layouts_match_the_reference_ffi(tmp_path):

@@ -125,14 +125,6 @@ def host() -> ctypes.CDLL:
 	h.x17h_decode_kernel_free.argtypes = [P]
 	h.x17h_decode_kernel_free.restype = None
 	h.x17h_decode_kernel_launch.argtypes = [P, P, P, P, P, P, P, P, P, SZ]
-	h.x17h_mfma_probe_new.argtypes = [P, ctypes.c_int, PP]
-	h.x17h_mfma_probe_free.argtypes = [P]
-	h.x17h_mfma_probe_free.restype = None
-	h.x17h_mfma_probe_launch.argtypes = [P, P, P, SZ, ctypes.POINTER(ctypes.c_double)]
-	h.x17h_copy_probe_new.argtypes = [P, PP]
-	h.x17h_copy_probe_free.argtypes = [P]
-	h.x17h_copy_probe_free.restype = None
-	h.x17h_copy_probe_launch.argtypes = [P, P, P]
 	_host = h
 	return h
 

@@ -471,47 +471,3 @@ class AttnDecodeKernel:
 				self._h = ctypes.c_void_p()
 		except Exception:
 			pass
-
-
-class MfmaProbe:
-	"""A loop of nothing but matrix-core instructions on register operands (measurement aid: what the matrix cores
-	sustain on given operand data).  kind: 0 int8, 1 e4m3, 2 f16."""
-
-	def __init__(self, device: Optional[Device], kind: int):
-		self.device = device
-		self._h = ctypes.c_void_p()
-		check(_ffi.host().x17h_mfma_probe_new(device._h if device is not None else None, kind, ctypes.byref(self._h)))
-
-	def launch(self, operands: Tensor, out: Tensor, iterations: int) -> float:
-		"""Returns the number of operations launched."""
-		ops = ctypes.c_double()
-		check(_ffi.host().x17h_mfma_probe_launch(self._h, operands._h, out._h, iterations, ctypes.byref(ops)))
-		return float(ops.value)
-
-	def __del__(self):
-		try:
-			if self._h:
-				_ffi.host().x17h_mfma_probe_free(self._h)
-				self._h = ctypes.c_void_p()
-		except Exception:
-			pass
-
-
-class CopyProbe:
-	"""A plain device-to-device copy kernel of known size (measurement aid for counter calibration)."""
-
-	def __init__(self, device: Optional[Device]):
-		self.device = device
-		self._h = ctypes.c_void_p()
-		check(_ffi.host().x17h_copy_probe_new(device._h if device is not None else None, ctypes.byref(self._h)))
-
-	def launch(self, src: Tensor, dst: Tensor) -> None:
-		check(_ffi.host().x17h_copy_probe_launch(self._h, src._h, dst._h))
-
-	def __del__(self):
-		try:
-			if self._h:
-				_ffi.host().x17h_copy_probe_free(self._h)
-				self._h = ctypes.c_void_p()
-		except Exception:
-			pass

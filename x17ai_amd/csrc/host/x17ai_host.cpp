@@ -680,13 +680,13 @@ namespace kernel_build {
 		return out;
 	}
 
-	static std::optional<size_t> meta_get(std::vector<std::pair<std::string, size_t>> const &m, char const *key) {
+	std::optional<size_t> meta_get(std::vector<std::pair<std::string, size_t>> const &m, char const *key) {
 		for (auto const &kv : m) if (kv.first == key) return kv.second;
 		return std::nullopt;
 	}
 
 	// kernel_build.rs:161-198
-	static std::unique_ptr<HipKernel> load_kernel(HipStream &stream, std::string const &path, char const *name, size_t smem, Diagnostics &diag) {
+	std::unique_ptr<HipKernel> load_kernel(HipStream &stream, std::string const &path, char const *name, size_t smem, Diagnostics &diag) {
 		if (path.find('\0') != std::string::npos) {
 			diag.add_error("kernel path contains a NUL byte");
 			return nullptr;
@@ -1350,8 +1350,6 @@ Status AttnDecodeKernel::launch(AttnDecodeArgs const &a) {
 
 using namespace x17;
 
-struct X17hDevice { std::shared_ptr<HipDevice> dev; };
-struct X17hTensor { std::shared_ptr<Tensor> t; };
 struct X17hTimer { std::unique_ptr<HipTimer> t; };
 struct X17hGemmKernel { std::unique_ptr<GemmKernel> k; };
 struct X17hAttnKernel { std::unique_ptr<AttnKernel> k; };
@@ -1646,80 +1644,6 @@ int x17h_decode_kernel_launch(X17hDecodeKernel *k, X17hTensor *q, X17hTensor *ca
 	AttnDecodeArgs a{q->t.get(), cache->t.get(), cache_len->t.get(), sink_k->t.get(), sink_v->t.get(), temp->t.get(), out->t.get(),
 	                 l != nullptr ? l->t.get() : nullptr, window_size};
 	return from_status(k->k->launch(a));
-}
-
-// ---- measurement aid: a plain copy kernel of known size (see kernels/copy_probe.hip)
-struct X17hCopyProbe { std::shared_ptr<HipDevice> dev; std::unique_ptr<HipKernel> k; size_t blocks; };
-
-int x17h_copy_probe_new(X17hDevice *dev, X17hCopyProbe **out) {
-	try {
-		Diagnostics diag;
-		auto built = kernel_build::build("copy_probe", "// copy probe\n", "copy_probe.hip", "copy_probe_meta.cpp", diag);
-		if (!built) return fail_diag("copy probe", diag);
-		auto meta = kernel_build::read_metadata_json(built->meta_json_path, diag);
-		if (!meta) return fail_diag("copy probe", diag);
-		auto p = std::make_unique<X17hCopyProbe>();
-		p->blocks = *kernel_build::meta_get(*meta, "BLOCKS");
-		if (dev != nullptr) {
-			p->k = kernel_build::load_kernel(*dev->dev->stream, built->code_object_path, "kernel", 0, diag);
-			if (!p->k) return fail_diag("copy probe", diag);
-			p->dev = dev->dev;
-		}
-		*out = p.release();
-		return 0;
-	} catch (std::exception const &e) { return fail(e.what()); }
-}
-void x17h_copy_probe_free(X17hCopyProbe *p) { delete p; }
-int x17h_copy_probe_launch(X17hCopyProbe *p, X17hTensor *src, X17hTensor *dst) {
-	if (!p->k) return fail("copy probe was built without a device");
-	if (src->t->bytes != dst->t->bytes || src->t->bytes % 16 != 0 || src->t->bytes / 16 > 0xFFFFFFFFull) return fail("copy probe needs equal sizes, multiple of 16 bytes");
-	void *s = src->t->ptr, *d = dst->t->ptr;
-	size_t n = src->t->bytes / 16;
-	void *args[3] = {&s, &n, &d};
-	size_t grid[3] = {p->blocks, 1, 1}, block[3] = {256, 1, 1};
-	return from_status(p->k->launch(*p->dev->stream, grid, block, 0, args));
-}
-
-// ---- measurement aid: a loop of nothing but matrix-core instructions (see kernels/mfma_probe.hip)
-struct X17hMfmaProbe { std::shared_ptr<HipDevice> dev; std::unique_ptr<HipKernel> k; size_t blocks, mfmas_per_iteration, ops_per_mfma; };
-
-int x17h_mfma_probe_new(X17hDevice *dev, int kind, X17hMfmaProbe **out) {
-	try {
-		if (kind < 0 || kind > 2) return fail("mfma probe kind: 0 int8, 1 e4m3, 2 f16");
-		Diagnostics diag;
-		std::string const name = "mfma_probe-kind" + std::to_string(kind);
-		auto built = kernel_build::build(name, "// matrix-core probe\n#define X17_PROBE_KIND " + std::to_string(kind) + "\n",
-		                                 "mfma_probe.hip", "mfma_probe_meta.cpp", diag);
-		if (!built) return fail_diag("mfma probe", diag);
-		auto meta = kernel_build::read_metadata_json(built->meta_json_path, diag);
-		if (!meta) return fail_diag("mfma probe", diag);
-		auto p = std::make_unique<X17hMfmaProbe>();
-		p->blocks = *kernel_build::meta_get(*meta, "BLOCKS");
-		p->mfmas_per_iteration = *kernel_build::meta_get(*meta, "MFMAS_PER_ITERATION");
-		p->ops_per_mfma = *kernel_build::meta_get(*meta, "OPS_PER_MFMA");
-		if (dev != nullptr) {
-			p->k = kernel_build::load_kernel(*dev->dev->stream, built->code_object_path, "kernel", 0, diag);
-			if (!p->k) return fail_diag("mfma probe", diag);
-			p->dev = dev->dev;
-		}
-		*out = p.release();
-		return 0;
-	} catch (std::exception const &e) { return fail(e.what()); }
-}
-void x17h_mfma_probe_free(X17hMfmaProbe *p) { delete p; }
-int x17h_mfma_probe_launch(X17hMfmaProbe *p, X17hTensor *operands, X17hTensor *out, size_t iterations, double *ops) {
-	if (!p->k) return fail("mfma probe was built without a device");
-	if (operands->t->bytes < 12 * 512 * 16) return fail("mfma probe needs 98304 bytes of operand data");
-	if (out->t->bytes < p->blocks * 512 * 4) return fail("mfma probe needs an output of 4 bytes per thread");
-	if (iterations > 0xFFFFFFFFull) return fail("mfma probe: too many iterations");
-	void *src = operands->t->ptr, *dst = out->t->ptr;
-	size_t n = iterations;
-	void *args[3] = {&src, &n, &dst};
-	size_t grid[3] = {p->blocks, 1, 1}, block[3] = {512, 1, 1};
-	if (ops != nullptr) {
-		*ops = double(p->blocks) * 8.0 * double(iterations) * double(p->mfmas_per_iteration) * double(p->ops_per_mfma);
-	}
-	return from_status(p->k->launch(*p->dev->stream, grid, block, 0, args));
 }
 
 } // extern "C"

@@ -183,6 +183,10 @@ namespace kernel_build {
 	std::optional<std::vector<std::pair<std::string, size_t>>> read_metadata_json(std::string const &path, Diagnostics &diag);
 	std::string kernels_dir();
 	std::string cache_dir();
+	std::optional<size_t> meta_get(std::vector<std::pair<std::string, size_t>> const &meta, char const *key);
+	// kernel_build.rs:161-198
+	std::unique_ptr<HipKernel> load_kernel(HipStream &stream, std::string const &code_object_path, char const *name,
+	                                       size_t smem_bytes, Diagnostics &diag);
 }
 
 // ---------------------------------------------------------------- GEMM (src/device/cuda/gemm.rs)
@@ -323,3 +327,7 @@ struct AttnDecodeKernel {
 };
 
 } // namespace x17
+
+// The handles of the flat C ABI (include/x17ai_host.h) that other libraries built on this layer take apart
+struct X17hDevice { std::shared_ptr<x17::HipDevice> dev; };
+struct X17hTensor { std::shared_ptr<x17::Tensor> t; };
