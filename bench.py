@@ -539,6 +539,45 @@ def single(dev, X, recipes, name, iters):
 		od = X.Tensor(dev, (S5, H * HD), X.INT8)
 		k = recipes.attn_decode_kernel(dev, H, HD, CAP, False)
 		fn, work, unit = (lambda: k.launch(qd, cache, lens, sk, sv, tp, od, None, W)), S5 * CAP * 2 * H * HD / 1e9, "GB/s of cache (rows with zero probability are not fetched)"
+	elif name == "decode_dense_config5":
+		# an all-zero query: every key scores the same, every 8-bit probability is 255, every K and V row is read
+		S5, CAP, H, HD, W = 64, 4096, 32, 128, 4096
+		one = _rand_codes(rng, (1, CAP, 2 * H * HD))
+		cache = X.Tensor.from_numpy(dev, np.ascontiguousarray(np.broadcast_to(one, (S5, CAP, 2 * H * HD))), X.INT8)
+		qd = X.Tensor.from_numpy(dev, np.zeros((S5, H * HD), np.int8), X.INT8)
+		lens = X.Tensor.from_numpy(dev, np.full(S5, CAP, np.uint32).view(np.float32), X.F32)
+		sk = X.Tensor.from_numpy(dev, _rand_codes(rng, (H, HD)), X.INT8)
+		sv = X.Tensor.from_numpy(dev, _rand_codes(rng, (H, HD)), X.INT8)
+		tp = X.Tensor.from_numpy(dev, np.ones(H, np.float32), X.F32)
+		od = X.Tensor(dev, (S5, H * HD), X.INT8)
+		k = recipes.attn_decode_kernel(dev, H, HD, CAP, False)
+		fn, work, unit = (lambda: k.launch(qd, cache, lens, sk, sv, tp, od, None, W)), S5 * CAP * 2 * H * HD / 1e9, "GB/s"
+	elif name in ("attn_kv_config4", "attn_qkv_config4", "ffn_f_config4", "attn_y_config4"):
+		M, H, HD = 32768, 16, 128
+		a = X.Tensor.from_numpy(dev, _rand_codes(rng, (M, D)), X.INT8)
+		if name == "attn_kv_config4":
+			b = X.Tensor.from_numpy(dev, _rand_codes(rng, (2 * H * HD, D)), X.INT8)
+			c, rr = X.Tensor(dev, (M, 2 * H * HD), X.INT8), X.Tensor(dev, (M, H), X.F32)
+			k = recipes.attn_kv_kernel(dev, D, 2 * H * HD, HD, False)
+			fn, work = (lambda: k.launch(a, b, c, rr)), k.n_ops(a, b) / 1e12
+		elif name == "attn_qkv_config4":
+			bq = X.Tensor.from_numpy(dev, _rand_codes(rng, (H * HD, D)), X.INT8)
+			b = X.Tensor.from_numpy(dev, _rand_codes(rng, (2 * H * HD, D)), X.INT8)
+			cq, c, rr = X.Tensor(dev, (M, H * HD), X.INT8), X.Tensor(dev, (M, 2 * H * HD), X.INT8), X.Tensor(dev, (M, H), X.F32)
+			k = recipes.attn_qkv_kernel(dev, D, H * HD, 2 * H * HD, HD, False)
+			fn, work = (lambda: k.launch_qkv(a, bq, b, cq, c, rr)), 2.0 * M * D * 3 * H * HD / 1e12
+		elif name == "ffn_f_config4":
+			b = X.Tensor.from_numpy(dev, _rand_codes(rng, (2 * F, D)), X.INT8)
+			c = X.Tensor(dev, (M, F), X.E4M3)
+			k = recipes.ffn_f_kernel(dev, D, 2 * F, False)
+			fn, work = (lambda: k.launch(a, b, c)), k.n_ops(a, b) / 1e12
+		else:
+			b = X.Tensor.from_numpy(dev, _rand_codes(rng, (2 * D, H * HD)), X.INT8)
+			r = X.Tensor.from_numpy(dev, _rand_codes(rng, (M, D)), X.INT8)
+			c = X.Tensor(dev, (M, D), X.E4M3)
+			k = recipes.attn_y_kernel(dev, D, H * HD, False)
+			fn, work = (lambda: k.launch(a, b, c, r)), k.n_ops(a, b) / 1e12
+		unit = "TOPS"
 	elif name == "rms_norm_config4":
 		rows = 32768
 		xb = X.Tensor.from_numpy(dev, (rng.standard_normal((rows, D), dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16), X.BF16)
@@ -552,7 +591,8 @@ def single(dev, X, recipes, name, iters):
 	                  "rate": work / med, "unit": unit}))
 
 
-ONLY_TARGETS = ("ffn_f_config2", "ffn_f_f8_config3", "ffn_y_f8_config4", "attn_config4", "attn_config5", "decode_config5", "rms_norm_config4")
+ONLY_TARGETS = ("ffn_f_config2", "ffn_f_f8_config3", "ffn_y_f8_config4", "attn_config4", "attn_config5", "decode_config5",
+                "decode_dense_config5", "attn_kv_config4", "attn_qkv_config4", "ffn_f_config4", "attn_y_config4", "rms_norm_config4")
 
 
 def main():
@@ -562,7 +602,9 @@ def main():
 	ap.add_argument("--warmup", type=int, default=10)
 	ap.add_argument("--no-extras", action="store_true")
 	ap.add_argument("--no-cpu", action="store_true")
-	ap.add_argument("--fused-qkv", action="store_true", help="headline block with the q and kv projections as one launch")
+	ap.add_argument("--separate-qkv", action="store_true",
+	                help="headline block with the q and kv projections as two launches, as src/main.rs launches them "
+	                     "(default: one launch that reads x once)")
 	ap.add_argument("--copy-probe", action="store_true",
 	                help="only run a 1 GiB device-to-device copy kernel (calibrates the HBM traffic counters)")
 	ap.add_argument("--mfma-probe", action="store_true",
@@ -602,7 +644,7 @@ def main():
 	if args.only:
 		single(dev, X, recipes, args.only, args.steps)
 		return
-	h = headline(dev, X, args.steps, args.warmup, args.fused_qkv)
+	h = headline(dev, X, args.steps, args.warmup, not args.separate_qkv)
 	value = h["rows"] * args.steps / h["wall_s"]
 	achieved = h["dominant_ops"] / h["dominant_mean_s"] / 1e12
 	traffic_file = "gemm_b8_ffn_y_f8_config4.txt"
