@@ -149,13 +149,13 @@ def headline(dev, X, steps, warmup, fused_qkv=False):
 
 
 def cpu_baseline():
-	"""The CPU oracle over a bounded sample of the config 4 block: the first 1024 tokens of one sequence through all
-	seven stages (attention: all 16 heads over those 1024 positions, window 512).  tokens / CPU seconds."""
+	"""The CPU oracle over a bounded sample of the config 4 block: the first 4096 tokens of one sequence through all
+	seven stages (attention: all 16 heads over those 4096 positions, window 512).  tokens / CPU seconds."""
 	from oracle import strict as S
 	from x17ai_amd import recipes
 	c = CONFIG4
 	D, H, HD, F, W = c["D"], c["H"], c["HD"], c["F"], c["W"]
-	n = 1024
+	n = 4096
 	inp = config4_inputs(np.random.default_rng(4000), n)
 	inp_scale = 1.0 / math.sqrt(D) / 64.0
 	t0 = time.perf_counter()
