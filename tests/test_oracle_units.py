@@ -196,6 +196,42 @@ def test_l2norm_epilogue_against_float64_and_order():
 	assert rrms[0, 0] == np.float32(want_scale)
 
 
+@pytest.mark.parametrize("hd", [32, 64, 128])
+def test_learned_scale_q_writer(hd):
+	"""cuda/qkvg_fwd_i8.cuh:145-219: L2 norm over every head of q, then a bf16 scale per column.  Pinned by (i) reduction to
+	the K halves of the L2-norm writer when every scale is 1 -- codes and rrms bit for bit --, (ii) the float64 closed form
+	q = x / sqrt(mean(x^2)) * scale on the FixedI8 grid, (iii) the scales being column-wise and applied AFTER the norm."""
+	m, n = 64, 512
+	acc = _acc(11 + hd, m, n)
+	ones = np.full(n, 0x3F80, np.uint16)                           # bf16 1.0
+	q1, r1 = S.epilogue_qnorm(acc, hd, 2.0 ** -70, 8.0, ones, want_rrms=True)
+	kvacc = np.zeros((m, 2 * n), np.int32)
+	kvacc.reshape(m, n // hd, 2, hd)[:, :, 0, :] = acc.reshape(m, n // hd, hd)
+	kv, rr = S.epilogue_l2norm(kvacc, hd, 2.0 ** -70, 1.0, 8.0)
+	assert np.array_equal(kv.reshape(m, n // hd, 2, hd)[:, :, 0, :], q1.reshape(m, n // hd, hd))
+	assert np.array_equal(rr.view(np.uint32), r1.view(np.uint32))
+	# float64 closed form with scales that differ per column (exactly representable in bf16: multiples of 1/64 in [0.5, 1.5))
+	rng = np.random.default_rng(5)
+	scale = (32 + rng.integers(0, 64, n)) / 64.0
+	dyn = (scale.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+	assert np.array_equal((dyn.astype(np.uint32) << 16).view(np.float32), scale.astype(np.float32))
+	got = S.epilogue_qnorm(acc, hd, 0.0, 8.0, dyn)
+	x = acc.astype(np.float64).reshape(m, n // hd, hd)
+	want = (x / np.sqrt((x * x).mean(-1, keepdims=True))).reshape(m, n) * scale * 8.0
+	want_codes = np.clip(np.rint(want), -127, 127)
+	d = np.abs(got.astype(np.float64) - want_codes)
+	assert d.max() <= 1 and np.mean(d > 0) < 1e-3
+	assert np.abs(got - want).max() <= 0.5 + 1e-3                  # each code within half a step of the exact value
+	# a rolled scale vector or scales applied per head instead of per column give another answer
+	assert not np.array_equal(S.epilogue_qnorm(acc, hd, 0.0, 8.0, np.roll(dyn, 1)), got)
+	per_head = np.repeat(dyn[::hd], hd)
+	assert not np.array_equal(S.epilogue_qnorm(acc, hd, 0.0, 8.0, per_head), got)
+	# eps only matters for an all-zero head: rsq(0) would be infinite, rsq(eps) * 0 is 0
+	z = acc.copy()
+	z[3, :hd] = 0
+	assert not S.epilogue_qnorm(z, hd, 2.0 ** -70, 8.0, dyn)[3, :hd].any()
+
+
 def test_gemm_f32_seq_against_float64():
 	r = _rng(11)
 	a = S.f32_to_e4m3((r.standard_normal((32, 512)) * 0.7).astype(np.float32))
