@@ -318,20 +318,49 @@ void kernel(
 
 		u32 const n_steps = kb_end - kb_begin;
 		if constexpr (!STRICT && !ROW_SCALES) {
-			// ---- speed build.  The same recurrence with the bookkeeping taken out of the key
-			// loop: a wave's steps fall into runs -- nothing to do, masked (the window's edge), fully visible, the
-			// diagonal, nothing to do -- and each run is its own loop; every step requests a tile (past the end the last
-			// one again, into a slot nobody reads any more), so the waits are constants; the tile requests take a
-			// scalar base and a lane offset; the 8-bit probabilities are rounded and turned into f16 by one addition
-			// and one byte shuffle per pair (PACK_MAGIC), the lift and the removal of the 1024 are one packed fma; the
-			// partial sums are kept at the scale of O (the maximum m_ref), so a moving maximum costs one exponential.
-			// O and the partial sums live at the scale of a reference maximum m_ref that is kept HEADROOM above the
-			// running maximum whenever it is set: the lift 2^(m - m_ref) of new probabilities then starts at 2^-12
-			// (8-bit integers times it are still exact f16 values) and O has to be brought down only after the
-			// maximum has grown by 17 (Gaussian scores move it by that much a few times per query block, not per tile).
-			constexpr f32 HEADROOM = 12.0f, LIFT0 = 1.0f / 4096.0f;
-			m_ref = m + HEADROOM;
+			// ---- speed build.  The same recurrence, rebuilt around what the kernel turned out to be bound by: the
+			// number of instructions of ANY kind a SIMD has to issue per step (scalar bookkeeping and waits count like
+			// vector arithmetic; with three wavefronts per SIMD an instruction costs 1.5-2.5 ns of SIMD time whatever it does).
+			//  * A wave's steps fall into runs -- nothing to do, masked (the window's edge), fully visible, the diagonal,
+			//    nothing to do -- and each run is its own loop.  Every step requests a tile (past the end the last one
+			//    again, into a slot nobody reads any more), so the waits are constants.
+			//  * The long run (fully visible steps) is unrolled over the four phases of the tile ring: every LDS address
+			//    is a register plus an immediate, and the ring arithmetic disappears from the scalar unit.
+			//  * The tile requests take a scalar base and a lane offset; M0 is set by one scalar addition.
+			//  * The 8-bit probabilities are rounded and turned into f16 by one fused multiply-add and one byte shuffle per
+			//    pair (PACK_MAGIC); the lift and the removal of the 1024 are one packed fma.
+			//  * O and the partial sums live at the scale of a reference maximum kept HEADROOM above the running one
+			//    whenever it is set: the lift of new probabilities then starts at 2^-12 (8-bit integers times it are still
+			//    exact f16 values), a moving maximum costs one exponential, and O has to be brought down only after the
+			//    maximum has grown by 17 (Gaussian scores move it by that much a few times per query block, not per tile).
+			//  * The score accumulators start at the bits of 1.5 * 2^23 instead of zero: the int32 sum 0x4B400000 + dot,
+			//    read as a float, is 12582912 + dot exactly (|dot| < 2^22), so no score is ever converted.  What refers to
+			//    a maximum lives in that biased domain: `ext` is the running extreme of sgn * (12582912 + dot) (exact) and
+			//    `mb` the subtrahend of the exponent, ext * |temperature| - lg2 255 rounded to a float.  That rounding (an
+			//    ulp of 12582912 * temperature) would move the maximum the probabilities are rounded against; its exact
+			//    remainder is therefore taken and 2^-remainder (`fine`) multiplies every probability inside operations that
+			//    are needed anyway (the rounding addition is the fused multiply-add above, the sums' lift carries it).
+			//  * The row maximum of a tile needs the partner lane's eight keys only when it moves: both lanes hold the same
+			//    `ext`, and the tile's maximum exceeds it exactly when one of the two halves does.
+			constexpr f32 HEADROOM = 12.0f, LIFT0 = 1.0f / 4096.0f, DOT_BIAS = 12582912.0f;
+			v16i s_bias;
+			X17_UNROLL for (int r = 0; r < 16; ++r) s_bias[r] = 0x4B400000;
+			asm volatile("" : "+v"(s_bias));          // (kept in registers: rebuilding it per step would cost what it saves)
+			f32 const abs_t = __builtin_fabsf(temperature);
+			f32 const sgn = positive_temperature ? 1.0f : -1.0f;
+			f32 ext = (f32(sink_dot) + DOT_BIAS) * sgn;
+			f32 mb, fine;
+			auto set_subtrahend = [&]() {
+				// ext * |t| as a rounded product and its exact remainder; prod - mb is exact (neighbouring floats)
+				f32 const prod = ext * abs_t;
+				f32 const low = fmaf32(ext, abs_t, -prod);
+				mb = prod - LOG2_PROB_SCALE;
+				fine = hw::ex2(-(((prod - mb) - LOG2_PROB_SCALE) + low));          // 2^-(what mb leaves over): close to 1
+			};
+			set_subtrahend();
+			f32 ext_ref = ext;                        // O and the sums refer to the maximum HEADROOM above this extreme's score
 			lift = LIFT0;
+			f32 sum_lift = LIFT0 * fine;
 			lift2 = v2h{(_Float16)LIFT0, (_Float16)LIFT0};
 			v2h neg_bias2 = {(_Float16)(-1024.0f * LIFT0), (_Float16)(-1024.0f * LIFT0)};      // -1024 * lift2
 			sum_lo = sum_lo * LIFT0;
@@ -344,31 +373,48 @@ void kernel(
 			// first block that lies inside the window of all 32 queries: q_wave0 + 31 - 32 kb <= wr
 			u32 const inside_kb = q_wave0 + 31 > wr ? (q_wave0 + 62 - wr) / 32 : 0;
 			u32 const inside_clamped = inside_kb < wave_kb_first ? wave_kb_first : (inside_kb > wave_kb_last ? wave_kb_last : inside_kb);
-			// (the fully visible steps take the row maximum over the integer dots, which needs a positive temperature;
-			// with any other temperature every step goes the way of the masked ones, which compare the scaled scores)
+			// (the fully visible steps take the row maximum over the scores' bits, which needs a positive temperature;
+			// with any other temperature every step goes the way of the masked ones)
 			u32 const first_full = (positive_temperature ? inside_clamped : wave_kb_last) - kb_begin;
 
+			// SLOT: the step's position in the tile ring (step % RING) as a compile-time number, or -1 for "compute it"
 			i8 const *load_src = kv_head + (size_t)(kb_begin * at::KV_PER_STEP) * KV_STRIDE;
-			u32 next_step = 0;
-			auto request_tiles = [&]() {
-				u32 const slot = next_step % at::RING;
+			u32 steps_requested = 0;
+			u32 const lds_wave = (u32)(size_t)X17_LDS_PTR(smem) + stage_lds;
+			auto request_tiles = [&]<int SLOT>(u32 step) __attribute__((always_inline)) {
 				if (CPR == 8 || stager) {
-					load_to_lds_16(smem + at::K_RING_OFFSET + slot * at::K_TILE_BYTES + stage_lds, load_src, stage_k_src);
-					load_to_lds_16(smem + at::RAW_V_RING_OFFSET + slot * at::RAW_V_TILE_BYTES + stage_lds, load_src, stage_v_src);
+					if constexpr (SLOT >= 0) {
+						asm volatile("s_add_i32 m0, %0, %1\n\tglobal_load_lds_dwordx4 %2, %3"
+						             :: "s"(lds_wave), "i"(at::K_RING_OFFSET + SLOT * at::K_TILE_BYTES), "v"(stage_k_src), "s"(load_src) : "memory", "m0", "scc");
+						asm volatile("s_add_i32 m0, %0, %1\n\tglobal_load_lds_dwordx4 %2, %3"
+						             :: "s"(lds_wave), "i"(at::RAW_V_RING_OFFSET + SLOT * at::RAW_V_TILE_BYTES), "v"(stage_v_src), "s"(load_src) : "memory", "m0", "scc");
+					} else {
+						u32 const slot = step % at::RING;
+						load_to_lds_16(smem + at::K_RING_OFFSET + slot * at::K_TILE_BYTES + stage_lds, load_src, stage_k_src);
+						load_to_lds_16(smem + at::RAW_V_RING_OFFSET + slot * at::RAW_V_TILE_BYTES + stage_lds, load_src, stage_v_src);
+					}
 				}
-				++next_step;
-				if (next_step < n_steps) {
+				++steps_requested;
+				if (steps_requested < n_steps) {
 					load_src += (size_t)at::KV_PER_STEP * KV_STRIDE;
 				}
 			};
 			// K tile i and raw V tile i + 1 have landed once at most the two requests of step i + 2 are in flight
-			auto stage = [&](u32 i) {
+			auto stage = [&]<int SLOT>(u32 i) __attribute__((always_inline)) {
 				__builtin_amdgcn_s_waitcnt(0x0F72);          // vmcnt(2)
 				__builtin_amdgcn_s_waitcnt(0xC07F);          // lgkmcnt(0): own LDS traffic of step i-1 is complete
 				__builtin_amdgcn_s_barrier();                // ... and so is everybody else's: tiles i are visible
-				request_tiles();                             // step i + 3 into the slot step i - 1 used
+				constexpr int NEXT_SLOT = SLOT < 0 ? -1 : (SLOT + (int)at::PREFETCH) % (int)at::RING;
+				request_tiles.template operator()<NEXT_SLOT>(i + at::PREFETCH);      // into the slot step i - 1 used
 			};
-			auto widen_next = [&](u32 i) { widen_v((i + 1) % at::RING, (i + 1) & 1); };
+			// raw V tile of step i + 1 -> f16 tile (i + 1) % 2
+			auto widen_next = [&]<int SLOT>(u32 i) __attribute__((always_inline)) {
+				if constexpr (SLOT >= 0) {
+					widen_v((SLOT + 1) % at::RING, (SLOT + 1) & 1);
+				} else {
+					widen_v((i + 1) % at::RING, (i + 1) & 1);
+				}
+			};
 			// maximum of a lane pair's two values, in both lanes
 			auto pair_max_i32 = [](i32 x) {
 				auto const r = __builtin_amdgcn_permlane32_swap((u32)x, (u32)x, false, false);
@@ -389,40 +435,54 @@ void kernel(
 					v_lane_off8[db] = v_granule_offset(8 + 4 * half + (t >> 2), 2 * db + dh) + 8 * (t & 3);
 				}
 			}
-			auto compute = [&]<bool MASKED>(u32 i) __attribute__((always_inline)) {
-				u32 const kb = kb_begin + i;
-				u8 const *k_tile = smem + at::K_RING_OFFSET + (i % at::RING) * at::K_TILE_BYTES;
-				u8 const *v_tile = smem + at::V_TILES_OFFSET + (i & 1) * at::V_TILE_BYTES;
-				v16i s_acc = {0};
+			u32 k_lane_off[K_SLICES];
+			X17_UNROLL for (u32 sl = 0; sl < K_SLICES; ++sl) k_lane_off[sl] = k_chunk_offset(qlane, 2 * sl + half);
+
+			auto compute = [&]<bool MASKED, int SLOT>(u32 i) __attribute__((always_inline)) {
+				u32 const k_slot = SLOT >= 0 ? (u32)SLOT : i % at::RING;
+				u32 const v_slot = SLOT >= 0 ? (u32)SLOT & 1u : i & 1u;
+				u8 const *k_tile = smem + at::K_RING_OFFSET + k_slot * at::K_TILE_BYTES;
+				u8 const *v_tile = smem + at::V_TILES_OFFSET + v_slot * at::V_TILE_BYTES;
+				v16i s_acc = s_bias;
 				X17_UNROLL for (u32 sl = 0; sl < K_SLICES; ++sl) {
-					v4i kf = *reinterpret_cast<v4i const *>(k_tile + k_chunk_offset(qlane, 2 * sl + half));
+					v4i kf = *reinterpret_cast<v4i const *>(k_tile + k_lane_off[sl]);
 					s_acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[sl], s_acc, 0, 0, 0);
 				}
-				widen_next(i);                                // (behind the matrix instructions, whose results are not ready yet)
-				u32 const key0 = kb * at::KV_PER_STEP;
+				widen_next.template operator()<SLOT>(i);      // (behind the matrix instructions, whose results are not ready yet)
 				X17_UNROLL for (u32 tile = 0; tile < 2; ++tile) {
-					f32 sc[8];
+					f32 y[8];
+					[[maybe_unused]] bool vis[8];
 					f32 tmax;
 					if constexpr (!MASKED) {
-						// the row maximum over the integer dots (the scaling is monotone), scaled once
+						// (positive temperature: sgn = 1; the biased scores are positive floats: their order is the order
+						// of their bits as integers)
+						X17_UNROLL for (u32 r = 0; r < 8; ++r) y[r] = u2f((u32)s_acc[8 * tile + r]);
 						i32 const *a = reinterpret_cast<i32 const *>(&s_acc) + 8 * tile;
 						auto mx = [](i32 x, i32 y) { return x > y ? x : y; };
 						i32 const imax = mx(mx(mx(mx(mx(mx(mx(a[0], a[1]), a[2]), a[3]), a[4]), a[5]), a[6]), a[7]);     // four max3-type operations
-						tmax = f32(pair_max_i32(imax)) * temperature;
+						tmax = u2f((u32)imax);
 					} else {
-						X17_UNROLL for (u32 r = 0; r < 8; ++r) sc[r] = f32(s_acc[8 * tile + r]) * temperature;
+						u32 const key0 = (kb_begin + i) * at::KV_PER_STEP;
 						u32 const first = qi - 1 - (key0 + 16 * tile + 4 * half);
+						f32 ym[8];
 						X17_UNROLL for (u32 r = 0; r < 8; ++r) {
 							u32 const distance = first - (8 * (r / 4) + (r % 4));
-							sc[r] = distance <= vis_bound ? sc[r] : -__builtin_inff();
+							vis[r] = distance <= vis_bound;
+							y[r] = u2f((u32)s_acc[8 * tile + r]) * sgn;
+							ym[r] = vis[r] ? y[r] : -__builtin_inff();
 						}
-						f32 const lmax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fmaxf(sc[0], sc[1]), __builtin_fmaxf(sc[2], sc[3])),
-						                                 __builtin_fmaxf(__builtin_fmaxf(sc[4], sc[5]), __builtin_fmaxf(sc[6], sc[7])));
-						tmax = __builtin_fmaxf(lmax, partner_f32(lmax, half));
+						tmax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fmaxf(ym[0], ym[1]), __builtin_fmaxf(ym[2], ym[3])),
+						                       __builtin_fmaxf(__builtin_fmaxf(ym[4], ym[5]), __builtin_fmaxf(ym[6], ym[7])));
 					}
-					if (__any(tmax > m)) {
-						m = tmax > m ? tmax : m;
-						lift = hw::ex2(m - m_ref);
+					if (__any(tmax > ext)) {
+						if constexpr (!MASKED) {
+							tmax = u2f((u32)pair_max_i32((i32)f2u(tmax)));
+						} else {
+							tmax = __builtin_fmaxf(tmax, partner_f32(tmax, half));
+						}
+						ext = tmax > ext ? tmax : ext;
+						set_subtrahend();
+						lift = hw::ex2(fmaf32(ext - ext_ref, abs_t, -HEADROOM));      // (the difference is exact)
 						if (__any(lift > MAX_LIFT)) {
 							// O and the partial sums come down to the scale of the new maximum
 							f32 const down = hw::rcp(lift) * LIFT0;
@@ -431,24 +491,27 @@ void kernel(
 							}
 							sum_lo = sum_lo * down;
 							sum_hi = sum_hi * down;
-							m_ref = m + HEADROOM;
+							ext_ref = ext;
 							lift = LIFT0;
 						}
 						lift2 = v2h{(_Float16)lift, (_Float16)lift};      // round to nearest
 						neg_bias2 = lift2 * v2h{(_Float16)-1024.0f, (_Float16)-1024.0f};     // exact
+						sum_lift = lift * fine;
 					}
-					f32 const shift = m - LOG2_PROB_SCALE;        // 255 * 2^(s - m) = 2^(s - (m - lg2 255))
 					f32 p[8];
-					if constexpr (!MASKED) {
-						X17_UNROLL for (u32 r = 0; r < 8; ++r) p[r] = hw::ex2(fmaf32(f32(s_acc[8 * tile + r]), temperature, -shift));
-					} else {
-						X17_UNROLL for (u32 r = 0; r < 8; ++r) p[r] = hw::ex2(sc[r] - shift);
+					X17_UNROLL for (u32 r = 0; r < 8; ++r) {
+						f32 const arg = fmaf32(y[r], abs_t, -mb);       // lg2 of 255 * 2^(score - maximum)
+						if constexpr (!MASKED) {
+							p[r] = hw::ex2(arg);
+						} else {
+							p[r] = hw::ex2(vis[r] ? arg : -__builtin_inff());
+						}
 					}
-					sum_lo = fmaf32((p[0] + p[1]) + (p[2] + p[3]), lift, sum_lo);
-					sum_hi = fmaf32((p[4] + p[5]) + (p[6] + p[7]), lift, sum_hi);
+					sum_lo = fmaf32((p[0] + p[1]) + (p[2] + p[3]), sum_lift, sum_lo);
+					sum_hi = fmaf32((p[4] + p[5]) + (p[6] + p[7]), sum_lift, sum_hi);
 					v4u pp;
 					X17_UNROLL for (int w = 0; w < 4; ++w) {
-						u32 const lo16 = f2u(p[2 * w] + PACK_MAGIC), hi16 = f2u(p[2 * w + 1] + PACK_MAGIC);
+						u32 const lo16 = f2u(fmaf32(p[2 * w], fine, PACK_MAGIC)), hi16 = f2u(fmaf32(p[2 * w + 1], fine, PACK_MAGIC));
 						u32 const pair = __builtin_amdgcn_perm(hi16, lo16, 0x05040100u);           // f16 (1024 + P) twice
 						pp[w] = __builtin_bit_cast(u32, __builtin_elementwise_fma(__builtin_bit_cast(v2h, pair), lift2, neg_bias2));
 					}
@@ -465,33 +528,38 @@ void kernel(
 					}
 				}
 			};
+			auto step = [&]<bool MASKED, int SLOT>(u32 i) __attribute__((always_inline)) {
+				stage.template operator()<SLOT>(i);
+				compute.template operator()<MASKED, SLOT>(i);
+			};
+			auto idle_step = [&](u32 i) __attribute__((always_inline)) {
+				stage.template operator()<-1>(i);
+				widen_next.template operator()<-1>(i);
+			};
 
 			__syncthreads();                      // previous head's tiles are no longer read
-			X17_UNROLL for (u32 j = 0; j < at::PREFETCH; ++j) request_tiles();
+			X17_UNROLL for (u32 j = 0; j < at::PREFETCH; ++j) request_tiles.template operator()<-1>(j);
 			__builtin_amdgcn_s_waitcnt(0x0F74);   // vmcnt(4): step 0 has landed
 			widen_v(0, 0);
 			u32 i = 0;
-			for (; i < first_active; ++i) {
-				stage(i);
-				widen_next(i);
+			for (; i < first_active; ++i) idle_step(i);
+			for (; i < first_full; ++i) step.template operator()<true, -1>(i);
+			// the fully visible run: single steps up to a multiple of the ring, whole rings, single steps again
+			for (; i < diagonal && i % at::RING != 0; ++i) step.template operator()<false, -1>(i);
+			static_assert(at::RING == 4, "the run below is written out for a ring of four");
+			for (; i + at::RING <= diagonal; i += at::RING) {
+				step.template operator()<false, 0>(i);
+				step.template operator()<false, 1>(i + 1);
+				step.template operator()<false, 2>(i + 2);
+				step.template operator()<false, 3>(i + 3);
 			}
-			for (; i < first_full; ++i) {
-				stage(i);
-				compute.template operator()<true>(i);
-			}
-			for (; i < diagonal; ++i) {
-				stage(i);
-				compute.template operator()<false>(i);
-			}
-			stage(i);
-			compute.template operator()<true>(i);
-			for (++i; i < n_steps; ++i) {
-				stage(i);
-				widen_next(i);
-			}
+			for (; i < diagonal; ++i) step.template operator()<false, -1>(i);
+			step.template operator()<true, -1>(i);
+			for (++i; i < n_steps; ++i) idle_step(i);
 			__builtin_amdgcn_s_waitcnt(0x0F70);   // the last requests write LDS: they land before the tiles are reused
-			// the partial sums are at the scale of m_ref: the common ending below takes them as if that were the maximum
-			m = m_ref;
+			// the partial sums are at the scale of the maximum HEADROOM above ext_ref's score: the common ending below
+			// takes them as if that were the maximum (sgn * ext_ref - 12582912 is that extreme's dot product, exactly)
+			m = fmaf32(fmaf32(ext_ref, sgn, -DOT_BIAS), temperature, HEADROOM);
 			lift = 1.0f;
 		} else {
 		// ---- pipeline prologue

@@ -50,6 +50,22 @@ using namespace x17;
 #define X17_OP "v_permlane32_swap_b32 %0, %0"
 #elif X17_PROBE_OP == 19
 #define X17_OP "s_add_u32 %1, %1, 3"
+#elif X17_PROBE_OP == 20
+#define X17_OP "v_lshl_add_u32 %0, %0, 16, %0"
+#elif X17_PROBE_OP == 21
+#define X17_OP "v_add3_u32 %0, %0, %0, %0"
+#elif X17_PROBE_OP == 22
+#define X17_OP "v_pack_b32_f16 %0, %0, %0"
+#elif X17_PROBE_OP == 23
+#define X17_OP "v_and_or_b32 %0, %0, %0, %0"
+#elif X17_PROBE_OP == 24
+#define X17_OP "v_cndmask_b32 %0, %0, %0, vcc"
+#elif X17_PROBE_OP == 25
+#define X17_OP "v_cmp_lt_f32 vcc, %0, %0"
+#elif X17_PROBE_OP == 26
+#define X17_OP "v_fmaak_f32 %0, %0, %0, 0x4b406400"
+#elif X17_PROBE_OP == 27
+#define X17_OP "v_mov_b32 %0, %0"
 #else
 #error "unknown X17_PROBE_OP"
 #endif
@@ -60,7 +76,7 @@ void kernel(f32 const *src, u32 iterations, f32 *out) {
 	X17_UNROLL for (int i = 0; i < 16; ++i) r[i] = src[threadIdx.x + i];
 	u32 s = iterations;
 	for (u32 it = 0; it < iterations; ++it) {
-		X17_UNROLL for (int i = 0; i < 16; ++i) asm volatile(X17_OP : "+v"(r[i]), "+s"(s) : : "scc");
+		X17_UNROLL for (int i = 0; i < 16; ++i) asm volatile(X17_OP : "+v"(r[i]), "+s"(s) : : "scc", "vcc");
 	}
 	f32 sum = f32(s);
 	X17_UNROLL for (int i = 0; i < 16; ++i) sum += r[i];

@@ -40,7 +40,8 @@ namespace {
 	char const *const VALU_OPS[] = {
 		"v_fma_f32", "v_add_f32", "v_mul_f32", "v_xor_b32", "v_add_u32", "v_cvt_f32_i32", "v_rndne_f32", "v_max_f32", "v_max3_i32",
 		"v_perm_b32", "v_cvt_pkrtz_f16_f32", "v_pk_mul_f16", "v_pk_fma_f16", "v_pk_add_f16", "v_med3_f32", "v_exp_f32", "v_rcp_f32",
-		"v_log_f32", "v_permlane32_swap_b32", "s_add_u32",
+		"v_log_f32", "v_permlane32_swap_b32", "s_add_u32", "v_lshl_add_u32", "v_add3_u32", "v_pack_b32_f16", "v_and_or_b32",
+		"v_cndmask_b32", "v_cmp_lt_f32", "v_fmaak_f32", "v_mov_b32",
 	};
 	constexpr int N_VALU_OPS = int(sizeof VALU_OPS / sizeof VALU_OPS[0]);
 }
