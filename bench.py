@@ -276,7 +276,9 @@ def mfma_probe(dev, X):
 
 def valu_probe(dev, X):
 	"""Issue rate of single vector instructions, in nanoseconds of SIMD time per wavefront-instruction, with 1, 2, 3,
-	4 and 8 wavefronts on every SIMD of the chip."""
+	4 and 8 wavefronts on every SIMD of the chip.  Entries named "group: ..." are composite loops without memory
+	traffic -- a matrix instruction next to vector instructions, and the instruction mix of one 32-key step of the
+	attention speed build -- and give nanoseconds of SIMD time per group."""
 	from x17ai_amd.probes import ValuProbe, valu_probe_ops
 	src = X.Tensor.from_numpy(dev, np.zeros(256, np.float32), X.F32)
 	out = X.Tensor(dev, (1024 * 8 * 64,), X.F32)

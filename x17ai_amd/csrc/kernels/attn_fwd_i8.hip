@@ -301,9 +301,10 @@ void kernel(
 		v16f o_acc[D_BLOCKS];                // O^T: lane = query, register r = dim 32*db + 8*(r/4) + 4*half + r%4
 		X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
 			X17_UNROLL for (int r4 = 0; r4 < 4; ++r4) {
-				u32 word = *reinterpret_cast<u32 const *>(sink_v + (size_t)head * HD + 32 * db + 8 * r4 + 4 * half);
+				// 255 * v for the int8 byte v, through the unsigned byte v + 128 (one conversion and one fma per value, all exact)
+				u32 const word = *reinterpret_cast<u32 const *>(sink_v + (size_t)head * HD + 32 * db + 8 * r4 + 4 * half) ^ 0x80808080u;
 				X17_UNROLL for (int b = 0; b < 4; ++b) {
-					o_acc[db][4 * r4 + b] = f32((i32)(i8)((word >> (8 * b)) & 0xFFu) * 255);
+					o_acc[db][4 * r4 + b] = fmaf32(f32((word >> (8 * b)) & 0xFFu), 255.0f, -32640.0f);
 				}
 			}
 		}
@@ -748,9 +749,9 @@ void kernel(
 		f32 s3 = half == 0 ? other_hi : sum_hi;
 		f32 total = (s0 + s1) + (s2 + s3);
 		if (l_out != nullptr && half == 0) {
-			l_out[(size_t)head * ((size_t)gridDim.z * seq_len) + row_base + qi] = strict::lg2(total) + m;
+			l_out[(size_t)head * ((size_t)gridDim.z * seq_len) + row_base + qi] = sfu::lg2(total) + m;
 		}
-		f32 inv = strict::rcp(total);
+		f32 inv = sfu::rcp(total);
 		if constexpr (!STRICT) {
 			inv = inv * sfu::rcp(lift);
 		}
@@ -778,8 +779,19 @@ void kernel(
 			// word g of this lane = dims 32*db + 8*g + 4*half .. +3
 			u32 word[4];
 			X17_UNROLL for (int g = 0; g < 4; ++g) {
-				word[g] = pack4_fixedi8(o_acc[db][4 * g] * inv, o_acc[db][4 * g + 1] * inv,
-				                        o_acc[db][4 * g + 2] * inv, o_acc[db][4 * g + 3] * inv);
+				if constexpr (STRICT) {
+					word[g] = pack4_fixedi8(o_acc[db][4 * g] * inv, o_acc[db][4 * g + 1] * inv,
+					                        o_acc[db][4 * g + 2] * inv, o_acc[db][4 * g + 3] * inv);
+				} else {
+					// the scaling rides in the rounding addition; clamping the rounded value gives what rounding the
+					// clamped one gives
+					constexpr f32 MAGIC = 12582912.0f;
+					u32 u[4];
+					X17_UNROLL for (int e = 0; e < 4; ++e) {
+						u[e] = f2u(__builtin_amdgcn_fmed3f(fmaf32(o_acc[db][4 * g + e], inv, MAGIC), MAGIC - 127.0f, MAGIC + 127.0f));
+					}
+					word[g] = __builtin_amdgcn_perm(u[1], u[0], 0x0c0c0400u) | __builtin_amdgcn_perm(u[3], u[2], 0x04000c0cu);
+				}
 			}
 			// The lane pair (lane, lane + 32) holds the 32 bytes of this block interleaved word by word; two
 			// cross-half swaps give the lower lane bytes 0..15 and the upper lane bytes 16..31, so that each

@@ -37,12 +37,18 @@ namespace {
 	}
 	size_t meta(Built const &b, char const *key) { auto v = kernel_build::meta_get(b.meta, key); return v ? *v : size_t(0); }
 
+	// entries 0..27 are single instructions (X17_PROBE_OP = the index), the rest composite loops (X17_PROBE_OP = 100 + ...)
 	char const *const VALU_OPS[] = {
 		"v_fma_f32", "v_add_f32", "v_mul_f32", "v_xor_b32", "v_add_u32", "v_cvt_f32_i32", "v_rndne_f32", "v_max_f32", "v_max3_i32",
 		"v_perm_b32", "v_cvt_pkrtz_f16_f32", "v_pk_mul_f16", "v_pk_fma_f16", "v_pk_add_f16", "v_med3_f32", "v_exp_f32", "v_rcp_f32",
 		"v_log_f32", "v_permlane32_swap_b32", "s_add_u32", "v_lshl_add_u32", "v_add3_u32", "v_pack_b32_f16", "v_and_or_b32",
 		"v_cndmask_b32", "v_cmp_lt_f32", "v_fmaak_f32", "v_mov_b32",
+		"group: f16 mfma 32x32x16 (4 accumulators)", "group: i8 mfma 32x32x32 + 8 v_fma_f32", "group: i8 mfma 32x32x32 + 8 v_perm_b32",
+		"group: i8 mfma 32x32x32 + 8 v_exp_f32", "group: i8 mfma 32x32x32 (dependent chain)",
+		"group: attention step, vector + matrix instructions", "group: attention step, all instructions",
 	};
+	constexpr int N_SINGLE_OPS = 28;
+	int probe_op_code(int index) { return index < N_SINGLE_OPS ? index : 100 + (index - N_SINGLE_OPS); }
 	constexpr int N_VALU_OPS = int(sizeof VALU_OPS / sizeof VALU_OPS[0]);
 }
 
@@ -108,7 +114,7 @@ int x17p_valu_probe_new(X17hDevice *dev, int op, X17pValuProbe **out) {
 	try {
 		if (op < 0 || op >= N_VALU_OPS) return fail("valu probe: unknown instruction index");
 		auto p = std::make_unique<X17pValuProbe>();
-		if (!build(dev, "valu_probe-op" + std::to_string(op), std::string("// vector-issue probe: ") + VALU_OPS[op] + "\n#define X17_PROBE_OP " + std::to_string(op) + "\n",
+		if (!build(dev, "valu_probe-op" + std::to_string(probe_op_code(op)), std::string("// issue probe: ") + VALU_OPS[op] + "\n#define X17_PROBE_OP " + std::to_string(probe_op_code(op)) + "\n",
 		           "valu_probe.hip", "valu_probe_meta.cpp", "valu probe", p->b)) return 1;
 		if (dev != nullptr) p->dev = dev->dev;
 		*out = p.release();

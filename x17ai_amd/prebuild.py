@@ -94,7 +94,7 @@ def _specs():
 	add(("copy_probe",))
 	for kind in (0, 1, 2):
 		add(("mfma_probe", kind))
-	for op in range(28):
+	for op in range(35):
 		add(("valu_probe", op))
 	# ---- tests/test_gpu_fullsize.py (the strict ffn pair, attention and decode kernels are listed above)
 	add(("attn", 16, 128, True))
