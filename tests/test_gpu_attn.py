@@ -65,7 +65,7 @@ def test_attn_strict_bit_exact(dev, t, h, hd, w):
 	assert np.array_equal(got_l.view(np.uint32), want_l.view(np.uint32))
 
 
-@pytest.mark.parametrize("t,h,hd,w", [(512, 2, 64, 128), (640, 2, 128, 256), (1024, 8, 64, 256)])
+@pytest.mark.parametrize("t,h,hd,w", [(512, 2, 64, 128), (640, 2, 128, 256), (1024, 8, 64, 256), (1536, 4, 32, 512), (1024, 2, 128, 0)])
 def test_attn_fast_within_one_code(dev, t, h, hd, w):
 	rng = rng_for("attn", t, h, hd, w)
 	q, kv, sk, sv, temp = _attn_inputs(rng, t, h, hd)
@@ -139,6 +139,32 @@ def test_attn_special_cases(dev):
 	assert np.all(np.abs(got_r.astype(np.int32) - 40) <= 1)
 	want_r, _ = S.attn_fwd_i8(q, kv2.reshape(t, -1), sk, sv2, temp, h, hd, 64)
 	assert np.array_equal(got_r, want_r)
+
+
+def test_attn_fast_temperature_signs_and_closed_forms(dev):
+	"""The speed build takes the row maximum over the scores' bits on fully visible tiles, which needs a positive head
+	temperature; heads with a negative or zero temperature go through its masked path instead.  All three kinds of
+	head in one launch against the oracle, and the closed forms: query 0 sees only the sink, constant V comes back
+	exactly when every probability is 255 (q = 0, or temperature 0)."""
+	t, h, hd, w = 768, 4, 64, 256
+	rng = rng_for("attn-fast-signs")
+	q, kv, sk, sv, _ = _attn_inputs(rng, t, h, hd)
+	temp = np.array([0.8, -0.6, 0.0, 1.3], np.float32)
+	kern = recipes.attn_kernel(dev, h, hd, False)
+	got, got_l = _run_attn(dev, kern, q, kv, sk, sv, temp, w)
+	want, want_l = S.attn_fwd_i8(q, kv, sk, sv, temp, h, hd, w)
+	d = np.abs(got.astype(np.int32) - want.astype(np.int32))
+	assert d.max() <= 1 and np.mean(d > 0) < 0.02, (d.max(), np.mean(d > 0))
+	assert np.max(np.abs(got_l - want_l)) < 1e-4
+	assert np.array_equal(got[0].reshape(h, hd), sv)
+	kv2 = kv.reshape(t, h, 2, hd).copy()
+	kv2[:, :, 1, :] = 40
+	sv2 = np.full_like(sv, 40)
+	got_c, _ = _run_attn(dev, kern, np.zeros_like(q), kv2.reshape(t, -1), sk, sv2, temp, w)
+	assert np.all(got_c == 40)
+	got_z, _ = _run_attn(dev, kern, q, kv2.reshape(t, -1), sk, sv2, temp, w)
+	assert np.all(got_z.reshape(t, h, hd)[:, 2, :] == 40)          # the head with temperature 0
+	assert np.all(np.abs(got_z.astype(np.int32) - 40) <= 1)
 
 
 def test_attn_launch_rejects_bad_arguments(dev):

@@ -56,7 +56,7 @@ def _specs():
 	# ---- tests/test_gpu_attn.py
 	for h, hd in ((4, 32), (2, 64), (2, 128), (8, 64)):
 		add(("attn", h, hd, True))
-	for h, hd in ((2, 64), (2, 128), (8, 64)):
+	for h, hd in ((2, 64), (2, 128), (8, 64), (4, 32), (4, 64)):
 		add(("attn", h, hd, False))
 	for h, hd, out in ((8, 64, BF16), (4, 32, BF16), (2, 128, BF16), (2, 64, INT8), (2, 64, BF16)):
 		add(("attn_rows", h, hd, out, True))
