@@ -123,8 +123,10 @@ X17_DEV u32 pack_f16(f32 lo, f32 hi) {
 // global source = a uniform 64-bit base in scalar registers + a 32-bit offset per lane (the compiler's own selection
 // forms a 64-bit address per lane with a 64-bit vector add in front of every load).
 X17_DEV void load_to_lds_16(u8 *lds_uniform, i8 const *src_uniform, u32 lane_offset) {
+	// (the address is the same in every lane; reading it from the first one tells the compiler so)
+	u32 const lds = __builtin_amdgcn_readfirstlane((u32)(size_t)X17_LDS_PTR(lds_uniform));
 	asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
-	             :: "s"((u32)(size_t)X17_LDS_PTR(lds_uniform)), "v"(lane_offset), "s"(src_uniform) : "memory", "m0");
+	             :: "s"(lds), "v"(lane_offset), "s"(src_uniform) : "memory", "m0");
 }
 
 // Speed build: p + PACK_MAGIC rounds p in [0, 256) to the nearest integer P (ties to even, as rintf) and leaves
@@ -378,35 +380,44 @@ void kernel(
 			// with any other temperature every step goes the way of the masked ones)
 			u32 const first_full = (positive_temperature ? inside_clamped : wave_kb_last) - kb_begin;
 
-			// SLOT: the step's position in the tile ring (step % RING) as a compile-time number, or -1 for "compute it"
-			i8 const *load_src = kv_head + (size_t)(kb_begin * at::KV_PER_STEP) * KV_STRIDE;
-			u32 steps_requested = 0;
+			// Tile requests.  Step s asks for K tile s + 3 and raw V tile s + 4, into the ring slots that K tile s - 1 and raw
+			// V tile s have just left (a V tile is widened -- by the thread that fetched it -- during the step before its
+			// use, so its slot is free one step earlier than a K slot): both tiles are on their way for three whole steps
+			// before anything waits for them.  The requests of a thread complete in the order V0, (K0, V1), (K1, V2), ...;
+			// step s needs the pair (K s, V s + 1), which leaves the two pairs behind it in flight.
+			// `src` is the address of tile min(s + 3, last) when step s makes its requests; V tile s + 4 is one tile further
+			// through a second lane offset, or the last tile again once the sequence ends.
+			// SLOT: the step's position in the tile rings (s % RING) as a compile-time number, or -1 for "compute it".
+			constexpr u32 TILE_STEP_BYTES = at::KV_PER_STEP * KV_STRIDE;
+			i8 const *src = kv_head + (size_t)(kb_begin * at::KV_PER_STEP) * KV_STRIDE;
+			u32 const stage_v_next = stage_v_src + TILE_STEP_BYTES;
 			u32 const lds_wave = (u32)(size_t)X17_LDS_PTR(smem) + stage_lds;
-			auto request_tiles = [&]<int SLOT>(u32 step) __attribute__((always_inline)) {
-				if (CPR == 8 || stager) {
-					if constexpr (SLOT >= 0) {
+			// SLOT >= 0 also says that tiles s + 3 and s + 4 both exist (the caller's loop bound)
+			auto request_tiles = [&]<int SLOT>(u32 s) __attribute__((always_inline)) {
+				if constexpr (SLOT >= 0) {
+					if (CPR == 8 || stager) {
 						asm volatile("s_add_i32 m0, %0, %1\n\tglobal_load_lds_dwordx4 %2, %3"
-						             :: "s"(lds_wave), "i"(at::K_RING_OFFSET + SLOT * at::K_TILE_BYTES), "v"(stage_k_src), "s"(load_src) : "memory", "m0", "scc");
+						             :: "s"(lds_wave), "i"(at::K_RING_OFFSET + ((SLOT + 3) % 4) * at::K_TILE_BYTES), "v"(stage_k_src), "s"(src) : "memory", "m0", "scc");
 						asm volatile("s_add_i32 m0, %0, %1\n\tglobal_load_lds_dwordx4 %2, %3"
-						             :: "s"(lds_wave), "i"(at::RAW_V_RING_OFFSET + SLOT * at::RAW_V_TILE_BYTES), "v"(stage_v_src), "s"(load_src) : "memory", "m0", "scc");
-					} else {
-						u32 const slot = step % at::RING;
-						load_to_lds_16(smem + at::K_RING_OFFSET + slot * at::K_TILE_BYTES + stage_lds, load_src, stage_k_src);
-						load_to_lds_16(smem + at::RAW_V_RING_OFFSET + slot * at::RAW_V_TILE_BYTES + stage_lds, load_src, stage_v_src);
+						             :: "s"(lds_wave), "i"(at::RAW_V_RING_OFFSET + SLOT * at::RAW_V_TILE_BYTES), "v"(stage_v_next), "s"(src) : "memory", "m0", "scc");
+					}
+					src += TILE_STEP_BYTES;
+				} else {
+					bool const more = s + 4 < n_steps;
+					if (CPR == 8 || stager) {
+						load_to_lds_16(smem + at::K_RING_OFFSET + ((s + 3) % at::RING) * at::K_TILE_BYTES + stage_lds, src, stage_k_src);
+						load_to_lds_16(smem + at::RAW_V_RING_OFFSET + (s % at::RING) * at::RAW_V_TILE_BYTES + stage_lds, src, more ? stage_v_next : stage_v_src);
+					}
+					if (more) {
+						src += TILE_STEP_BYTES;
 					}
 				}
-				++steps_requested;
-				if (steps_requested < n_steps) {
-					load_src += (size_t)at::KV_PER_STEP * KV_STRIDE;
-				}
 			};
-			// K tile i and raw V tile i + 1 have landed once at most the two requests of step i + 2 are in flight
 			auto stage = [&]<int SLOT>(u32 i) __attribute__((always_inline)) {
-				__builtin_amdgcn_s_waitcnt(0x0F72);          // vmcnt(2)
+				__builtin_amdgcn_s_waitcnt(0x0F74);          // vmcnt(4): K tile i and raw V tile i + 1 have landed
 				__builtin_amdgcn_s_waitcnt(0xC07F);          // lgkmcnt(0): own LDS traffic of step i-1 is complete
 				__builtin_amdgcn_s_barrier();                // ... and so is everybody else's: tiles i are visible
-				constexpr int NEXT_SLOT = SLOT < 0 ? -1 : (SLOT + (int)at::PREFETCH) % (int)at::RING;
-				request_tiles.template operator()<NEXT_SLOT>(i + at::PREFETCH);      // into the slot step i - 1 used
+				request_tiles.template operator()<SLOT>(i);
 			};
 			// raw V tile of step i + 1 -> f16 tile (i + 1) % 2
 			auto widen_next = [&]<int SLOT>(u32 i) __attribute__((always_inline)) {
@@ -539,16 +550,24 @@ void kernel(
 			};
 
 			__syncthreads();                      // previous head's tiles are no longer read
-			X17_UNROLL for (u32 j = 0; j < at::PREFETCH; ++j) request_tiles.template operator()<-1>(j);
-			__builtin_amdgcn_s_waitcnt(0x0F74);   // vmcnt(4): step 0 has landed
+			// (every workgroup walks at least four tiles: 0 .. 3 exist)
+			if (CPR == 8 || stager) {
+				load_to_lds_16(smem + at::RAW_V_RING_OFFSET + stage_lds, src, stage_v_src);
+				X17_UNROLL for (u32 j = 0; j < 3; ++j) {
+					load_to_lds_16(smem + at::K_RING_OFFSET + j * at::K_TILE_BYTES + stage_lds, src + j * TILE_STEP_BYTES, stage_k_src);
+					load_to_lds_16(smem + at::RAW_V_RING_OFFSET + (j + 1) * at::RAW_V_TILE_BYTES + stage_lds, src + j * TILE_STEP_BYTES, stage_v_next);
+				}
+			}
+			src += 3 * TILE_STEP_BYTES;
+			__builtin_amdgcn_s_waitcnt(0x0F76);   // vmcnt(6): raw V tile 0 has landed
 			widen_v(0, 0);
 			u32 i = 0;
 			for (; i < first_active; ++i) idle_step(i);
 			for (; i < first_full; ++i) step.template operator()<true, -1>(i);
 			// the fully visible run: single steps up to a multiple of the ring, whole rings, single steps again
 			for (; i < diagonal && i % at::RING != 0; ++i) step.template operator()<false, -1>(i);
-			static_assert(at::RING == 4, "the run below is written out for a ring of four");
-			for (; i + at::RING <= diagonal; i += at::RING) {
+			static_assert(at::RING == 4 && at::PREFETCH == 3, "the run below and the requests are written out for rings of four");
+			for (; i + at::RING <= diagonal && i + 2 * at::RING <= n_steps; i += at::RING) {
 				step.template operator()<false, 0>(i);
 				step.template operator()<false, 1>(i + 1);
 				step.template operator()<false, 2>(i + 2);
