@@ -78,7 +78,8 @@ def test_attn_fast_within_one_code(dev, t, h, hd, w):
 
 
 @pytest.mark.parametrize("t,h,hd,w,strict", [(448, 2, 64, 128, True), (192, 4, 32, 0, True), (1088, 2, 128, 256, True),
-                                             (1088, 2, 128, 256, False), (16384 + 64, 2, 128, 512, False)])
+                                             (1088, 2, 128, 256, False), (16384 + 64, 2, 128, 512, False),
+                                             (128, 2, 64, 0, False), (192, 2, 128, 64, False)])
 def test_attn_sequence_lengths_that_are_multiples_of_64_only(dev, t, h, hd, w, strict):
 	"""src/device/cuda/attn.rs:398-404 accepts seq_len % 64 == 0; the query block here holds 128 queries.  The last
 	block of such a sequence starts 64 queries early: every output against the oracle (strict builds bit for bit)."""
