@@ -44,7 +44,8 @@ PEAK_F16_TFLOPS = 2500.0     # dense f16
 # launches per measurement, after the reference's own harnesses (attn_fwd_i8.cu:117-182, ffn_f_fwd_f8.cu:108-161):
 # 50 warm-up launches, 100 timed (attention: 10 timed), median and minimum reported
 GEMM_WARM, GEMM_TIMED = 50, 100
-ATTN_WARM, ATTN_TIMED = 5, 10
+ATTN_WARM, ATTN_TIMED = 50, 10     # (attn_fwd_i8.cu:117: int warmup = 50)
+DECODE_WARM, DECODE_TIMED = 50, 100
 
 
 def profile_traffic(file_name):
@@ -376,7 +377,7 @@ def extras(dev, X, recipes):
 		for name, fn in block.stages(xb, wts, outs):
 			if fused and name != "attn_qkv":
 				continue
-			iters, warm = (ATTN_TIMED, ATTN_WARM) if name == "attn_fwd_i8" else (30, 10)
+			iters, warm = (ATTN_TIMED, ATTN_WARM) if name == "attn_fwd_i8" else (GEMM_TIMED, GEMM_WARM)
 			med, mn = _median_launch(dev, X, fn, iters, warm)
 			c4[name + "_us"] = med * 1e6
 			if name in ops:
@@ -432,7 +433,7 @@ def extras(dev, X, recipes):
 	c5 = {}
 	for strict in (False, True):
 		k5 = recipes.attn_kernel(dev, H5, HD5, strict)
-		med, _ = _median_launch(dev, X, lambda: k5.launch(q5, kv5, sk5, sv5, tp5, o5, None, W5), ATTN_TIMED, 3)
+		med, _ = _median_launch(dev, X, lambda: k5.launch(q5, kv5, sk5, sv5, tp5, o5, None, W5), ATTN_TIMED, ATTN_WARM)
 		p5 = W5 * (W5 - 1) // 2 + (T5 - W5) * W5
 		tag = "strict" if strict else "fast"
 		c5[f"prefill_{tag}_ms"] = med * 1e3
@@ -441,7 +442,7 @@ def extras(dev, X, recipes):
 	rs5 = row_scale_tensors(T5, H5)
 	ob5 = X.Tensor(dev, (T5, H5 * HD5), X.BF16)
 	k5r = recipes.attn_row_scaled_kernel(dev, H5, HD5, X.BF16, False)
-	med, _ = _median_launch(dev, X, lambda: k5r.launch_row_scaled(q5, kv5, sk5, sv5, tp5, ob5, None, W5, *rs5), ATTN_TIMED, 3)
+	med, _ = _median_launch(dev, X, lambda: k5r.launch_row_scaled(q5, kv5, sk5, sv5, tp5, ob5, None, W5, *rs5), ATTN_TIMED, ATTN_WARM)
 	c5["prefill_row_scaled_bf16_ms"] = med * 1e3
 	c5["prefill_row_scaled_bf16_tops"] = 4.0 * HD5 * H5 * p5 / med / 1e12
 	del q5, kv5, o5, ob5, rs5
@@ -458,13 +459,13 @@ def extras(dev, X, recipes):
 		tag = "strict" if strict else "fast"
 		# dense case: an all-zero query gives every key the same score, so every 8-bit probability is 255 and every
 		# K and V row of the window is read -- the roofline figure of the kernel
-		med, _ = _median_launch(dev, X, lambda: kd.launch(q_flat, cache, lens, sk5, sv5, tp5, od, None, W5), 30, 10)
+		med, _ = _median_launch(dev, X, lambda: kd.launch(q_flat, cache, lens, sk5, sv5, tp5, od, None, W5), DECODE_TIMED, DECODE_WARM)
 		c5[f"decode_dense_{tag}_us"] = med * 1e6
 		c5[f"decode_dense_{tag}_gbs"] = nbytes / med / 1e9
 		c5[f"decode_dense_{tag}_frac_of_hbm"] = nbytes / med / 1e9 / PEAK_HBM_GBS
 		# Gaussian queries and cache: about 99 % of the 8-bit probabilities are 0 and their V rows are not fetched.
 		# The rate below divides the WHOLE cache by the time: work avoided, not bandwidth (it can exceed the HBM peak).
-		med, _ = _median_launch(dev, X, lambda: kd.launch(qd, cache, lens, sk5, sv5, tp5, od, None, W5), 30, 10)
+		med, _ = _median_launch(dev, X, lambda: kd.launch(qd, cache, lens, sk5, sv5, tp5, od, None, W5), DECODE_TIMED, DECODE_WARM)
 		c5[f"decode_gaussian_{tag}_us"] = med * 1e6
 		c5[f"decode_gaussian_{tag}_cache_gbs_work_avoided"] = nbytes / med / 1e9
 	# the cache as a row-scaled prefill leaves it: one scale per (row, head) of k and v, bf16 output
@@ -474,7 +475,7 @@ def extras(dev, X, recipes):
 	f32t = lambda a: X.Tensor.from_numpy(dev, np.ascontiguousarray(a, dtype=np.float32), X.F32)
 	rsd = [f32t(0.125 * (0.75 + 0.5 * rng.random((S5, H5)))), f32t(np.broadcast_to(scale_one[0], (S5, H5, CAP))), f32t(vw5), f32t(sw5), f32t(os5)]
 	odb = X.Tensor(dev, (S5, H5 * HD5), X.BF16)
-	med, _ = _median_launch(dev, X, lambda: kd_rows.launch_row_scaled(qd, cache, lens, sk5, sv5, tp5, odb, None, W5, *rsd), 30, 10)
+	med, _ = _median_launch(dev, X, lambda: kd_rows.launch_row_scaled(qd, cache, lens, sk5, sv5, tp5, odb, None, W5, *rsd), DECODE_TIMED, DECODE_WARM)
 	c5["decode_row_scaled_bf16_us"] = med * 1e6
 	out["config5_long_context"] = c5
 	# what the matrix cores sustain with no memory traffic at all, beside the nominal peaks used above
