@@ -125,7 +125,9 @@ X17_DEV u32 pack_f16(f32 lo, f32 hi) {
 X17_DEV void load_to_lds_16(u8 *lds_uniform, i8 const *src_uniform, u32 lane_offset) {
 	// (the address is the same in every lane; reading it from the first one tells the compiler so)
 	u32 const lds = __builtin_amdgcn_readfirstlane((u32)(size_t)X17_LDS_PTR(lds_uniform));
-	asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+	// (gfx9 family: a scalar write of M0 needs one wait state before a direct-to-LDS load reads it; the compiler
+	// inserts it for its own loads and cannot see into this string)
+	asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
 	             :: "s"(lds), "v"(lane_offset), "s"(src_uniform) : "memory", "m0");
 }
 
@@ -396,9 +398,9 @@ void kernel(
 			auto request_tiles = [&]<int SLOT>(u32 s) __attribute__((always_inline)) {
 				if constexpr (SLOT >= 0) {
 					if (CPR == 8 || stager) {
-						asm volatile("s_add_i32 m0, %0, %1\n\tglobal_load_lds_dwordx4 %2, %3"
+						asm volatile("s_add_i32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
 						             :: "s"(lds_wave), "i"(at::K_RING_OFFSET + ((SLOT + 3) % 4) * at::K_TILE_BYTES), "v"(stage_k_src), "s"(src) : "memory", "m0", "scc");
-						asm volatile("s_add_i32 m0, %0, %1\n\tglobal_load_lds_dwordx4 %2, %3"
+						asm volatile("s_add_i32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
 						             :: "s"(lds_wave), "i"(at::RAW_V_RING_OFFSET + SLOT * at::RAW_V_TILE_BYTES), "v"(stage_v_next), "s"(src) : "memory", "m0", "scc");
 					}
 					src += TILE_STEP_BYTES;

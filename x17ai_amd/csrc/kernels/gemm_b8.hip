@@ -444,7 +444,9 @@ struct LaneOffsets {
 // compiler's own selection forms a 64-bit address per lane in ONE vector register pair for every load: a 64-bit
 // vector add per load, each waiting until the previous load has read the pair (measured 3-5 % of the kernel).
 X17_DEV void load_to_lds_16(u8 *lds_uniform, u8 const *src_uniform, u32 lane_offset) {
-	asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+	// (gfx9 family: a scalar write of M0 needs one wait state before a direct-to-LDS load reads it; the compiler
+	// inserts it for its own loads and cannot see into this string)
+	asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
 	             :: "s"((u32)(size_t)X17_LDS_PTR(lds_uniform)), "v"(lane_offset), "s"(src_uniform) : "memory", "m0");
 }
 
