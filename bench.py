@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized block-forward path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] [--only KERNEL] [--copy-probe]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] [--only KERNEL]
 
 Headline (the JSON line's `value`): benchmark config 4, the full quantized block forward over
 4 sequences x 8192 tokens, d_model 2048, 16 heads x 128, window 512, d_ff 8192:
@@ -247,57 +247,6 @@ def cpu_extras():
 	return out
 
 
-def mfma_probe(dev, X):
-	"""Loops of nothing but MFMAs on register operands, all-zero and Gaussian data: what the matrix cores of this
-	machine sustain (the clock under dense MFMA load depends on how much the operands toggle)."""
-	from x17ai_amd.probes import MfmaProbe
-	rng = np.random.default_rng(7)
-	out = X.Tensor(dev, (256 * 512,), X.F32)
-	result = {}
-	for kind, name, peak in ((0, "int8", PEAK_INT8_TOPS), (1, "e4m3", PEAK_INT8_TOPS), (2, "f16", PEAK_INT8_TOPS / 2)):
-		probe = MfmaProbe(dev, kind)
-		if kind == 0:
-			gauss = _rand_codes(rng, (12 * 512 * 16,))
-		elif kind == 1:
-			gauss = rng.integers(0x20, 0x50, 12 * 512 * 16).astype(np.uint8).view(np.int8)       # normal e4m3 codes
-			gauss = np.where(rng.random(gauss.shape) < 0.5, gauss, gauss | np.int8(-128)).astype(np.int8)
-		else:
-			gauss = rng.standard_normal(12 * 512 * 8).astype(np.float16).view(np.int8)
-		for data_name, data in (("zeros", np.zeros(12 * 512 * 16, np.int8)), ("gaussian", gauss)):
-			operands = X.Tensor.from_numpy(dev, np.ascontiguousarray(data), X.INT8)
-			ops = [0.0]
-
-			def fn():
-				ops[0] = probe.launch(operands, out, 4096)
-			med, mn = _median_launch(dev, X, fn, 10, 3)
-			result[f"{name}_{data_name}"] = {"median_us": med * 1e6, "tops": ops[0] / med / 1e12,
-			                                 "frac_of_nominal_peak": ops[0] / med / 1e12 / peak}
-	return result
-
-
-def valu_probe(dev, X):
-	"""Issue rate of single vector instructions, in nanoseconds of SIMD time per wavefront-instruction, with 1, 2, 3,
-	4 and 8 wavefronts on every SIMD of the chip.  Entries named "group: ..." are composite loops without memory
-	traffic -- a matrix instruction next to vector instructions, and the instruction mix of one 32-key step of the
-	attention speed build -- and give nanoseconds of SIMD time per group."""
-	from x17ai_amd.probes import ValuProbe, valu_probe_ops
-	src = X.Tensor.from_numpy(dev, np.zeros(256, np.float32), X.F32)
-	out = X.Tensor(dev, (1024 * 8 * 64,), X.F32)
-	result = {}
-	for op, name in enumerate(valu_probe_ops()):
-		probe = ValuProbe(dev, op)
-		row = {}
-		for waves in (1, 2, 3, 4, 8):
-			n = [0.0]
-
-			def fn():
-				n[0] = probe.launch(src, out, waves, 1024)
-			med, mn = _median_launch(dev, X, fn, 5, 2)
-			row[f"waves_{waves}"] = mn * 1e9 / n[0]
-		result[name] = row
-	return result
-
-
 def extras(dev, X, recipes):
 	out = {}
 	rng = np.random.default_rng(3000)
@@ -478,8 +427,6 @@ def extras(dev, X, recipes):
 	med, _ = _median_launch(dev, X, lambda: kd_rows.launch_row_scaled(qd, cache, lens, sk5, sv5, tp5, odb, None, W5, *rsd), DECODE_TIMED, DECODE_WARM)
 	c5["decode_row_scaled_bf16_us"] = med * 1e6
 	out["config5_long_context"] = c5
-	# what the matrix cores sustain with no memory traffic at all, beside the nominal peaks used above
-	out["mfma_probe"] = mfma_probe(dev, X)
 	return out
 
 
@@ -608,14 +555,6 @@ def main():
 	ap.add_argument("--separate-qkv", action="store_true",
 	                help="headline block with the q and kv projections as two launches, as src/main.rs launches them "
 	                     "(default: one launch that reads x once)")
-	ap.add_argument("--copy-probe", action="store_true",
-	                help="only run a 1 GiB device-to-device copy kernel (calibrates the HBM traffic counters)")
-	ap.add_argument("--mfma-probe", action="store_true",
-	                help="only run loops of nothing but MFMAs on register operands (all-zero and Gaussian data; int8, "
-	                     "e4m3, f16): what the matrix cores of this machine sustain, beside the nominal peaks")
-	ap.add_argument("--valu-probe", action="store_true",
-	                help="only run loops of one vector instruction each (issue rate per instruction and wavefronts per SIMD: "
-	                     "what bounds the attention kernel's softmax)")
 	ap.add_argument("--only", choices=ONLY_TARGETS,
 	                help="launch one kernel of one workload --steps times and print its median (used for the profiles)")
 	args = ap.parse_args()
@@ -627,23 +566,6 @@ def main():
 	from x17ai_amd import recipes
 
 	dev = X.Device(0)
-	if args.copy_probe:
-		from x17ai_amd.probes import CopyProbe
-		n = 1 << 30
-		src = X.Tensor.from_numpy(dev, np.zeros(n, np.int8), X.INT8)
-		dst = X.Tensor(dev, (n,), X.INT8)
-		probe = CopyProbe(dev)
-		for _ in range(5):
-			probe.launch(src, dst)
-		dev.synchronize()
-		print(json.dumps({"copy_probe_bytes_read": n, "copy_probe_bytes_written": n, "launches": 5}))
-		return
-	if args.mfma_probe:
-		print(json.dumps({"mfma_probe": mfma_probe(dev, X)}))
-		return
-	if args.valu_probe:
-		print(json.dumps({"valu_probe_ns_per_wave_instruction_per_simd": valu_probe(dev, X)}))
-		return
 	if args.only:
 		single(dev, X, recipes, args.only, args.steps)
 		return

@@ -39,12 +39,8 @@ def test_host_library_exports_every_declared_entry_point():
 	assert declared and not [s for s in declared if s not in exported]
 
 
-def test_probe_library_exports_its_header_and_the_product_header_names_no_probe():
-	"""The benchmark's measurement aids live in their own header and library."""
-	declared = _declared("x17ai_probe.h")
-	path = os.path.join(os.path.dirname(_ffi.lib_paths()["host"]), "libx17ai_probe.so")
-	exported = set(_exported(path))
-	assert declared and not [s for s in declared if s not in exported]
+def test_the_product_headers_and_libraries_hold_no_measurement_aids():
+	assert sorted(os.listdir(os.path.join(ROOT, "include"))) == ["x17ai_hip_shim.h", "x17ai_host.h"]
 	assert not [s for s in _declared("x17ai_host.h") if "probe" in s]
 	assert not [s for s in _exported(_ffi.lib_paths()["host"]) if "probe" in s and s.startswith("x17h_")]
 

@@ -91,11 +91,6 @@ def _specs():
 	add(("attn", 8, 64, False))
 	add(("attn_rows", 32, 128, BF16, False))
 	add(("decode_rows", 32, 128, 4096, BF16, False))
-	add(("copy_probe",))
-	for kind in (0, 1, 2):
-		add(("mfma_probe", kind))
-	for op in range(35):
-		add(("valu_probe", op))
 	# ---- tests/test_gpu_fullsize.py (the strict ffn pair, attention and decode kernels are listed above)
 	add(("attn", 16, 128, True))
 	add(("attn_rows", 32, 128, BF16, True))
@@ -162,18 +157,6 @@ def _build_one(spec) -> str:
 		return recipes.rms_norm_kernel(None, spec[1], spec[2]).name
 	if kind == "dequant":
 		return recipes.dequant_gemm_kernel(None, spec[1], spec[2], spec[3], spec[4], spec[5], spec[6]).name
-	if kind == "mfma_probe":
-		from .probes import MfmaProbe
-		MfmaProbe(None, spec[1])
-		return f"mfma_probe-kind{spec[1]}"
-	if kind == "copy_probe":
-		from .probes import CopyProbe
-		CopyProbe(None)
-		return "copy_probe"
-	if kind == "valu_probe":
-		from .probes import ValuProbe
-		ValuProbe(None, spec[1])
-		return f"valu_probe-op{spec[1]}"
 	if kind == "acc_probe":
 		k, n = 1024, 256
 		cfg = GemmConfig(GemmInputConfig(INT8, k, None, False), GemmInputConfig(INT8, k, n, True), INT8)
