@@ -36,7 +36,9 @@ enum { X17H_EPI_SCALE = 0, X17H_EPI_GEGLU = 1, X17H_EPI_RESIDUAL = 2, X17H_EPI_R
        /* no counterpart in gemm.rs: run-time per-row x per-column f32 scales, bf16 output */
        X17H_EPI_DEQUANT = 4,
        /* the older Q writer with a learned bf16 scale per column, cuda/qkvg_fwd_i8.cuh:145-219 (launch: extra =
-        * q_norm_scales bf16 [b_rows]; head_dim, eps and out_scale as for RMSNorm, no V halves) */
+        * q_norm_scales bf16 [b_rows]; head_dim, eps and out_scale as for RMSNorm, no V halves; inp_scale = the factor
+        * applied after the learned scales, 1.0 or 0 for none -- the old writer's base class, which is gone from the
+        * reference tree, was built with 1 / sqrt(MODEL_DIM), cuda/qkvg_fwd_i8.cuh:151-159) */
        X17H_EPI_QNORM = 5,
        /* no counterpart in gemm.rs: the q (Scale) and kv (RMSNorm) projections as one launch, x17h_gemm_kernel_launch_qkv */
        X17H_EPI_QKV = 6 };

@@ -201,10 +201,13 @@ def epilogue_l2norm(acc, head_dim: int, eps: float, inp_scale: float, out_scale:
 	return c, rrms
 
 
-def epilogue_qnorm(acc, head_dim: int, eps: float, out_scale: float, dyn_bf16, want_rrms: bool = False):
+def epilogue_qnorm(acc, head_dim: int, eps: float, out_scale: float, dyn_bf16, want_rrms: bool = False,
+                   post_scale: float = 1.0):
 	"""The learned-scale Q writer (cuda/qkvg_fwd_i8.cuh:145-219; hook cuda/gemm_b8.cuh:761-824): every head_dim raw
 	columns are one head, L2-normalised like the K halves of epilogue_l2norm, then multiplied by a bf16 scale per
-	column (dyn_bf16: uint16 bit patterns, [N_raw]).  Returns q codes int8 [M, N_raw] (and rrms [M, N_raw / head_dim])."""
+	column (dyn_bf16: uint16 bit patterns, [N_raw]) and, when post_scale != 1, by f32(post_scale) (the factor of the
+	old writer's vanished base class, cuda/qkvg_fwd_i8.cuh:151-159).  Returns q codes int8 [M, N_raw] (and rrms
+	[M, N_raw / head_dim])."""
 	acc = np.ascontiguousarray(acc, dtype=np.int32)
 	dyn = np.ascontiguousarray(dyn_bf16, dtype=np.uint16)
 	m, n_raw = acc.shape
@@ -213,7 +216,7 @@ def epilogue_qnorm(acc, head_dim: int, eps: float, out_scale: float, dyn_bf16, w
 	rrms = np.empty((m, n_raw // head_dim), dtype=np.float32) if want_rrms else None
 	head_scale = out_scale * float(np.sqrt(np.float64(head_dim)))
 	lib().x17o_epilogue_qnorm(_p(acc), _p(c), _p(rrms) if want_rrms else None, _p(dyn), _sz(m), _sz(n_raw), _sz(head_dim),
-	                          ctypes.c_double(eps), ctypes.c_double(head_scale))
+	                          ctypes.c_double(eps), ctypes.c_double(head_scale), ctypes.c_double(post_scale))
 	return (c, rrms) if want_rrms else c
 
 

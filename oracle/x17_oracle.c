@@ -419,13 +419,17 @@ X17_EXPORT void x17o_epilogue_l2norm(const int32_t *acc, int8_t *C, float *rrms,
  * with dyn a bf16 vector of N_raw learned scales (given as bf16 bit patterns).  The old writer adds no eps
  * (qkvg_fwd_i8.cuh:56) and takes head_scale = sqrt(hd) * 8 (:205); the live hook adds EPS (gemm_b8.cuh:808).
  * rrms (may be NULL) receives scale per (row, head).
- * Parity note: the old writer's final store goes through a base class (b8::FixedI8MatrixWriter) that no longer
- * exists in the reference tree; the FixedI8 conversion of the live writers (clamp to +-127, round to nearest even)
- * is assumed for it. */
+ * PARITY UNPINNED for the final store, in two points.  The old writer hands its f32 values to a base class,
+ * b8::FixedI8MatrixWriter<M, N, constexpr_inv_sqrt(MODEL_DIM)> (cuda/qkvg_fwd_i8.cuh:151-159), that no longer exists
+ * in the reference tree.  (1) Its conversion: the FixedI8 conversion of the live writers (clamp to +-127, round to
+ * nearest even) is assumed.  (2) Its template constant 1 / sqrt(MODEL_DIM): the live successor's f32 overload
+ * multiplies by its SCALE unless that is 1 (ScaledMatrixWriter, cuda/gemm_b8.cuh:307-324); whether the vanished base
+ * did the same to the normalised q cannot be read from the tree.  `post_scale` is that factor: 1.0 stores
+ * (x * scale) * dyn as it is, 1 / sqrt(K) is the other reading, one more f32 multiply before the conversion. */
 X17_EXPORT void x17o_epilogue_qnorm(const int32_t *acc, int8_t *C, float *rrms, const uint16_t *dyn_bf16,
-                                    size_t M, size_t N_raw, size_t hd, double eps, double head_scale) {
+                                    size_t M, size_t N_raw, size_t hd, double eps, double head_scale, double post_scale) {
 	size_t heads = N_raw / hd;
-	float feps = (float)eps, fhs = (float)head_scale;
+	float feps = (float)eps, fhs = (float)head_scale, fps = (float)post_scale;
 	#pragma omp parallel for schedule(static)
 	for (size_t m = 0; m < M; ++m) {
 		for (size_t h = 0; h < heads; ++h) {
@@ -443,7 +447,9 @@ X17_EXPORT void x17o_epilogue_qnorm(const int32_t *acc, int8_t *C, float *rrms, 
 				uint32_t bits = (uint32_t)dyn_bf16[h * hd + d] << 16;
 				float dyn;
 				memcpy(&dyn, &bits, 4);
-				c[d] = fixedi8(((float)a[d] * scale) * dyn);
+				float t = ((float)a[d] * scale) * dyn;
+				if (fps != 1.0f) t = t * fps;
+				c[d] = fixedi8(t);
 			}
 			if (rrms != NULL) rrms[m * heads + h] = scale;
 		}

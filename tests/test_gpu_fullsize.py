@@ -341,3 +341,23 @@ def test_config4_block_chain(dev):
 	for name in ("q", "kv"):
 		assert np.array_equal(fused[name], got[name]), name
 	assert np.array_equal(fused["k_rrms"].view(np.uint32), got["k_rrms"].view(np.uint32))
+
+
+def test_benched_speed_builds_against_strict_builds(dev):
+	"""Every speed build bench.py times outside the config 4 chain, at the size it is timed at, against its strict build
+	over ALL outputs (tests/fast_builds.py; the figures of one run are tests/golden/fast_builds_vs_strict.json): config 5
+	decode with ragged lengths, flat-score sequences and the dense all-zero-query case, plain and row-scaled; the
+	row-scaled bf16 prefill over all 65536 x 4096 outputs; the dequantising GEMM pair of config 2."""
+	from tests import fast_builds as FB
+	d = FB.decode(dev)
+	assert d["hist_abs_code_diff_0_1_2_3_more"][2:] == [0, 0, 0] and d["mismatched"] < 0.02 * d["elements"], d
+	assert d["l_max_abs"] < 1e-4 and d["dense_sequences_mismatched"] < 0.02 * 8 * 4096, d
+	r = FB.decode_row_scaled(dev)
+	assert r["frac_mismatched"] < 1e-3 and r["beyond_one_step_and_floor"] == 0 and r["l_max_abs"] < 1e-4, r
+	p = FB.prefill_row_scaled(dev)
+	assert p["frac_mismatched"] < 0.06 and p["beyond_one_step_and_floor"] < 1e-4 * p["elements"], p
+	assert p["rel_l2"] < 2e-3 and p["max_abs"] <= 0.0625 and p["l_max_abs"] < 1e-4, p
+	q = FB.dequant_pair(dev)
+	assert q["plain_bf16"]["mismatched"] == 0, q                   # no approximate operation upstream of the store
+	g = q["geglu_bf16"]
+	assert g["frac_mismatched"] < 1e-4 and g["beyond_one_step_and_floor"] == 0 and g["rel_l2"] < 1e-4, g

@@ -129,6 +129,25 @@ def test_learned_scale_q_writer_bit_exact(dev, hd):
 	assert not np.array_equal(S.epilogue_qnorm(S.gemm_i32(a, b), hd, 0.0, 8.0, np.roll(dyn, 1)), want)
 
 
+def test_learned_scale_q_writer_with_the_base_writer_scale(dev):
+	"""The old writer's base class was built with SCALE = 1 / sqrt(MODEL_DIM) (cuda/qkvg_fwd_i8.cuh:151-159) and is
+	gone from the reference tree; the live scaled writer's f32 overload applies its SCALE (cuda/gemm_b8.cuh:307-324).
+	That reading is one constant away: post_scale = 1 / sqrt(K), one more f32 multiply before the conversion."""
+	m, k, n, hd = 512, 512, 512, 64
+	rng = rng_for("qnorm-post")
+	a, b = i8_codes(rng, (m, k)), i8_codes(rng, (n, k))
+	dyn = _bf16_bits(8.0 + 8.0 * rng.random(n))                 # (large learned scales keep the codes off zero)
+	post = 1.0 / math.sqrt(k)
+	kern = recipes.attn_q_norm_kernel(dev, k, n, hd, 0.0, True, post)
+	c = X.Tensor(dev, (m, n), X.INT8)
+	kern.launch(_up(dev, a, X.INT8), _up(dev, b, X.INT8), c, _up(dev, dyn, X.BF16))
+	want = S.epilogue_qnorm(S.gemm_i32(a, b), hd, 0.0, 8.0, dyn, post_scale=post)
+	got = c.download()
+	assert np.array_equal(got, want)
+	assert len(np.unique(got)) > 20
+	assert not np.array_equal(want, S.epilogue_qnorm(S.gemm_i32(a, b), hd, 0.0, 8.0, dyn))
+
+
 def test_learned_scale_q_writer_with_eps_at_a_full_width(dev):
 	"""The hook that survives in the live header adds EPS (cuda/gemm_b8.cuh:808); 1024 columns = four column tiles."""
 	m, k, n, hd = 512, 2048, 1024, 128

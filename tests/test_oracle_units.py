@@ -230,6 +230,17 @@ def test_learned_scale_q_writer(hd):
 	z = acc.copy()
 	z[3, :hd] = 0
 	assert not S.epilogue_qnorm(z, hd, 2.0 ** -70, 8.0, dyn)[3, :hd].any()
+	# the factor of the old writer's vanished base class (1 / sqrt(MODEL_DIM), cuda/qkvg_fwd_i8.cuh:151-159) is an
+	# explicit argument: post_scale = 1 is the default above; a power of two moves every unsaturated code exactly;
+	# 1 / sqrt(K) follows the float64 closed form times that factor
+	assert np.array_equal(S.epilogue_qnorm(acc, hd, 0.0, 8.0, dyn, post_scale=1.0), got)
+	half = S.epilogue_qnorm(acc, hd, 0.0, 4.0, dyn)                      # out_scale 4 = out_scale 8 times 0.5 ...
+	assert np.array_equal(S.epilogue_qnorm(acc, hd, 0.0, 8.0, dyn, post_scale=0.5)[np.abs(got) < 127], half[np.abs(got) < 127])
+	ps = 1.0 / np.sqrt(np.float64(2048.0))
+	scaled = S.epilogue_qnorm(acc, hd, 0.0, 8.0 * 32.0, dyn, post_scale=ps)   # (out_scale 256 keeps the codes off zero)
+	want_s = want * 32.0 * ps
+	assert np.abs(scaled - np.clip(want_s, -127, 127)).max() <= 0.5 + 1e-3
+	assert len(np.unique(scaled)) > 20
 
 
 def test_gemm_f32_seq_against_float64():

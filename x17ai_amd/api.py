@@ -230,7 +230,11 @@ class DequantConfig:
 @dataclasses.dataclass
 class QNormConfig:
 	"""The reference's older Q writer (cuda/qkvg_fwd_i8.cuh:145-219; hook cuda/gemm_b8.cuh:761-824): every head_dim
-	raw columns are one L2-normalised head, times a learned bf16 scale per column passed at launch."""
+	raw columns are one L2-normalised head, times a learned bf16 scale per column passed at launch.  `inp_scale` is
+	the factor applied after the learned scales: the old writer hands its values to a base class built with
+	1 / sqrt(MODEL_DIM) (cuda/qkvg_fwd_i8.cuh:151-159) that no longer exists in the reference tree; 1.0 stores them as
+	they are, 1 / sqrt(K) is the other reading (the live scaled writer's f32 overload applies its scale,
+	cuda/gemm_b8.cuh:307-324)."""
 	eps: float
 	head_dim: int
 	out_scale: float

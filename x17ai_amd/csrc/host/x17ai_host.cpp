@@ -829,11 +829,13 @@ std::unique_ptr<GemmKernel> GemmKernel::create(std::shared_ptr<HipDevice> device
 	};
 	if (auto const *c = std::get_if<QNormConfig>(&e)) {
 		if (g.c_dtype != DType::Int8 || g.a.dtype != DType::Int8 || g.b.dtype != DType::Int8) { diag.add_error("QNorm epilogue requires i8 inputs and an i8 output"); return nullptr; }
-		if (!std::isfinite(c->eps) || c->eps < 0.0 || !finite_pos(c->out_scale.value)) { diag.add_error("invalid QNorm epilogue values"); return nullptr; }
+		if (!std::isfinite(c->eps) || c->eps < 0.0 || !finite_pos(c->out_scale.value) || !finite_pos(c->post_scale.value)) { diag.add_error("invalid QNorm epilogue values"); return nullptr; }
 		if (c->head_dim != 32 && c->head_dim != 64 && c->head_dim != 128) { diag.add_error("QNorm GEMM epilogue requires head_dim in {32, 64, 128}"); return nullptr; }
 		if (b_rows % c->head_dim != 0) { diag.add_error("QNorm GEMM raw output columns must be whole heads"); return nullptr; }
 		head_dim = c->head_dim;
-		common << "#define X17_INP_SCALE 1.0\n#define X17_OUT_SCALE " << format_cpp_f64(c->out_scale.value) << "\n";
+		// X17_INP_SCALE: the factor applied after the learned scales (the old writer's base class carried
+		// 1 / sqrt(MODEL_DIM), cuda/qkvg_fwd_i8.cuh:151-159; 1.0 stores the normalised values as they are)
+		common << "#define X17_INP_SCALE " << format_cpp_f64(c->post_scale.value) << "\n#define X17_OUT_SCALE " << format_cpp_f64(c->out_scale.value) << "\n";
 		common << "#define X17_HEAD_DIM " << c->head_dim << "\n#define X17_EPS " << format_cpp_f64(c->eps) << "\n";
 		// cuda/qkvg_fwd_i8.cuh:205
 		common << "#define X17_HEAD_SCALE " << format_cpp_f64(c->out_scale.value * std::sqrt(double(c->head_dim)))
@@ -1492,7 +1494,7 @@ int x17h_gemm_kernel_new(X17hDevice *dev, char const *kernel_name, X17hGemmConfi
 			case X17H_EPI_RESIDUAL: e = ResidualConfig{inp, outs}; break;
 			case X17H_EPI_RMSNORM: e = RMSNormConfig{c->eps, c->head_dim, c->sep_dim, inp, outs}; break;
 			case X17H_EPI_DEQUANT: e = DequantConfig{c->activation == X17H_ACT_GEGLU}; break;
-			case X17H_EPI_QNORM: e = QNormConfig{c->eps, c->head_dim, outs}; break;
+			case X17H_EPI_QNORM: e = QNormConfig{c->eps, c->head_dim, outs, Scale{c->inp_scale == 0.0 ? 1.0 : c->inp_scale, "post_scale"}}; break;
 			case X17H_EPI_QKV:
 				e = QkvConfig{c->q_cols, ScaleConfig{Scale{c->q_inp_scale, "q inp_scale"}, Scale{c->q_out_scale, "q out_scale"}},
 				              RMSNormConfig{c->eps, c->head_dim, c->sep_dim, inp, outs}};

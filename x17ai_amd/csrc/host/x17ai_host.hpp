@@ -201,7 +201,7 @@ struct GeGluConfig { Scale inp_scale, out_scale; };
 struct DequantConfig { bool geglu; };
 // The reference's older Q writer (cuda/qkvg_fwd_i8.cuh:145-219; hook cuda/gemm_b8.cuh:761-824): every head_dim raw
 // columns are one L2-normalised head, multiplied by a learned bf16 scale per column given at launch.
-struct QNormConfig { double eps; size_t head_dim; Scale out_scale; };
+struct QNormConfig { double eps; size_t head_dim; Scale out_scale; Scale post_scale{1.0, "1"}; };   // post_scale: the factor of the old writer's base class (1 = none)
 // The q and the kv projection of src/main.rs:387-493 as ONE launch over the same token rows (no counterpart in
 // gemm.rs, which launches them one after the other): raw columns [0, q_cols) come from the q weights and go through
 // the Scale writer `q`, the remaining b.rows - q_cols come from the kv weights and go through the RMSNorm writer `kv`.

@@ -327,6 +327,13 @@ struct NaturalWriters {
 				y[1] = y[1] * u2f(d[0] & 0xFFFF0000u);
 				y[2] = y[2] * u2f(d[1] << 16);
 				y[3] = y[3] * u2f(d[1] & 0xFFFF0000u);
+				// The old writer hands its f32 values to a base writer built with SCALE = 1 / sqrt(MODEL_DIM)
+				// (cuda/qkvg_fwd_i8.cuh:151-159); that base class is gone from the tree, and the live scaled writer's f32
+				// overload multiplies by its SCALE unless it is 1 (cuda/gemm_b8.cuh:307-324).  X17_INP_SCALE carries that
+				// factor (1.0: stored as is).
+				if constexpr (f32(f64(X17_INP_SCALE)) != 1.0f) {
+					X17_UNROLL for (int e = 0; e < 4; ++e) y[e] = y[e] * f32(f64(X17_INP_SCALE));
+				}
 			}
 			w[g] = pack4_fixedi8(y[0], y[1], y[2], y[3]);
 		}

@@ -6,6 +6,7 @@ content hash); a machine that runs the tests should find all of them already bui
 from __future__ import annotations
 
 import concurrent.futures
+import math
 import os
 import subprocess
 
@@ -42,6 +43,7 @@ def _specs():
 		add(("attn_q_norm", 512, 512, hd, 0.0))
 		add(("attn_qkv", 512, 256, 512, hd, True))
 	add(("attn_q_norm", 2048, 1024, 128, recipes.L2_NORM_EPS))
+	add(("attn_q_norm", 512, 512, 64, 0.0, 1.0 / math.sqrt(512)))
 	for hd in (64, 128):                 # L2-norm writer on a walk of more tiles than workgroups
 		add(("attn_kv", 256, 2048, hd))
 	# shapes off the 256-grid (rows % 64, raw columns % 128 as the reference accepts them)
@@ -130,7 +132,7 @@ def _build_one(spec) -> str:
 	if kind == "attn_q":
 		return recipes.attn_q_kernel(None, spec[1], spec[2]).name
 	if kind == "attn_q_norm":
-		return recipes.attn_q_norm_kernel(None, spec[1], spec[2], spec[3], spec[4]).name
+		return recipes.attn_q_norm_kernel(None, spec[1], spec[2], spec[3], spec[4], True, spec[5] if len(spec) > 5 else 1.0).name
 	if kind == "attn_qkv":
 		return recipes.attn_qkv_kernel(None, spec[1], spec[2], spec[3], spec[4], spec[5]).name
 	if kind == "ffn_f":

@@ -62,13 +62,16 @@ def attn_qkv_kernel(device: Optional[Device], model_dim: int, q_proj_outputs: in
 
 
 def attn_q_norm_kernel(device: Optional[Device], model_dim: int, q_proj_outputs: int, head_dim: int,
-                       eps: float = 0.0, strict: bool = True) -> GemmKernel:
+                       eps: float = 0.0, strict: bool = True, post_scale: float = 1.0) -> GemmKernel:
 	"""The reference's older Q projection with learned scales (attn_q_fwd_i8.cu:30-34 loads q_norm_scales.bin for
 	it; writer cuda/qkvg_fwd_i8.cuh:145-219): x[i8] . Wq[i8]^T, every head L2-normalised to sqrt(head_dim) * 8 and
 	multiplied by a bf16 scale per column (launch(x, wq, q, q_norm_scales)).  eps = 0 is the old writer; the hook
-	that survives in cuda/gemm_b8.cuh:761-824 adds L2_NORM_EPS."""
-	cfg = QNormConfig(eps, head_dim, FIXED_I8_SCALE)
-	return GemmKernel(device, f"attn_q_norm_fwd-k{model_dim}-n{q_proj_outputs}-hd{head_dim}-{_mode(strict)}",
+	that survives in cuda/gemm_b8.cuh:761-824 adds L2_NORM_EPS.  post_scale: the factor applied after the learned
+	scales -- the old writer's base class (gone from the reference tree) was built with 1 / sqrt(model_dim),
+	cuda/qkvg_fwd_i8.cuh:151-159; 1.0 stores the normalised values as they are."""
+	cfg = QNormConfig(eps, head_dim, FIXED_I8_SCALE, post_scale)
+	tag = "" if post_scale == 1.0 else f"-post{post_scale:.6g}"
+	return GemmKernel(device, f"attn_q_norm_fwd-k{model_dim}-n{q_proj_outputs}-hd{head_dim}{tag}-{_mode(strict)}",
 	                  _gemm(INT8, INT8, INT8, model_dim, q_proj_outputs), cfg, strict)
 
 
