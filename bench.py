@@ -48,16 +48,29 @@ ATTN_WARM, ATTN_TIMED = 50, 10     # (attn_fwd_i8.cu:117: int warmup = 50)
 DECODE_WARM, DECODE_TIMED = 50, 100
 
 
-def profile_traffic(file_name):
+def profile_traffic(file_name, kernel_name):
 	"""HBM bytes per launch as the rocprofv3 summary under profiles/ records them (the line
-	`roofline.traffic: N bytes per launch`), or None when the file or the line is missing."""
+	`roofline.traffic: N bytes per launch`), with the content hash of the kernel build that summary was taken from
+	(`roofline.kernel_key: HASH`, the kernel cache's build.key).  Returns (bytes, key) -- bytes is None when the file or
+	the line is missing, or when the kernel being timed now was built from other sources or parameters than the
+	profiled one (a summary of another build says nothing about this one)."""
 	import re
+	from x17ai_amd import _ffi
 	try:
 		with open(os.path.join(ROOT, "profiles", file_name)) as fh:
-			m = re.search(r"^roofline\.traffic:\s*([0-9]+)\s*bytes per launch", fh.read(), re.M)
-		return int(m.group(1)) if m else None
+			text = fh.read()
 	except OSError:
-		return None
+		return None, None
+	m = re.search(r"^roofline\.traffic:\s*([0-9]+)\s*bytes per launch", text, re.M)
+	k = re.search(r"^roofline\.kernel_key:\s*([0-9a-f]+)", text, re.M)
+	try:
+		with open(os.path.join(_ffi.kernel_cache_dir(), kernel_name, "build.key")) as fh:
+			current = fh.read().strip()
+	except OSError:
+		current = None
+	if not m or not k or current is None or k.group(1) != current:
+		return None, current
+	return int(m.group(1)), current
 
 
 def _rand_i8(rng, shape):
@@ -144,7 +157,7 @@ def headline(dev, X, steps, warmup, fused_qkv=False):
 	dev.synchronize()
 	wall = time.perf_counter() - t0
 	ops = block.n_ops(rows)
-	return {"wall_s": wall, "rows": rows, "dominant_ops": ops[dominant],
+	return {"wall_s": wall, "rows": rows, "dominant_ops": ops[dominant], "dominant_kernel_name": block.k_ffn_y.name,
 	        "dominant_mean_s": sum(t.elapsed_seconds() for t in timers) / steps,
 	        "stage_names": [name for name, _ in stages]}
 
@@ -573,7 +586,7 @@ def main():
 	value = h["rows"] * args.steps / h["wall_s"]
 	achieved = h["dominant_ops"] / h["dominant_mean_s"] / 1e12
 	traffic_file = "gemm_b8_ffn_y_f8_config4.txt"
-	traffic = profile_traffic(traffic_file)
+	traffic, kernel_key = profile_traffic(traffic_file, h["dominant_kernel_name"])
 	c = CONFIG4
 	line = {
 		"metric": "block-fwd tokens/sec at 1 MI355X (config 4: full quantized block forward); int8/fp8 TOPS and % of "
@@ -589,6 +602,7 @@ def main():
 		"roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
 		             "frac": achieved / PEAK_F16_TFLOPS, "traffic": traffic,
 		             "traffic_source": "profiles/" + traffic_file if traffic is not None else None,
+		             "kernel_key": kernel_key,
 		             "kernel": "gemm_b8 (ffn_y_fwd_f8: M=32768, K=8192, N_raw=4096, e4m3 x int8 widened to f16, gated-residual epilogue)",
 		             "mean_launch_us": h["dominant_mean_s"] * 1e6},
 	}

@@ -175,8 +175,13 @@ def test_attn_launch_rejects_bad_arguments(dev):
 	q, kv, sk, sv, temp = _attn_inputs(rng, 256, h, hd)
 	with pytest.raises(X.X17Error, match="window_size must be zero or divisible by 16"):
 		_run_attn(dev, kern, q, kv, sk, sv, temp, 24)
-	with pytest.raises(X.X17Error, match="seq_len must be divisible by 64 and at least 128"):
+	with pytest.raises(X.X17Error, match="at least one query block of 128"):
 		_run_attn(dev, kern, q[:64], kv[:64], sk, sv, temp, 0)
+	# a last block that overhangs recomputes its neighbour's queries from q: the output may not alias an input
+	qt = X.Tensor.from_numpy(dev, q, X.INT8)
+	with pytest.raises(X.X17Error, match="must not share memory with q or kv"):
+		kern.launch(qt, X.Tensor.from_numpy(dev, kv, X.INT8), X.Tensor.from_numpy(dev, sk, X.INT8), X.Tensor.from_numpy(dev, sv, X.INT8),
+		            X.Tensor.from_numpy(dev, temp, X.F32), qt, None, 0)
 	with pytest.raises(X.X17Error, match="kv has 128 rows, but should have 256"):
 		_run_attn(dev, kern, q, kv[:128], sk, sv, temp, 0)
 

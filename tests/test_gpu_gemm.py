@@ -228,6 +228,44 @@ def test_shapes_of_the_reference_that_are_not_whole_tiles(dev):
 		recipes.attn_q_kernel(dev, k, 128)
 
 
+def test_more_writers_on_shapes_that_are_not_whole_tiles(dev):
+	"""The remaining writers off the 256-grid, 320 token rows (a full tile and an overhanging one): the dequantising
+	writer (row and column scale indexing) with and without GeGLU and the learned-scale Q writer on 384 raw columns,
+	the fused q + kv kernel with 256 q columns + 384 kv columns (the moved-back column tile lies wholly on the kv
+	side), and head_dim 128 -- kv alone and fused -- with overhanging rows."""
+	m, k, n = 320, 512, 384
+	rng = rng_for("tails-2")
+	a, b = i8_codes(rng, (m, k)), i8_codes(rng, (n, k))
+	acc = S.gemm_i32(a, b)
+	inp = 1.0 / math.sqrt(k) / 64.0
+	ta, tb = _up(dev, a, X.INT8), _up(dev, b, X.INT8)
+	rs = (0.01 + 0.01 * rng.random(m)).astype(np.float32)
+	cs = (0.01 + 0.01 * rng.random(n)).astype(np.float32)
+	for geglu in (False, True):
+		c = X.Tensor(dev, (m, n // 2 if geglu else n), X.BF16)
+		recipes.dequant_gemm_kernel(dev, k, n, X.INT8, X.INT8, geglu, True).launch_dequant(ta, tb, c, _up(dev, rs, X.F32), _up(dev, cs, X.F32))
+		assert np.array_equal(c.download(), S.epilogue_dequant(acc, rs, cs, geglu)), geglu
+	dyn = _bf16_bits(0.25 + 1.5 * rng.random(n))
+	c = X.Tensor(dev, (m, n), X.INT8)
+	recipes.attn_q_norm_kernel(dev, k, n, 64, 0.0).launch(ta, tb, c, _up(dev, dyn, X.BF16))
+	assert np.array_equal(c.download(), S.epilogue_qnorm(acc, 64, 0.0, 8.0, dyn))
+	# fused q + kv: 256 + 384 raw columns, head_dim 64; then 256 + 512 with head_dim 128 (rows off the grid only)
+	for nq, nkv, hd in ((256, 384, 64), (256, 512, 128)):
+		wq, wkv = i8_codes(rng, (nq, k)), i8_codes(rng, (nkv, k))
+		q, kv = X.Tensor(dev, (m, nq), X.INT8), X.Tensor(dev, (m, nkv), X.INT8)
+		rrms = X.Tensor(dev, (m, nkv // (2 * hd)), X.F32)
+		recipes.attn_qkv_kernel(dev, k, nq, nkv, hd).launch_qkv(ta, _up(dev, wq, X.INT8), _up(dev, wkv, X.INT8), q, kv, rrms)
+		want_kv, want_r = S.epilogue_l2norm(S.gemm_i32(a, wkv), hd, recipes.L2_NORM_EPS, inp, 8.0)
+		assert np.array_equal(q.download(), S.epilogue_scale(S.gemm_i32(a, wq), inp, 8.0)), (nq, nkv, hd)
+		assert np.array_equal(kv.download(), want_kv), (nq, nkv, hd)
+		assert np.array_equal(rrms.download().view(np.uint32), want_r.view(np.uint32)), (nq, nkv, hd)
+		if hd == 128:
+			kv2, rr2 = X.Tensor(dev, (m, nkv), X.INT8), X.Tensor(dev, (m, nkv // (2 * hd)), X.F32)
+			recipes.attn_kv_kernel(dev, k, nkv, hd).launch(ta, _up(dev, wkv, X.INT8), kv2, rr2)
+			assert np.array_equal(kv2.download(), want_kv)
+			assert np.array_equal(rr2.download().view(np.uint32), want_r.view(np.uint32))
+
+
 @pytest.mark.parametrize("store", [X.E4M3, X.INT8])
 @pytest.mark.parametrize("m,k,n", SHAPES)
 def test_geglu_epilogue(dev, m, k, n, store):
@@ -460,8 +498,19 @@ def test_launch_rejects_bad_arguments(dev):
 		kern.launch(X.Tensor(dev, (256, 2 * k), X.INT8), b, c)
 	with pytest.raises(X.X17Error, match="must be 2D"):
 		kern.launch(X.Tensor(dev, (256, k, 1), X.INT8), b, c)
-	with pytest.raises(X.X17Error, match="at least one tile"):
+	with pytest.raises(X.X17Error, match="hold at least one 256 x 256 tile"):
 		kern.launch(X.Tensor(dev, (64, k), X.INT8), b, X.Tensor(dev, (64, n), X.INT8))
+	with pytest.raises(X.X17Error, match="hold at least one 256 x 256 tile"):
+		kern.launch(X.Tensor(dev, (192, k), X.INT8), b, X.Tensor(dev, (192, n), X.INT8))     # divisible by 64, below a tile
+	# an overhanging tile recomputes its neighbour's rows: an in-place gated residual would read what another
+	# workgroup has already overwritten
+	kr = recipes.attn_y_kernel(dev, n // 2, k, True, X.INT8)
+	xr = X.Tensor(dev, (256, n // 2), X.INT8)
+	with pytest.raises(X.X17Error, match="must not share memory with the residual"):
+		kr.launch(a, b, xr, xr)
+	# the fused q + kv entry point on a kernel that is not one
+	with pytest.raises(X.X17Error, match="is not a fused q . kv kernel"):
+		kern.launch_qkv(a, b, b, c, c, X.Tensor(dev, (256, 1), X.F32))
 	with pytest.raises(X.X17Error, match="is not on device"):
 		kern.launch(X.Tensor(None, (256, k), X.INT8), b, c)
 	kern.launch(a, b, c)

@@ -733,6 +733,13 @@ static unsigned ctz(size_t v) { unsigned n = 0; while ((v & 1) == 0) { v >>= 1; 
 
 static int kind_of(DType d) { return d == DType::E4m3 ? 1 : 0; }
 
+// Two tensors share bytes.  Tiles that overhang a matrix edge are moved back and recompute rows or columns of their
+// neighbour; that is only the same store twice as long as no output aliases an input another workgroup still reads.
+static bool overlaps(Tensor const &x, Tensor const &y) {
+	auto const xb = reinterpret_cast<uintptr_t>(x.ptr), yb = reinterpret_cast<uintptr_t>(y.ptr);
+	return x.bytes != 0 && y.bytes != 0 && xb < yb + y.bytes && yb < xb + x.bytes;
+}
+
 std::unique_ptr<GemmKernel> GemmKernel::create(std::shared_ptr<HipDevice> device, std::string const &kernel_name,
                                                GemmConfig const &g, EpilogueConfig const &e, bool strict_math, Diagnostics &diag) {
 	// gemm.rs:451-476 (the reference aborts with todo!() on these; here they are errors)
@@ -914,6 +921,9 @@ Status GemmKernel::launch(GemmArgs const &args) {
 	Status s = tensor_check::matrix_shape(op, "a", *args.a, std::nullopt, a_cols, *device, a_dtype, a_shape);
 	if (!s.is_ok()) return s;
 	if (epilogue_kind == 6) return launch_qkv(args, a_shape[0]);
+	if (args.b2 != nullptr || args.c2 != nullptr) {
+		return Status::err(TensorOpError::Other, "GEMM kernel " + name + " is not a fused q + kv kernel: it takes one weight matrix and one output");
+	}
 	s = tensor_check::matrix_shape(op, "b", *args.b, b_rows, a_cols, *device, b_dtype, b_shape);
 	if (!s.is_ok()) return s;
 	size_t const a_rows = a_shape[0], b_rows_v = b_shape[0];
@@ -929,12 +939,18 @@ Status GemmKernel::launch(GemmArgs const &args) {
 		if (args.extra == nullptr) return Status::err(TensorOpError::Other, "Residual GEMM needs a residual tensor");
 		s = tensor_check::matrix_shape(op, "residual", *args.extra, a_rows, out_cols, *device, DType::Int8, tmp);
 		if (!s.is_ok()) return s;
+		if (overlaps(*args.c, *args.extra)) {
+			return Status::err(TensorOpError::Other, "Residual GEMM output c must not share memory with the residual (no in-place update)");
+		}
+	}
+	if (overlaps(*args.c, *args.a) || overlaps(*args.c, *args.b)) {
+		return Status::err(TensorOpError::Other, std::string(op) + " output c must not share memory with an input");
 	}
 	// gemm.rs:607-614: rows % 64 == 0, raw columns % 128 == 0 (the reference's tile shape); here from one tile upwards
 	if (a_rows % 64 != 0 || b_rows_v % 128 != 0 || a_rows < metadata.M_PER_BLOCK || b_rows_v < metadata.N_PER_BLOCK) {
 		return Status::err(TensorOpError::Other, std::string(op) + " raw output shape [" + std::to_string(a_rows) + ", "
-			+ std::to_string(b_rows_v) + "] must be divisible by [64, 128] and at least one tile [" + std::to_string(metadata.M_PER_BLOCK) + ", "
-			+ std::to_string(metadata.N_PER_BLOCK) + "]");
+			+ std::to_string(b_rows_v) + "] must be divisible by [64, 128] (as in the reference) and hold at least one "
+			+ std::to_string(metadata.M_PER_BLOCK) + " x " + std::to_string(metadata.N_PER_BLOCK) + " tile of this kernel");
 	}
 	if (epilogue_kind == 4) {
 		if (args.extra == nullptr || args.extra2 == nullptr) {
@@ -1005,6 +1021,11 @@ Status GemmKernel::launch_qkv(GemmArgs const &args, size_t a_rows) {
 			+ std::to_string(metadata.M_PER_BLOCK));
 	}
 	if (a_rows > 0xFFFFFFFFull) return Status::err(TensorOpError::Other, std::string(op) + " sizes exceed 32 bits (the kernel's row counts are u32)");
+	for (Tensor const *o : {args.c, args.c2}) {
+		if (overlaps(*o, *args.a) || overlaps(*o, *args.b) || overlaps(*o, *args.b2)) {
+			return Status::err(TensorOpError::Other, std::string(op) + " outputs must not share memory with an input");
+		}
+	}
 	void *a_ptr = args.a->ptr;
 	size_t a_rows_arg = a_rows;
 	void *b_ptr = args.b->ptr;
@@ -1136,6 +1157,10 @@ Status AttnKernel::launch(AttnKernelArgs const &a) {
 		s = tensor_check::matrix_shape("attention", "l", *a.l, config.n_heads, rows, *device, DType::F32, tmp);
 		if (!s.is_ok()) return s;
 	}
+	if (overlaps(*a.out, *a.q) || overlaps(*a.out, *a.kv)) {
+		// (a last query block that would overhang is moved back and recomputes its neighbour's queries from q)
+		return Status::err(TensorOpError::Other, "attention output must not share memory with q or kv");
+	}
 	if (a.batch == 0 || rows % a.batch != 0) {
 		return Status::err(TensorOpError::Other, "attention rows (" + std::to_string(rows) + ") must be divisible by batch (" + std::to_string(a.batch) + ")");
 	}
@@ -1144,8 +1169,8 @@ Status AttnKernel::launch(AttnKernelArgs const &a) {
 	// that would overhang starts earlier instead (it recomputes some of its neighbour's queries and stores the same
 	// bytes), so the same lengths are accepted from one block upwards.
 	if (seq_len % 64 != 0 || seq_len < metadata.Q_PER_BLOCK) {
-		return Status::err(TensorOpError::Other, "attention seq_len must be divisible by 64 and at least " + std::to_string(metadata.Q_PER_BLOCK)
-			+ ", got " + std::to_string(seq_len));
+		return Status::err(TensorOpError::Other, "attention seq_len must be divisible by 64 (as in the reference) and hold at least one query block of "
+			+ std::to_string(metadata.Q_PER_BLOCK) + ", got " + std::to_string(seq_len));
 	}
 	if (a.window_size > 0 && a.window_size % 16 != 0) {
 		return Status::err(TensorOpError::Other, "attention window_size must be zero or divisible by 16, got " + std::to_string(a.window_size));

@@ -53,6 +53,10 @@ def _specs():
 	for hd in (32, 64):
 		add(("attn_kv", 512, 384, hd))
 	add(("mixed", 512, 384, False))
+	for geglu in (False, True):
+		add(("dequant", 512, 384, INT8, INT8, geglu, True))
+	add(("attn_q_norm", 512, 384, 64, 0.0))
+	add(("attn_qkv", 512, 256, 384, 64, True))
 	add(("attn_q", 384, 1024))           # the shortest K with the deeper token ring, more tiles than workgroups
 	add(("ffn_f_f8", 384, 512, True))
 	# ---- tests/test_gpu_attn.py
@@ -120,6 +124,7 @@ def _specs():
 	add(("block", 2048, 64, 32, 2048, None, True))
 	add(("block", 512, 8, 32, 256, None, True))          # tests/test_gpu_files.py
 	add(("attn_q", 128, 256))
+	add(("attn_y", 128, 128, True, INT8))                # tests/test_gpu_gemm.py: the launcher's alias check
 	return s
 
 
