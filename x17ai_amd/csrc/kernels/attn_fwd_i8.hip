@@ -322,7 +322,7 @@ void kernel(
 #endif
 
 		u32 const n_steps = kb_end - kb_begin;
-		if constexpr (!STRICT && !ROW_SCALES) {
+		if constexpr (!STRICT) {
 			// ---- speed build.  The same recurrence, rebuilt around what the kernel turned out to be bound by: the
 			// number of instructions of ANY kind a SIMD has to issue per step (scalar bookkeeping and waits count like
 			// vector arithmetic; with three wavefronts per SIMD an instruction costs 1.5-2.5 ns of SIMD time whatever it does).
@@ -347,20 +347,36 @@ void kernel(
 			//    are needed anyway (the rounding addition is the fused multiply-add above, the sums' lift carries it).
 			//  * The row maximum of a tile needs the partner lane's eight keys only when it moves: both lanes hold the same
 			//    `ext`, and the tile's maximum exceeds it exactly when one of the two halves does.
+			//  * Row-scaled build: a key's scale is not monotone in the dot product and the 16 registers of the bias words are
+			//    not there to spend (they cost spills inside the loop), so the accumulators start at zero and
+			//    z = f32(dot) * k_scale (a conversion and a multiplication per score); the
+			//    extremes are taken over z as floats, and -- z being small -- the subtrahend ext * |t| - lg2 255 rounds to
+			//    within 4e-6 of its value: no remainder is carried (`fine` is 1) and the value row's weight takes its place
+			//    in the rounding fused multiply-add, P = rne(p * v_weight).  The first wavefront requests the step's 32 key
+			//    scales and 32 value weights with the K tile (one more load in flight per prefetched step: its waits count
+			//    three loads per step).  Scales are taken to be non-negative (absmax / 127): the sign of a query's
+			//    temperature is then the head's.
 			constexpr f32 HEADROOM = 12.0f, LIFT0 = 1.0f / 4096.0f, DOT_BIAS = 12582912.0f;
 			v16i s_bias;
-			X17_UNROLL for (int r = 0; r < 16; ++r) s_bias[r] = 0x4B400000;
-			asm volatile("" : "+v"(s_bias));          // (kept in registers: rebuilding it per step would cost what it saves)
+			X17_UNROLL for (int r = 0; r < 16; ++r) s_bias[r] = ROW_SCALES ? 0 : 0x4B400000;
+			if constexpr (!ROW_SCALES) {
+				asm volatile("" : "+v"(s_bias));      // (kept in registers: rebuilding it per step would cost what it saves)
+			}
 			f32 const abs_t = __builtin_fabsf(temperature);
 			f32 const sgn = positive_temperature ? 1.0f : -1.0f;
-			f32 ext = (f32(sink_dot) + DOT_BIAS) * sgn;
+			f32 ext = ROW_SCALES ? (f32(sink_dot) * 0.125f) * sgn : (f32(sink_dot) + DOT_BIAS) * sgn;
 			f32 mb, fine;
 			auto set_subtrahend = [&]() {
-				// ext * |t| as a rounded product and its exact remainder; prod - mb is exact (neighbouring floats)
-				f32 const prod = ext * abs_t;
-				f32 const low = fmaf32(ext, abs_t, -prod);
-				mb = prod - LOG2_PROB_SCALE;
-				fine = hw::ex2(-(((prod - mb) - LOG2_PROB_SCALE) + low));          // 2^-(what mb leaves over): close to 1
+				if constexpr (ROW_SCALES) {
+					mb = fmaf32(ext, abs_t, -LOG2_PROB_SCALE);
+					fine = 1.0f;
+				} else {
+					// ext * |t| as a rounded product and its exact remainder; prod - mb is exact (neighbouring floats)
+					f32 const prod = ext * abs_t;
+					f32 const low = fmaf32(ext, abs_t, -prod);
+					mb = prod - LOG2_PROB_SCALE;
+					fine = hw::ex2(-(((prod - mb) - LOG2_PROB_SCALE) + low));          // 2^-(what mb leaves over): close to 1
+				}
 			};
 			set_subtrahend();
 			f32 ext_ref = ext;                        // O and the sums refer to the maximum HEADROOM above this extreme's score
@@ -395,8 +411,23 @@ void kernel(
 			u32 const stage_v_next = stage_v_src + TILE_STEP_BYTES;
 			u32 const lds_wave = (u32)(size_t)X17_LDS_PTR(smem) + stage_lds;
 			// SLOT >= 0 also says that tiles s + 3 and s + 4 both exist (the caller's loop bound)
+			// row-scaled build, first wavefront: lane l < 32 fetches the scale of key l of the K tile being requested, lane
+			// 32 + l the weight of its value row (4 bytes per lane, one 256-byte slot of the scale ring)
+			[[maybe_unused]] f32 const *sc_src = nullptr;
+#if X17_ATTN_ROW_SCALES
+			sc_src = (half == 0 ? k_scale : v_weight) + (size_t)head * ((size_t)gridDim.z * seq_len) + row_base
+			         + (size_t)kb_begin * at::KV_PER_STEP + qlane;
+#endif
+#define X17_REQUEST_SCALES(ring_slot) \
+			if (wave == 0) { \
+				__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(sc_src), X17_LDS_PTR(smem + at::SCALE_RING_OFFSET + (ring_slot) * at::SCALE_TILE_BYTES), 4, 0, 0); \
+			}
 			auto request_tiles = [&]<int SLOT>(u32 s) __attribute__((always_inline)) {
 				if constexpr (SLOT >= 0) {
+					if constexpr (ROW_SCALES) {
+						X17_REQUEST_SCALES((SLOT + 3) % 4)
+						sc_src += at::KV_PER_STEP;
+					}
 					if (CPR == 8 || stager) {
 						asm volatile("s_add_i32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
 						             :: "s"(lds_wave), "i"(at::K_RING_OFFSET + ((SLOT + 3) % 4) * at::K_TILE_BYTES), "v"(stage_k_src), "s"(src) : "memory", "m0", "scc");
@@ -406,6 +437,10 @@ void kernel(
 					src += TILE_STEP_BYTES;
 				} else {
 					bool const more = s + 4 < n_steps;
+					if constexpr (ROW_SCALES) {
+						X17_REQUEST_SCALES((s + 3) % at::RING)
+						sc_src += __builtin_amdgcn_readfirstlane(more ? at::KV_PER_STEP : 0u);
+					}
 					if (CPR == 8 || stager) {
 						load_to_lds_16(smem + at::K_RING_OFFSET + ((s + 3) % at::RING) * at::K_TILE_BYTES + stage_lds, src, stage_k_src);
 						load_to_lds_16(smem + at::RAW_V_RING_OFFSET + (s % at::RING) * at::RAW_V_TILE_BYTES + stage_lds, src, more ? stage_v_next : stage_v_src);
@@ -416,7 +451,11 @@ void kernel(
 				}
 			};
 			auto stage = [&]<int SLOT>(u32 i) __attribute__((always_inline)) {
-				__builtin_amdgcn_s_waitcnt(0x0F74);          // vmcnt(4): K tile i and raw V tile i + 1 have landed
+				if (ROW_SCALES && wave == 0) {
+					__builtin_amdgcn_s_waitcnt(0x0F76);      // vmcnt(6): three loads per step in the first wavefront
+				} else {
+					__builtin_amdgcn_s_waitcnt(0x0F74);      // vmcnt(4): K tile i and raw V tile i + 1 have landed
+				}
 				__builtin_amdgcn_s_waitcnt(0xC07F);          // lgkmcnt(0): own LDS traffic of step i-1 is complete
 				__builtin_amdgcn_s_barrier();                // ... and so is everybody else's: tiles i are visible
 				request_tiles.template operator()<SLOT>(i);
@@ -467,7 +506,23 @@ void kernel(
 					f32 y[8];
 					[[maybe_unused]] bool vis[8];
 					f32 tmax;
-					if constexpr (!MASKED) {
+					// row-scaled build: this lane's 8 keys of the tile are 4 * half + {0..3} and 8 + 4 * half + {0..3}
+					[[maybe_unused]] f32 const *sc = nullptr;
+					[[maybe_unused]] f32 z[8];
+					if constexpr (ROW_SCALES) {
+						sc = reinterpret_cast<f32 const *>(smem + at::SCALE_RING_OFFSET + k_slot * at::SCALE_TILE_BYTES) + 16 * tile + 4 * half;
+						v4f const k0 = *reinterpret_cast<v4f const *>(sc), k1 = *reinterpret_cast<v4f const *>(sc + 8);
+						X17_UNROLL for (u32 r = 0; r < 4; ++r) {
+							z[r] = f32(s_acc[8 * tile + r]) * k0[r];
+							z[4 + r] = f32(s_acc[8 * tile + 4 + r]) * k1[r];
+						}
+					}
+					if constexpr (!MASKED && ROW_SCALES) {
+						// (non-negative temperature: sgn = 1)
+						X17_UNROLL for (u32 r = 0; r < 8; ++r) y[r] = z[r];
+						tmax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fmaxf(y[0], y[1]), __builtin_fmaxf(y[2], y[3])),
+						                       __builtin_fmaxf(__builtin_fmaxf(y[4], y[5]), __builtin_fmaxf(y[6], y[7])));
+					} else if constexpr (!MASKED) {
 						// (positive temperature: sgn = 1; the biased scores are positive floats: their order is the order
 						// of their bits as integers)
 						X17_UNROLL for (u32 r = 0; r < 8; ++r) y[r] = u2f((u32)s_acc[8 * tile + r]);
@@ -482,14 +537,14 @@ void kernel(
 						X17_UNROLL for (u32 r = 0; r < 8; ++r) {
 							u32 const distance = first - (8 * (r / 4) + (r % 4));
 							vis[r] = distance <= vis_bound;
-							y[r] = u2f((u32)s_acc[8 * tile + r]) * sgn;
+							y[r] = ROW_SCALES ? z[r] * sgn : u2f((u32)s_acc[8 * tile + r]) * sgn;
 							ym[r] = vis[r] ? y[r] : -__builtin_inff();
 						}
 						tmax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fmaxf(ym[0], ym[1]), __builtin_fmaxf(ym[2], ym[3])),
 						                       __builtin_fmaxf(__builtin_fmaxf(ym[4], ym[5]), __builtin_fmaxf(ym[6], ym[7])));
 					}
 					if (__any(tmax > ext)) {
-						if constexpr (!MASKED) {
+						if constexpr (!MASKED && !ROW_SCALES) {
 							tmax = u2f((u32)pair_max_i32((i32)f2u(tmax)));
 						} else {
 							tmax = __builtin_fmaxf(tmax, partner_f32(tmax, half));
@@ -524,8 +579,14 @@ void kernel(
 					sum_lo = fmaf32((p[0] + p[1]) + (p[2] + p[3]), sum_lift, sum_lo);
 					sum_hi = fmaf32((p[4] + p[5]) + (p[6] + p[7]), sum_lift, sum_hi);
 					v4u pp;
+					[[maybe_unused]] f32 vw[8];
+					if constexpr (ROW_SCALES) {
+						v4f const w0 = *reinterpret_cast<v4f const *>(sc + 32), w1 = *reinterpret_cast<v4f const *>(sc + 40);
+						X17_UNROLL for (u32 r = 0; r < 4; ++r) { vw[r] = w0[r]; vw[4 + r] = w1[r]; }
+					}
 					X17_UNROLL for (int w = 0; w < 4; ++w) {
-						u32 const lo16 = f2u(fmaf32(p[2 * w], fine, PACK_MAGIC)), hi16 = f2u(fmaf32(p[2 * w + 1], fine, PACK_MAGIC));
+						f32 const f_lo = ROW_SCALES ? vw[2 * w] : fine, f_hi = ROW_SCALES ? vw[2 * w + 1] : fine;
+						u32 const lo16 = f2u(fmaf32(p[2 * w], f_lo, PACK_MAGIC)), hi16 = f2u(fmaf32(p[2 * w + 1], f_hi, PACK_MAGIC));
 						u32 const pair = __builtin_amdgcn_perm(hi16, lo16, 0x05040100u);           // f16 (1024 + P) twice
 						pp[w] = __builtin_bit_cast(u32, __builtin_elementwise_fma(__builtin_bit_cast(v2h, pair), lift2, neg_bias2));
 					}
@@ -556,12 +617,20 @@ void kernel(
 			if (CPR == 8 || stager) {
 				load_to_lds_16(smem + at::RAW_V_RING_OFFSET + stage_lds, src, stage_v_src);
 				X17_UNROLL for (u32 j = 0; j < 3; ++j) {
+					if constexpr (ROW_SCALES) {
+						X17_REQUEST_SCALES(j)
+						sc_src += at::KV_PER_STEP;
+					}
 					load_to_lds_16(smem + at::K_RING_OFFSET + j * at::K_TILE_BYTES + stage_lds, src + j * TILE_STEP_BYTES, stage_k_src);
 					load_to_lds_16(smem + at::RAW_V_RING_OFFSET + (j + 1) * at::RAW_V_TILE_BYTES + stage_lds, src + j * TILE_STEP_BYTES, stage_v_next);
 				}
 			}
 			src += 3 * TILE_STEP_BYTES;
-			__builtin_amdgcn_s_waitcnt(0x0F76);   // vmcnt(6): raw V tile 0 has landed
+			if (ROW_SCALES && wave == 0) {
+				__builtin_amdgcn_s_waitcnt(0x0F79);   // vmcnt(9): raw V tile 0 has landed (three loads per later tile)
+			} else {
+				__builtin_amdgcn_s_waitcnt(0x0F76);   // vmcnt(6): raw V tile 0 has landed
+			}
 			widen_v(0, 0);
 			u32 i = 0;
 			for (; i < first_active; ++i) idle_step(i);
@@ -581,7 +650,7 @@ void kernel(
 			__builtin_amdgcn_s_waitcnt(0x0F70);   // the last requests write LDS: they land before the tiles are reused
 			// the partial sums are at the scale of the maximum HEADROOM above ext_ref's score: the common ending below
 			// takes them as if that were the maximum (sgn * ext_ref - 12582912 is that extreme's dot product, exactly)
-			m = fmaf32(fmaf32(ext_ref, sgn, -DOT_BIAS), temperature, HEADROOM);
+			m = ROW_SCALES ? fmaf32(ext_ref * sgn, temperature, HEADROOM) : fmaf32(fmaf32(ext_ref, sgn, -DOT_BIAS), temperature, HEADROOM);
 			lift = 1.0f;
 		} else {
 		// ---- pipeline prologue
