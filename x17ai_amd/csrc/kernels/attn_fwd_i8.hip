@@ -303,6 +303,24 @@ void kernel(
 		f32 sum_hi = 0.25f * PROB_SCALE;     // partial sum of key quad `2 + half`
 		// (the lane pair holds the reference's four partial sums two-and-two; each starts at 63.75)
 		v16f o_acc[D_BLOCKS];                // O^T: lane = query, register r = dim 32*db + 8*(r/4) + 4*half + r%4
+		if constexpr (!STRICT && !ROW_SCALES) {
+			// Speed build: O starts at 255 * sink_v at the scale 2^-12 its accumulation starts from (see below), and the
+			// matrix cores compute that as the outer product (sink_v) x (255 * 2^-12): key slot 0 of the V^T operand
+			// holds the sink value of the lane's dim, key slot 0 of the P^T operand the constant, every other slot is
+			// zero -- one product per element, exact.  (A few instructions per 32 dims instead of a conversion, a fused
+			// multiply-add and a multiplication per element.)
+			typedef short v8s __attribute__((ext_vector_type(8)));
+			_Float16 const p0 = half == 0 ? (_Float16)(PROB_SCALE / 4096.0f) : (_Float16)0.0f;
+			v8s pz = {0, 0, 0, 0, 0, 0, 0, 0};
+			pz[0] = __builtin_bit_cast(short, p0);
+			X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
+				_Float16 const v0 = half == 0 ? (_Float16)(f32)(i32)sink_v[(size_t)head * HD + 32 * db + qlane] : (_Float16)0.0f;
+				v8s vz = {0, 0, 0, 0, 0, 0, 0, 0};
+				vz[0] = __builtin_bit_cast(short, v0);
+				v16f const zero = {0};
+				o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, vz), __builtin_bit_cast(v8h, pz), zero, 0, 0, 0);
+			}
+		} else
 		X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
 			X17_UNROLL for (int r4 = 0; r4 < 4; ++r4) {
 				// 255 * v for the int8 byte v, through the unsigned byte v + 128 (one conversion and one fma per value, all exact)
@@ -386,8 +404,10 @@ void kernel(
 			v2h neg_bias2 = {(_Float16)(-1024.0f * LIFT0), (_Float16)(-1024.0f * LIFT0)};      // -1024 * lift2
 			sum_lo = sum_lo * LIFT0;
 			sum_hi = sum_hi * LIFT0;
-			X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
-				X17_UNROLL for (int r = 0; r < 16; ++r) o_acc[db][r] = o_acc[db][r] * LIFT0;
+			if constexpr (ROW_SCALES) {
+				X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
+					X17_UNROLL for (int r = 0; r < 16; ++r) o_acc[db][r] = o_acc[db][r] * LIFT0;
+				}
 			}
 			u32 const first_active = wave_kb_first - kb_begin;
 			u32 const diagonal = wave_kb_last - kb_begin;
