@@ -184,18 +184,18 @@ void kernel(
 	size_t const row_base = (size_t)seq * seq_len;          // first row of this sequence
 	// position of the block's first query; a last block that would overhang the sequence (lengths are multiples of 64,
 	// src/device/cuda/attn.rs:398-404) starts earlier and recomputes some of its neighbour's queries
-	u32 const q_block0 = q_block_index * at::Q_PER_BLOCK + at::Q_PER_BLOCK > seq_len ? seq_len - at::Q_PER_BLOCK : q_block_index * at::Q_PER_BLOCK;
+	u32 const q_block0 = at::block_first_query(q_block_index, seq_len);
 	u32 const q_wave0 = q_block0 + wave * at::Q_PER_WAVE;
 	u32 const qi = q_wave0 + qlane;                         // this lane's query position
 
 	// cuda/attn_fwd_i8.cuh:408-412 -- window 0 means "no window"; otherwise rounded up to 16
-	u32 const wr = window_size == 0 ? 0xFFFFFFFFu : ((window_size - 1) / 16 + 1) * 16;
+	u32 const wr = at::rounded_window(window_size);
 	u32 const vis_bound = wr - 1 < 0x7FFFFFFFu ? wr - 1 : 0x7FFFFFFFu;
 
 	// key blocks (32 keys) the workgroup walks, and the sub-range this wave needs
-	u32 const kb_begin = (q_block0 - (q_block0 < wr ? q_block0 : wr)) / at::KV_PER_STEP;
-	u32 const kb_end = q_block0 / at::KV_PER_STEP + at::Q_WAVES;             // exclusive
-	u32 const wave_kb_first = (q_wave0 - (q_wave0 < wr ? q_wave0 : wr)) / at::KV_PER_STEP;
+	u32 const kb_begin = at::first_key_block(q_block0, wr);
+	u32 const kb_end = at::end_key_block(q_block0);                          // exclusive
+	u32 const wave_kb_first = at::first_key_block(q_wave0, wr);
 	u32 const wave_kb_last = q_wave0 / at::KV_PER_STEP;                      // inclusive
 
 	for (u32 hh = 0; hh < HPK; ++hh) {
@@ -206,14 +206,12 @@ void kernel(
 		// ---- staging helpers for one 32-key block.  Both K and V travel global -> LDS without passing
 		// through registers (thread t fetches 16-byte chunk t of each tile), PREFETCH steps ahead; one step
 		// before its use a V tile is widened LDS -> LDS by the threads that fetched it.
-		bool const stager = tid < 32 * CPR;
+		bool const stager = at::is_stager(tid);
 		u32 stage_k_src = 0, stage_v_src = 0, widen_dst = 0;
 		if (stager) {
-			// lane `tid` fills stored chunk `tid` of the K tile; find which logical chunk lives there
-			u32 line = tid >> 3;
-			u32 n = (line << 3) | ((tid & 7) ^ ((line >> 1) & 7));
-			stage_k_src = (n / CPR) * KV_STRIDE + (n % CPR) * 16;
-			stage_v_src = (tid / CPR) * KV_STRIDE + HD + (tid % CPR) * 16;
+			// lane `tid` fills stored chunk `tid` of the K tile (attn_tile.h finds which logical chunk lives there)
+			stage_k_src = at::stage_k_offset(tid, KV_STRIDE);
+			stage_v_src = at::stage_v_offset(tid, KV_STRIDE);
 			widen_dst = v_granule_offset(tid / CPR, tid % CPR);
 		}
 		u32 const stage_lds = wave * 1024;                // wave-uniform part of the direct-to-LDS address
@@ -456,7 +454,7 @@ void kernel(
 					}
 					src += TILE_STEP_BYTES;
 				} else {
-					bool const more = s + 4 < n_steps;
+					bool const more = at::further_tile_exists(s, n_steps);
 					if constexpr (ROW_SCALES) {
 						X17_REQUEST_SCALES((s + 3) % at::RING)
 						sc_src += __builtin_amdgcn_readfirstlane(more ? at::KV_PER_STEP : 0u);

@@ -407,16 +407,16 @@ struct NaturalWriters {
 // and serves a ds_read_b128 sixteen lanes at a time, so sixteen consecutive rows must land in sixteen
 // different 16-byte slots of the bank line: with 128-byte rows two rows share a bank line and the row
 // PAIR index has to be mixed in, with 64-byte rows the row QUAD index.
-constexpr u32 CHUNKS = gt::K_STEP / 16;
-constexpr u32 SWZ_SHIFT = gt::K_STEP == 128 ? 1 : 2;
-constexpr u32 UNIT_ROWS = 64 / CHUNKS;                      // rows one 64-lane x 16-byte direct-to-LDS load fills
+constexpr u32 CHUNKS = gt::CHUNKS;
+constexpr u32 SWZ_SHIFT = gt::SWZ_SHIFT;
+constexpr u32 UNIT_ROWS = gt::UNIT_ROWS;                    // rows one 64-lane x 16-byte direct-to-LDS load fills
 // With eight waves, two per SIMD, only the first of each pair (waves 0 .. 3) requests tiles.  The arbiter serves
 // that wave first: with the loads shared evenly it ended its step early and sat at the barrier while its partner,
 // the same loads to issue between its MFMAs, finished alone.  (Splitting the weight units 6:2, 4:4, 2:6 or 0:8
 // between the two measured the same as 8:0.)
-constexpr u32 LOADER_WAVES = WAVES == 8 ? 4 : WAVES;      // (a four-wave workgroup has one wave per SIMD)
-constexpr u32 X_UNITS = gt::M_PER_BLOCK / UNIT_ROWS / LOADER_WAVES; // such loads per loading wave, step and tile
-constexpr u32 W_UNITS = gt::N_PER_BLOCK / UNIT_ROWS / LOADER_WAVES;
+constexpr u32 LOADER_WAVES = gt::LOADER_WAVES;            // (a four-wave workgroup has one wave per SIMD)
+constexpr u32 X_UNITS = gt::X_UNITS;                      // such loads per loading wave, step and tile
+constexpr u32 W_UNITS = gt::W_UNITS;
 constexpr u32 LOADS_PER_STAGE = X_UNITS + W_UNITS;
 static_assert((X_UNITS * UNIT_ROWS) % 16 == 0 && (W_UNITS * UNIT_ROWS) % 16 == 0, "a wave's share must keep the swizzle phase");
 
@@ -427,10 +427,7 @@ constexpr bool LANE_UNIT_OFFSETS = gt::WAVES_PER_SIMD == 1;
 constexpr u32 X_OFFSETS = LANE_UNIT_OFFSETS ? X_UNITS : 2;
 constexpr u32 W_OFFSETS = LANE_UNIT_OFFSETS ? W_UNITS : 2;
 X17_DEV constexpr u32 w_unit_row(u32 r0) {   // weight row that LDS weight row r0 (a multiple of the unit) starts from
-	if (NATURAL_COLS) {
-		return r0;
-	}
-	return gt::WAVE_N * (r0 / gt::WAVE_N) + 16 * ((r0 % gt::WAVE_N) / 32) + 4 * ((r0 % 32) / 8);
+	return gt::w_unit_row(r0, NATURAL_COLS);
 }
 struct LaneOffsets {
 	u32 x_src[X_OFFSETS];   // per-lane byte offset into A for a direct-to-LDS load (even / odd load unit, or per unit)
@@ -831,22 +828,9 @@ void kernel(
 	u32 const n_groups = gridDim.x * gridDim.y * gridDim.z;
 	u32 const group = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
 	auto tile_coords = [&](u32 lin, u32 &tile_m, u32 &tile_n) {
-#ifdef X17_GEMM_BAND
-		constexpr u32 BAND = X17_GEMM_BAND;
-#else
-		constexpr u32 BAND = 2048 / gt::M_PER_BLOCK;
-#endif
-		if (total % 8 == 0) {
-			lin = (lin % 8) * (total / 8) + lin / 8;
-		}
-		u32 band_tiles = BAND * tiles_n;
-		u32 band = lin / band_tiles;
-		u32 in_band = lin % band_tiles;
-		u32 rows_in_band = (tiles_m - band * BAND) < BAND ? (tiles_m - band * BAND) : BAND;
-		tile_m = (band * BAND + in_band % rows_in_band) * gt::M_PER_BLOCK;
-		tile_n = (in_band / rows_in_band) * gt::N_PER_BLOCK;
-		tile_m = tile_m + gt::M_PER_BLOCK > a_rows ? a_rows - gt::M_PER_BLOCK : tile_m;
-		tile_n = tile_n + gt::N_PER_BLOCK > N_RAW ? N_RAW - gt::N_PER_BLOCK : tile_n;
+		gt::TileOrigin const o = gt::tile_origin(lin, a_rows, N_RAW, gt::BAND);
+		tile_m = o.m;
+		tile_n = o.n;
 	};
 	if (group >= total) {
 		return;
@@ -860,13 +844,12 @@ void kernel(
 
 	LaneOffsets lo;
 	{
-		u32 j = lane / CHUNKS, p = lane % CHUNKS;     // row inside a load unit, stored chunk position
+		// (row inside a load unit and logical chunk of the stored chunk position: gemm_tile.h)
 		u32 even_odd_x[2], even_odd_w[2];
 		X17_UNROLL for (u32 odd = 0; odd < 2; ++odd) {
-			u32 key = ((odd * UNIT_ROWS + j) >> SWZ_SHIFT) & (CHUNKS - 1);
-			u32 chunk = p ^ key;
-			even_odd_x[odd] = j * K_TOTAL + 16 * chunk;
-			even_odd_w[odd] = (NATURAL_COLS ? j : (gt::WAVE_N / 2) * ((j >> 2) & 1) + 4 * (j >> 3) + (j & 3)) * K_TOTAL + 16 * chunk;
+			u32 const chunk = gt::lane_chunk(lane, odd);
+			even_odd_x[odd] = gt::x_lane_row(lane) * K_TOTAL + 16 * chunk;
+			even_odd_w[odd] = gt::w_lane_row(lane, NATURAL_COLS) * K_TOTAL + 16 * chunk;
 		}
 		if constexpr (LANE_UNIT_OFFSETS) {
 			u32 const w_first = wave * W_UNITS * UNIT_ROWS;

@@ -63,6 +63,61 @@ constexpr unsigned MAX_BLOCKS = 256;
 // (two workgroups per compute unit when a workgroup has four waves); 128 x 128 waves need all 512.
 constexpr unsigned WAVES_PER_SIMD = (WAVE_M / 32) * (WAVE_N / 32) <= 8 ? 2 : 1;
 
+// ---- index arithmetic of the tile requests (global -> LDS, 16 bytes per lane).  The kernel calls these; so does the
+// host-side audit (gemm_requests_audit.cpp), which enumerates every request of a launch on the CPU and checks that it
+// stays inside its operand.
+// LDS rows hold K_STEP bytes = CHUNKS chunks of 16; one 64-lane load fills UNIT_ROWS rows ("a load unit").
+constexpr unsigned CHUNKS = K_STEP / 16;
+constexpr unsigned SWZ_SHIFT = K_STEP == 128 ? 1 : 2;
+constexpr unsigned UNIT_ROWS = 64 / CHUNKS;
+// With eight waves, two per SIMD, only the first of each pair (waves 0 .. 3) requests tiles.
+constexpr unsigned LOADER_WAVES = WAVES_M * WAVES_N == 8 ? 4 : WAVES_M * WAVES_N;
+constexpr unsigned X_UNITS = M_PER_BLOCK / UNIT_ROWS / LOADER_WAVES;   // load units per loading wave, step and tile
+constexpr unsigned W_UNITS = N_PER_BLOCK / UNIT_ROWS / LOADER_WAVES;
+// The weight row that LDS weight row r0 (a multiple of UNIT_ROWS) starts from.  With WN = WAVE_N columns per wave, LDS
+// weight row R = WN*wn + 32*bn + i holds weight row WN*wn + (WN/2)*((i/4)%2) + 16*bn + 4*(i/8) + i%4 (so that a lane
+// collects consecutive output columns); the head-normalising writers keep the natural order.
+constexpr unsigned w_unit_row(unsigned r0, bool natural) {
+	return natural ? r0 : WAVE_N * (r0 / WAVE_N) + 16 * ((r0 % WAVE_N) / 32) + 4 * ((r0 % 32) / 8);
+}
+// Row inside its load unit, as an operand row offset, and 16-byte chunk of the K step that lane `lane` fetches
+// (`odd`: parity of the unit, which shifts the swizzle phase).
+constexpr unsigned x_lane_row(unsigned lane) { return lane / CHUNKS; }
+constexpr unsigned w_lane_row(unsigned lane, bool natural) {
+	unsigned const j = lane / CHUNKS;
+	return natural ? j : (WAVE_N / 2) * ((j >> 2) & 1) + 4 * (j >> 3) + (j & 3);
+}
+constexpr unsigned lane_chunk(unsigned lane, unsigned odd) {
+	unsigned const j = lane / CHUNKS, p = lane % CHUNKS;
+	return p ^ (((odd * UNIT_ROWS + j) >> SWZ_SHIFT) & (CHUNKS - 1));
+}
+// First token row and first raw column of tile `lin` of the persistent walk: each XCD (the hardware deals workgroups
+// round-robin to 8 of them) gets a contiguous run of tiles, walked in bands of `band` token tiles; a last tile that
+// would overhang the matrix is moved back to end at its edge.
+struct TileOrigin { unsigned m, n; };
+constexpr TileOrigin tile_origin(unsigned lin, unsigned a_rows, unsigned n_raw, unsigned band) {
+	unsigned const tiles_m = (a_rows + M_PER_BLOCK - 1) / M_PER_BLOCK;
+	unsigned const tiles_n = (n_raw + N_PER_BLOCK - 1) / N_PER_BLOCK;
+	unsigned const total = tiles_m * tiles_n;
+	if (total % 8 == 0) {
+		lin = (lin % 8) * (total / 8) + lin / 8;
+	}
+	unsigned const band_tiles = band * tiles_n;
+	unsigned const b = lin / band_tiles;
+	unsigned const in_band = lin % band_tiles;
+	unsigned const rows_in_band = (tiles_m - b * band) < band ? (tiles_m - b * band) : band;
+	unsigned m = (b * band + in_band % rows_in_band) * M_PER_BLOCK;
+	unsigned n = (in_band / rows_in_band) * N_PER_BLOCK;
+	m = m + M_PER_BLOCK > a_rows ? a_rows - M_PER_BLOCK : m;
+	n = n + N_PER_BLOCK > n_raw ? n_raw - N_PER_BLOCK : n;
+	return TileOrigin{m, n};
+}
+#ifdef X17_GEMM_BAND
+constexpr unsigned BAND = X17_GEMM_BAND;
+#else
+constexpr unsigned BAND = 2048 / M_PER_BLOCK;
+#endif
+
 static_assert(M_PER_BLOCK == 128 || M_PER_BLOCK == 256, "tokens per workgroup: 128 or 256");
 static_assert(WAVE_M == 64 || WAVE_M == 128, "a wave owns 64 or 128 tokens");
 static_assert(WAVE_N == 128 || WAVE_N == 64, "a wave owns 128 or 64 raw output columns");
