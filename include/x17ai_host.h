@@ -130,6 +130,11 @@ typedef struct X17hAttnConfig {
 	 * the kernel whose q/k/v codes carry one f32 scale per (row, head); out_dtype is then X17H_INT8
 	 * (FixedI8 codes) or X17H_BF16 (real values), otherwise X17H_INT8 */
 	int row_scales; int out_dtype;
+	/* backward_q != 0 builds the backward-with-respect-to-q kernel of this configuration instead of the forward
+	 * (launched with x17h_attn_kernel_launch_d_q).  The reference's attn_d_q.cuh:1-410 is its bf16 generation; the
+	 * int8 generation has no backward there yet, so the operands are defined here: the forward's q, kv, sinks and
+	 * temperatures, its FixedI8 output and log-sum-exp L, dO as bf16 -> dQ as bf16 (with respect to the real q) */
+	int backward_q;
 } X17hAttnConfig;
 /* AttnKernel::new, attn.rs:170-232 */
 int x17h_attn_kernel_new(X17hDevice *dev, char const *kernel_name, X17hAttnConfig const *config, X17hAttnKernel **out);
@@ -148,6 +153,13 @@ int x17h_attn_kernel_launch_row_scaled(X17hAttnKernel *k, X17hTensor *q, X17hTen
                                        X17hTensor *l, size_t window_size, size_t batch,
                                        X17hTensor *q_scale, X17hTensor *k_scale, X17hTensor *v_weight,
                                        X17hTensor *sink_v_weight, X17hTensor *out_scale);
+/* Launch of a kernel built with backward_q (structure of attn_d_q.cuh:70-383: P from L, D = rowsum(dO * O) written to
+ * `d` for a later dK/dV kernel, dS = P (dP - D), dQ = dS . K).  out: the forward's output i8 [rows, o_stride];
+ * d_out: bf16 [rows, o_stride]; d_q: bf16 [rows, q_stride] (written); l: f32 [n_heads, rows]; d: f32 [n_heads, rows]
+ * (written; may be NULL). */
+int x17h_attn_kernel_launch_d_q(X17hAttnKernel *k, X17hTensor *q, X17hTensor *kv, X17hTensor *sink_k, X17hTensor *sink_v,
+                                X17hTensor *attn_temperature, X17hTensor *out, X17hTensor *d_out, X17hTensor *d_q,
+                                X17hTensor *l, X17hTensor *d, size_t window_size, size_t batch);
 /* AttnKernelConfig::n_ops, attn.rs:72-84 */
 double x17h_attn_kernel_n_ops(X17hAttnKernel *k, size_t seq_len, size_t window_size);
 int x17h_attn_kernel_metadata(X17hAttnKernel *k, size_t out[3]);

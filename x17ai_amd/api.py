@@ -351,6 +351,8 @@ class AttnKernelConfig:         # attn.rs:45-84
 	# extension: q/k/v codes with one f32 scale per (row, head); out_dtype INT8 (FixedI8) or, with row scales, BF16
 	row_scales: bool = False
 	out_dtype: int = INT8
+	# builds the backward-with-respect-to-q kernel (attn_d_q_i8.hip) instead of the forward: AttnKernel.launch_d_q
+	backward_q: bool = False
 
 	def heads_per_kernel(self) -> int:
 		return 1 if self.head_dim == 0 else max(128 // self.head_dim, 1)
@@ -364,7 +366,7 @@ class AttnKernel:
 
 	def __init__(self, device: Optional[Device], kernel_name: str, config: AttnKernelConfig, strict_math: bool = True):
 		c = _ffi.AttnConfigC(config.dtype, config.n_heads, config.head_dim, config.q_stride, config.kv_stride,
-		                     config.o_stride, int(strict_math), int(config.row_scales), config.out_dtype)
+		                     config.o_stride, int(strict_math), int(config.row_scales), config.out_dtype, int(config.backward_q))
 		self.device = device
 		self.name = kernel_name
 		self.config = config
@@ -386,6 +388,14 @@ class AttnKernel:
 		check(_ffi.host().x17h_attn_kernel_launch_row_scaled(
 			self._h, q._h, kv._h, sink_k._h, sink_v._h, attn_temperature._h, out._h, l._h if l is not None else None,
 			window_size, batch, q_scale._h, k_scale._h, v_weight._h, sink_v_weight._h, out_scale._h))
+
+	def launch_d_q(self, q: Tensor, kv: Tensor, sink_k: Tensor, sink_v: Tensor, attn_temperature: Tensor, out: Tensor,
+	               d_out: Tensor, d_q: Tensor, l: Tensor, d: Optional[Tensor], window_size: int, batch: int = 1) -> None:
+		"""Launch of a kernel built with config.backward_q: the forward's operands, its output `out` (i8) and
+		log-sum-exp `l`, dO `d_out` (bf16) -> dQ `d_q` (bf16, with respect to the real q) and D `d` (f32 [H, rows])."""
+		check(_ffi.host().x17h_attn_kernel_launch_d_q(
+			self._h, q._h, kv._h, sink_k._h, sink_v._h, attn_temperature._h, out._h, d_out._h, d_q._h, l._h,
+			d._h if d is not None else None, window_size, batch))
 
 	def n_ops(self, seq_len: int, window_size: int) -> float:
 		return float(_ffi.host().x17h_attn_kernel_n_ops(self._h, seq_len, window_size))

@@ -580,7 +580,7 @@ namespace kernel_build {
 		uint64_t h = 0xCBF29CE484222325ull;
 		h = fnv1a(h, common_text);
 		h = fnv1a(h, device_flags());
-		char const *deps[] = {"x17_device.h", "gemm_tile.h", "attn_tile.h", "rms_norm_tile.h", "decode_tile.h"};
+		char const *deps[] = {"x17_device.h", "gemm_tile.h", "attn_tile.h", "rms_norm_tile.h", "decode_tile.h", "attn_bwd_tile.h"};
 		std::string text;
 		for (char const *d : deps) {
 			if (read_file(kdir + "/" + d, text)) h = fnv1a(h, text);
@@ -1095,7 +1095,12 @@ std::unique_ptr<AttnKernel> AttnKernel::create(std::shared_ptr<HipDevice> device
 	if (config.row_scales) {
 		common << "#define X17_ATTN_ROW_SCALES 1\n#define X17_ATTN_OUT_BF16 " << (config.out_dtype == DType::Bf16 ? 1 : 0) << "\n";
 	}
-	auto built = kernel_build::build(kernel_name, common.str(), "attn_fwd_i8.hip", "attn_meta.cpp", diag);
+	if (config.backward_q && (config.row_scales || config.out_dtype != DType::Int8)) {
+		diag.add_error("the attention backward kernel takes FixedI8 operands at the fixed scale (no row scales, i8 forward output)");
+		return nullptr;
+	}
+	auto built = config.backward_q ? kernel_build::build(kernel_name, common.str(), "attn_d_q_i8.hip", "attn_bwd_meta.cpp", diag)
+	                               : kernel_build::build(kernel_name, common.str(), "attn_fwd_i8.hip", "attn_meta.cpp", diag);
 	if (!built) return nullptr;
 	auto meta = kernel_build::read_metadata_json(built->meta_json_path, diag);
 	if (!meta) return nullptr;
@@ -1121,6 +1126,7 @@ std::unique_ptr<AttnKernel> AttnKernel::create(std::shared_ptr<HipDevice> device
 // attn.rs:353-447
 Status AttnKernel::launch(AttnKernelArgs const &a) {
 	if (!device || !kernel) return Status::err(TensorOpError::Other, "attention kernel " + name + " was built without a device");
+	if (config.backward_q) return Status::err(TensorOpError::Other, "attention kernel " + name + " is a backward kernel: use launch_d_q");
 	size_t shp[2], tmp[2];
 	Status s = tensor_check::matrix_shape("attention", "q", *a.q, std::nullopt, config.q_stride, *device, config.dtype, shp);
 	if (!s.is_ok()) return s;
@@ -1191,6 +1197,63 @@ Status AttnKernel::launch(AttnKernelArgs const &a) {
 	// the plain kernel takes the first nine arguments only
 	void *raw_args[14] = {&seq_len_arg, &q_ptr, &kv_ptr, &sk, &sv, &tp, &out_ptr, &l_ptr, &window_arg,
 	                      &scale_ptrs[0], &scale_ptrs[1], &scale_ptrs[2], &scale_ptrs[3], &scale_ptrs[4]};
+	size_t grid[3] = {(seq_len + metadata.Q_PER_BLOCK - 1) / metadata.Q_PER_BLOCK, config.head_group_cnt(), a.batch};
+	size_t block[3] = {metadata.THREADS_PER_BLOCK, 1, 1};
+	return kernel->launch(*device->stream, grid, block, metadata.SMEM_BYTES, raw_args);
+}
+
+// The backward with respect to q: the forward's inputs, its output and log-sum-exp, and dO (bf16) -> dQ (bf16), D.
+Status AttnKernel::launch_d_q(AttnKernelArgs const &a) {
+	if (!device || !kernel) return Status::err(TensorOpError::Other, "attention kernel " + name + " was built without a device");
+	if (!config.backward_q) return Status::err(TensorOpError::Other, "attention kernel " + name + " is a forward kernel");
+	if (a.l == nullptr || a.d_out == nullptr || a.d_q == nullptr) {
+		return Status::err(TensorOpError::Other, "attention backward needs l, d_out and d_q");
+	}
+	char const *op = "attention backward";
+	size_t shp[2], tmp[2];
+	Status s = tensor_check::matrix_shape(op, "q", *a.q, std::nullopt, config.q_stride, *device, config.dtype, shp);
+	if (!s.is_ok()) return s;
+	size_t const rows = shp[0];
+	s = tensor_check::matrix_shape(op, "kv", *a.kv, rows, config.kv_stride, *device, config.dtype, tmp);
+	if (!s.is_ok()) return s;
+	s = tensor_check::matrix_shape(op, "sink_k", *a.sink_k, config.n_heads, config.head_dim, *device, config.dtype, tmp);
+	if (!s.is_ok()) return s;
+	s = tensor_check::matrix_shape(op, "sink_v", *a.sink_v, config.n_heads, config.head_dim, *device, config.dtype, tmp);
+	if (!s.is_ok()) return s;
+	s = tensor_check::vector_shape(op, "attn_temperature", *a.attn_temperature, config.n_heads, *device, DType::F32);
+	if (!s.is_ok()) return s;
+	s = tensor_check::matrix_shape(op, "out", *a.out, rows, config.o_stride, *device, DType::Int8, tmp);
+	if (!s.is_ok()) return s;
+	s = tensor_check::matrix_shape(op, "d_out", *a.d_out, rows, config.o_stride, *device, DType::Bf16, tmp);
+	if (!s.is_ok()) return s;
+	s = tensor_check::matrix_shape(op, "d_q", *a.d_q, rows, config.q_stride, *device, DType::Bf16, tmp);
+	if (!s.is_ok()) return s;
+	s = tensor_check::matrix_shape(op, "l", *a.l, config.n_heads, rows, *device, DType::F32, tmp);
+	if (!s.is_ok()) return s;
+	if (a.d != nullptr) {
+		s = tensor_check::matrix_shape(op, "d", *a.d, config.n_heads, rows, *device, DType::F32, tmp);
+		if (!s.is_ok()) return s;
+	}
+	for (Tensor const *in : {a.q, a.kv, a.out, a.d_out}) {
+		if (overlaps(*a.d_q, *in)) return Status::err(TensorOpError::Other, "attention backward output d_q must not share memory with an input");
+	}
+	if (a.batch == 0 || rows % a.batch != 0) {
+		return Status::err(TensorOpError::Other, "attention rows (" + std::to_string(rows) + ") must be divisible by batch (" + std::to_string(a.batch) + ")");
+	}
+	size_t const seq_len = rows / a.batch;
+	if (seq_len % 64 != 0 || seq_len < metadata.Q_PER_BLOCK) {
+		return Status::err(TensorOpError::Other, "attention seq_len must be divisible by 64 (as in the reference) and hold at least one query block of "
+			+ std::to_string(metadata.Q_PER_BLOCK) + ", got " + std::to_string(seq_len));
+	}
+	if (a.window_size > 0 && a.window_size % 16 != 0) {
+		return Status::err(TensorOpError::Other, "attention window_size must be zero or divisible by 16, got " + std::to_string(a.window_size));
+	}
+	if (rows > 0xFFFFFFFFull || a.window_size > 0xFFFFFFFFull) return Status::err(TensorOpError::Other, "attention sizes exceed 32 bits");
+	size_t seq_len_arg = seq_len, window_arg = a.window_size;
+	void *q_ptr = a.q->ptr, *kv_ptr = a.kv->ptr, *sk = a.sink_k->ptr, *sv = a.sink_v->ptr, *tp = a.attn_temperature->ptr;
+	void *out_ptr = a.out->ptr, *do_ptr = a.d_out->ptr, *dq_ptr = a.d_q->ptr, *l_ptr = a.l->ptr;
+	void *d_ptr = a.d != nullptr ? a.d->ptr : nullptr;
+	void *raw_args[12] = {&seq_len_arg, &q_ptr, &kv_ptr, &sk, &sv, &tp, &out_ptr, &do_ptr, &dq_ptr, &l_ptr, &d_ptr, &window_arg};
 	size_t grid[3] = {(seq_len + metadata.Q_PER_BLOCK - 1) / metadata.Q_PER_BLOCK, config.head_group_cnt(), a.batch};
 	size_t block[3] = {metadata.THREADS_PER_BLOCK, 1, 1};
 	return kernel->launch(*device->stream, grid, block, metadata.SMEM_BYTES, raw_args);
@@ -1576,7 +1639,7 @@ int x17h_attn_kernel_new(X17hDevice *dev, char const *kernel_name, X17hAttnConfi
 		if (!valid_dtype(c->dtype)) return fail("unknown dtype");
 		if (!valid_dtype(c->out_dtype)) return fail("unknown out_dtype");
 		AttnKernelConfig cfg{DType(c->dtype), c->n_heads, c->head_dim, c->q_stride, c->kv_stride, c->o_stride,
-		                     c->row_scales != 0, DType(c->out_dtype)};
+		                     c->row_scales != 0, DType(c->out_dtype), c->backward_q != 0};
 		Diagnostics diag;
 		auto k = AttnKernel::create(dev != nullptr ? dev->dev : nullptr, kernel_name, cfg, c->strict_math != 0, diag);
 		if (!k) return fail_diag("attention", diag);
@@ -1603,6 +1666,19 @@ int x17h_attn_kernel_launch_row_scaled(X17hAttnKernel *k, X17hTensor *q, X17hTen
 	                 l != nullptr ? l->t.get() : nullptr, window_size, batch,
 	                 q_scale->t.get(), k_scale->t.get(), v_weight->t.get(), sink_v_weight->t.get(), out_scale->t.get()};
 	return from_status(k->k->launch(a));
+}
+int x17h_attn_kernel_launch_d_q(X17hAttnKernel *k, X17hTensor *q, X17hTensor *kv, X17hTensor *sink_k, X17hTensor *sink_v,
+                                X17hTensor *temp, X17hTensor *out, X17hTensor *d_out, X17hTensor *d_q, X17hTensor *l, X17hTensor *d,
+                                size_t window_size, size_t batch) {
+	if (q == nullptr || kv == nullptr || sink_k == nullptr || sink_v == nullptr || temp == nullptr || out == nullptr
+	    || d_out == nullptr || d_q == nullptr || l == nullptr) {
+		return fail("attention backward launch needs q, kv, the sinks, the temperatures, out, d_out, d_q and l");
+	}
+	AttnKernelArgs args{q->t.get(), kv->t.get(), sink_k->t.get(), sink_v->t.get(), temp->t.get(), out->t.get(), l->t.get(), window_size, batch};
+	args.d_out = d_out->t.get();
+	args.d_q = d_q->t.get();
+	args.d = d != nullptr ? d->t.get() : nullptr;
+	return from_status(k->k->launch_d_q(args));
 }
 double x17h_attn_kernel_n_ops(X17hAttnKernel *k, size_t seq_len, size_t window_size) { return k->k->config.n_ops(seq_len, window_size); }
 int x17h_attn_kernel_metadata(X17hAttnKernel *k, size_t out[3]) {

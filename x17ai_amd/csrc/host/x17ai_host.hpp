@@ -254,6 +254,9 @@ struct AttnKernelConfig {
 	// out_dtype is Int8 (FixedI8 codes) or, in the row-scaled build only, Bf16 (real values).
 	bool row_scales = false;
 	DType out_dtype = DType::Int8;
+	// Builds the backward-with-respect-to-q kernel (attn_d_q_i8.hip; the reference's attn_d_q.cuh is its bf16
+	// generation) instead of the forward: launched through AttnKernel::launch_d_q.
+	bool backward_q = false;
 	size_t heads_per_kernel() const;
 	size_t head_group_cnt() const;
 	size_t head_group_dim() const;
@@ -268,6 +271,9 @@ struct AttnKernelArgs {
 	// row-scaled kernels only: f32 [n_heads, rows] scales of q and k, weights (<= 1) of the value rows, and per head
 	// the weight of the sink value and the output scale
 	Tensor const *q_scale = nullptr, *k_scale = nullptr, *v_weight = nullptr, *sink_v_weight = nullptr, *out_scale = nullptr;
+	// backward_q kernels only: `out` is the forward's output (an input here), `l` its log-sum-exp (required);
+	// d_out bf16 [rows, o_stride] in, d_q bf16 [rows, q_stride] out, d f32 [n_heads, rows] out (may be null)
+	Tensor const *d_out = nullptr, *d_q = nullptr, *d = nullptr;
 };
 
 struct AttnLauncherMetadata { size_t THREADS_PER_BLOCK, SMEM_BYTES, Q_PER_BLOCK; };
@@ -282,6 +288,7 @@ struct AttnKernel {
 	static std::unique_ptr<AttnKernel> create(std::shared_ptr<HipDevice> device, std::string const &kernel_name,
 	                                           AttnKernelConfig const &config, bool strict_math, Diagnostics &diag);
 	Status launch(AttnKernelArgs const &args);
+	Status launch_d_q(AttnKernelArgs const &args);
 };
 
 // ---------------------------------------------------------------- rms_norm, decode
@@ -312,6 +319,9 @@ struct AttnDecodeArgs {
 	size_t window_size;
 	// row-scaled kernels only: q_scale [S, H], k_scale and v_weight [S, H, capacity], sink_v_weight and out_scale [H]
 	Tensor const *q_scale = nullptr, *k_scale = nullptr, *v_weight = nullptr, *sink_v_weight = nullptr, *out_scale = nullptr;
+	// backward_q kernels only: `out` is the forward's output (an input here), `l` its log-sum-exp (required);
+	// d_out bf16 [rows, o_stride] in, d_q bf16 [rows, q_stride] out, d f32 [n_heads, rows] out (may be null)
+	Tensor const *d_out = nullptr, *d_q = nullptr, *d = nullptr;
 };
 
 struct AttnDecodeKernel {

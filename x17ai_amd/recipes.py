@@ -82,6 +82,14 @@ def attn_kernel(device: Optional[Device], n_heads: int, head_dim: int, strict: b
 	return AttnKernel(device, f"attn_fwd_i8-h{n_heads}-hd{head_dim}-{_mode(strict)}", cfg, strict)
 
 
+def attn_d_q_kernel(device: Optional[Device], n_heads: int, head_dim: int, strict: bool = True) -> AttnKernel:
+	"""The backward of attn_kernel with respect to q (structure of the reference's attn_d_q.cuh:70-383 on the int8
+	generation's forward): launch_d_q(q, kv, sink_k, sink_v, temperatures, out, d_out, d_q, l, d, window)."""
+	w = n_heads * head_dim
+	cfg = AttnKernelConfig(INT8, n_heads, head_dim, w, 2 * w, w, False, INT8, True)
+	return AttnKernel(device, f"attn_d_q_i8-h{n_heads}-hd{head_dim}-{_mode(strict)}", cfg, strict)
+
+
 def attn_row_scaled_kernel(device: Optional[Device], n_heads: int, head_dim: int, out_dtype: int = BF16,
                            strict: bool = True) -> AttnKernel:
 	"""The attention kernel over int8 codes with one scale per (row, head) -- symmetric absmax / 127
