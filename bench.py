@@ -358,6 +358,22 @@ def extras(dev, X, recipes):
 			c4[name + "_frac_of_int8_peak"] = c4[name + "_tops"] / PEAK_INT8_TOPS
 	c4["ffn_y_f8_frac_of_f16_peak"] = c4["ffn_y_f8_tops"] / PEAK_F16_TFLOPS
 	out["config4_block_stages"] = c4
+	# the attention backward with respect to q at the same attention shape (first kernel of the backward path)
+	rowsb = T * B
+	qb_ = X.Tensor.from_numpy(dev, _rand_codes(rng, (rowsb, H * HD)), X.INT8)
+	kvb = X.Tensor.from_numpy(dev, _rand_codes(rng, (rowsb, 2 * H * HD)), X.INT8)
+	skb = X.Tensor.from_numpy(dev, _rand_codes(rng, (H, HD)), X.INT8)
+	svb = X.Tensor.from_numpy(dev, _rand_codes(rng, (H, HD)), X.INT8)
+	tpb = X.Tensor.from_numpy(dev, (0.5 + rng.random(H)).astype(np.float32), X.F32)
+	ob, lb = X.Tensor(dev, (rowsb, H * HD), X.INT8), X.Tensor(dev, (H, rowsb), X.F32)
+	recipes.attn_kernel(dev, H, HD, False).launch(qb_, kvb, skb, svb, tpb, ob, lb, W, B)
+	dob = X.Tensor.from_numpy(dev, (rng.standard_normal((rowsb, H * HD), dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16), X.BF16)
+	dqb, ddb = X.Tensor(dev, (rowsb, H * HD), X.BF16), X.Tensor(dev, (H, rowsb), X.F32)
+	kb_ = recipes.attn_d_q_kernel(dev, H, HD, False)
+	med, _ = _median_launch(dev, X, lambda: kb_.launch_d_q(qb_, kvb, skb, svb, tpb, ob, dob, dqb, lb, ddb, W, B), ATTN_TIMED, ATTN_WARM)
+	out["config4_attn_d_q"] = {"median_us": med * 1e6, "tops": 6.0 * HD * H * B * pairs / med / 1e12,
+	                           "note": "QK on the int8 matrix cores, dP and dQ on the f16 cores: 6 hd multiply-adds per visible (query, key) pair"}
+	del qb_, kvb, ob, lb, dob, dqb, ddb
 
 	# ---- config 1: attention T=1024, H=8, hd=64, W=256
 	T1, H1, HD1, W1 = 1024, 8, 64, 256
@@ -490,6 +506,38 @@ def single(dev, X, recipes, name, iters):
 		k = recipes.attn_kernel(dev, H, HD, False)
 		pairs = W * (W - 1) // 2 + (T - W) * W
 		fn, work, unit = (lambda: k.launch(q, kv, sk, sv, tp, o, l, W, B)), 4.0 * HD * H * B * pairs / 1e12, "TOPS"
+	elif name == "attn_row_scaled_config5":
+		T, H, HD, W = 65536, 32, 128, 4096
+		q = X.Tensor.from_numpy(dev, _rand_codes(rng, (T, H * HD)), X.INT8)
+		kv = X.Tensor.from_numpy(dev, _rand_codes(rng, (T, 2 * H * HD)), X.INT8)
+		sk = X.Tensor.from_numpy(dev, _rand_codes(rng, (H, HD)), X.INT8)
+		sv = X.Tensor.from_numpy(dev, _rand_codes(rng, (H, HD)), X.INT8)
+		tp = X.Tensor.from_numpy(dev, np.ones(H, np.float32), X.F32)
+		scales = [(0.125 * (0.75 + 0.5 * rng.random((H, T)))).astype(np.float32) for _ in range(3)]
+		vw, sw, osc = recipes.attn_row_scale_operands(scales[2], X.BF16)
+		rs = [X.Tensor.from_numpy(dev, np.ascontiguousarray(a, dtype=np.float32), X.F32) for a in (scales[0], scales[1], vw, sw, osc)]
+		o = X.Tensor(dev, (T, H * HD), X.BF16)
+		k = recipes.attn_row_scaled_kernel(dev, H, HD, X.BF16, False)
+		pairs = W * (W - 1) // 2 + (T - W) * W
+		fn, work, unit = (lambda: k.launch_row_scaled(q, kv, sk, sv, tp, o, None, W, *rs)), 4.0 * HD * H * pairs / 1e12, "TOPS"
+	elif name == "attn_d_q_config4":
+		# the backward with respect to q at the attention shape of config 4 (QK + dP + dQ: 6 hd multiply-adds per pair)
+		T, B, H, HD, W = 8192, 4, 16, 128, 512
+		rows = T * B
+		q = X.Tensor.from_numpy(dev, _rand_codes(rng, (rows, H * HD)), X.INT8)
+		kv = X.Tensor.from_numpy(dev, _rand_codes(rng, (rows, 2 * H * HD)), X.INT8)
+		sk = X.Tensor.from_numpy(dev, _rand_codes(rng, (H, HD)), X.INT8)
+		sv = X.Tensor.from_numpy(dev, _rand_codes(rng, (H, HD)), X.INT8)
+		tp = X.Tensor.from_numpy(dev, (0.5 + rng.random(H)).astype(np.float32), X.F32)
+		o = X.Tensor(dev, (rows, H * HD), X.INT8)
+		l = X.Tensor(dev, (H, rows), X.F32)
+		recipes.attn_kernel(dev, H, HD, False).launch(q, kv, sk, sv, tp, o, l, W, B)
+		d_o = X.Tensor.from_numpy(dev, (rng.standard_normal((rows, H * HD), dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16), X.BF16)
+		dq = X.Tensor(dev, (rows, H * HD), X.BF16)
+		dd = X.Tensor(dev, (H, rows), X.F32)
+		k = recipes.attn_d_q_kernel(dev, H, HD, False)
+		pairs = W * (W - 1) // 2 + (T - W) * W
+		fn, work, unit = (lambda: k.launch_d_q(q, kv, sk, sv, tp, o, d_o, dq, l, dd, W, B)), 6.0 * HD * H * B * pairs / 1e12, "TOPS"
 	elif name == "decode_config5":
 		S5, CAP, H, HD, W = 64, 4096, 32, 128, 4096
 		one = _rand_codes(rng, (1, CAP, 2 * H * HD))
@@ -554,7 +602,8 @@ def single(dev, X, recipes, name, iters):
 	                  "rate": work / med, "unit": unit}))
 
 
-ONLY_TARGETS = ("ffn_f_config2", "ffn_f_f8_config3", "ffn_y_f8_config4", "attn_config4", "attn_config5", "decode_config5",
+ONLY_TARGETS = ("ffn_f_config2", "ffn_f_f8_config3", "ffn_y_f8_config4", "attn_config4", "attn_config5", "attn_row_scaled_config5",
+                "attn_d_q_config4", "decode_config5",
                 "decode_dense_config5", "attn_kv_config4", "attn_qkv_config4", "ffn_f_config4", "attn_y_config4", "rms_norm_config4")
 
 

@@ -72,6 +72,7 @@ def _specs():
 	for h, hd in ((8, 64), (2, 128), (4, 32), (2, 64)):
 		add(("attn_d_q", h, hd, True))
 	add(("attn_d_q", 8, 64, False))
+	add(("attn_d_q", 16, 128, False))                    # bench.py
 	for h, hd, cap in ((4, 32, 256), (4, 64, 256), (2, 128, 512), (2, 32, 4096), (2, 64, 4096)):
 		add(("decode", h, hd, cap, True))
 	for h, hd, cap, out in ((4, 64, 256, BF16), (2, 128, 512, BF16), (4, 32, 256, INT8)):
