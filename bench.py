@@ -319,12 +319,12 @@ def extras(dev, X, recipes):
 	x3 = X.Tensor.from_numpy(dev, e4m3_rand((M3, D3)), X.E4M3)
 	w13 = X.Tensor.from_numpy(dev, e4m3_rand((2 * F3, D3)), X.E4M3)
 	f3 = X.Tensor(dev, (M3, F3), X.E4M3)
-	c3 = {"ffn_f_f8": gemm_entry(recipes.ffn_f_f8_kernel(dev, D3, 2 * F3, False), x3, w13, f3, None, PEAK_FP8_TFLOPS, 30, 10)}
+	c3 = {"ffn_f_f8": gemm_entry(recipes.ffn_f_f8_kernel(dev, D3, 2 * F3, False), x3, w13, f3, None, PEAK_FP8_TFLOPS)}
 	del w13
 	w23 = X.Tensor.from_numpy(dev, e4m3_rand((2 * D3, F3)), X.E4M3)
 	r3 = X.Tensor.from_numpy(dev, _rand_codes(rng, (M3, D3)), X.INT8)
 	y3 = X.Tensor(dev, (M3, D3), X.E4M3)
-	c3["ffn_y_f8"] = gemm_entry(recipes.ffn_y_kernel(dev, D3, F3, False, X.E4M3, X.E4M3), f3, w23, y3, r3, PEAK_FP8_TFLOPS, 30, 10)
+	c3["ffn_y_f8"] = gemm_entry(recipes.ffn_y_kernel(dev, D3, F3, False, X.E4M3, X.E4M3), f3, w23, y3, r3, PEAK_FP8_TFLOPS)
 	out["config3_fp8_ffn"] = c3
 	del x3, w23, f3, r3, y3
 
