@@ -373,7 +373,13 @@ def extras(dev, X, recipes):
 	med, _ = _median_launch(dev, X, lambda: kb_.launch_d_q(qb_, kvb, skb, svb, tpb, ob, dob, dqb, lb, ddb, W, B), ATTN_TIMED, ATTN_WARM)
 	out["config4_attn_d_q"] = {"median_us": med * 1e6, "tops": 6.0 * HD * H * B * pairs / med / 1e12,
 	                           "note": "QK on the int8 matrix cores, dP and dQ on the f16 cores: 6 hd multiply-adds per visible (query, key) pair"}
-	del qb_, kvb, ob, lb, dob, dqb, ddb
+	# ... and with respect to k and v (consumes the D the dQ launch wrote)
+	dkvb = X.Tensor(dev, (rowsb, 2 * H * HD), X.BF16)
+	kkv = recipes.attn_d_kv_kernel(dev, H, HD, False)
+	med, _ = _median_launch(dev, X, lambda: kkv.launch_d_kv(qb_, kvb, tpb, dob, lb, ddb, dkvb, W, B), ATTN_TIMED, ATTN_WARM)
+	out["config4_attn_d_kv"] = {"median_us": med * 1e6, "tops": 8.0 * HD * H * B * pairs / med / 1e12,
+	                            "note": "QK on the int8 matrix cores, dP, dV and dK on the bf16 cores: 8 hd multiply-adds per visible (query, key) pair"}
+	del qb_, kvb, ob, lb, dob, dqb, ddb, dkvb
 
 	# ---- config 1: attention T=1024, H=8, hd=64, W=256
 	T1, H1, HD1, W1 = 1024, 8, 64, 256
@@ -538,6 +544,26 @@ def single(dev, X, recipes, name, iters):
 		k = recipes.attn_d_q_kernel(dev, H, HD, False)
 		pairs = W * (W - 1) // 2 + (T - W) * W
 		fn, work, unit = (lambda: k.launch_d_q(q, kv, sk, sv, tp, o, d_o, dq, l, dd, W, B)), 6.0 * HD * H * B * pairs / 1e12, "TOPS"
+	elif name == "attn_d_kv_config4":
+		# the backward with respect to k and v at the attention shape of config 4 (QK + dP + dV + dK: 8 hd multiply-adds per pair)
+		T, B, H, HD, W = 8192, 4, 16, 128, 512
+		rows = T * B
+		q = X.Tensor.from_numpy(dev, _rand_codes(rng, (rows, H * HD)), X.INT8)
+		kv = X.Tensor.from_numpy(dev, _rand_codes(rng, (rows, 2 * H * HD)), X.INT8)
+		sk = X.Tensor.from_numpy(dev, _rand_codes(rng, (H, HD)), X.INT8)
+		sv = X.Tensor.from_numpy(dev, _rand_codes(rng, (H, HD)), X.INT8)
+		tp = X.Tensor.from_numpy(dev, (0.5 + rng.random(H)).astype(np.float32), X.F32)
+		o = X.Tensor(dev, (rows, H * HD), X.INT8)
+		l = X.Tensor(dev, (H, rows), X.F32)
+		recipes.attn_kernel(dev, H, HD, False).launch(q, kv, sk, sv, tp, o, l, W, B)
+		d_o = X.Tensor.from_numpy(dev, (rng.standard_normal((rows, H * HD), dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16), X.BF16)
+		dq = X.Tensor(dev, (rows, H * HD), X.BF16)
+		dd = X.Tensor(dev, (H, rows), X.F32)
+		recipes.attn_d_q_kernel(dev, H, HD, False).launch_d_q(q, kv, sk, sv, tp, o, d_o, dq, l, dd, W, B)
+		dkv = X.Tensor(dev, (rows, 2 * H * HD), X.BF16)
+		k = recipes.attn_d_kv_kernel(dev, H, HD, False)
+		pairs = W * (W - 1) // 2 + (T - W) * W
+		fn, work, unit = (lambda: k.launch_d_kv(q, kv, tp, d_o, l, dd, dkv, W, B)), 8.0 * HD * H * B * pairs / 1e12, "TOPS"
 	elif name == "decode_config5":
 		S5, CAP, H, HD, W = 64, 4096, 32, 128, 4096
 		one = _rand_codes(rng, (1, CAP, 2 * H * HD))
@@ -603,7 +629,7 @@ def single(dev, X, recipes, name, iters):
 
 
 ONLY_TARGETS = ("ffn_f_config2", "ffn_f_f8_config3", "ffn_y_f8_config4", "attn_config4", "attn_config5", "attn_row_scaled_config5",
-                "attn_d_q_config4", "decode_config5",
+                "attn_d_q_config4", "attn_d_kv_config4", "decode_config5",
                 "decode_dense_config5", "attn_kv_config4", "attn_qkv_config4", "ffn_f_config4", "attn_y_config4", "rms_norm_config4")
 
 

@@ -135,6 +135,10 @@ typedef struct X17hAttnConfig {
 	 * int8 generation has no backward there yet, so the operands are defined here: the forward's q, kv, sinks and
 	 * temperatures, its FixedI8 output and log-sum-exp L, dO as bf16 -> dQ as bf16 (with respect to the real q) */
 	int backward_q;
+	/* backward_kv != 0 builds the backward-with-respect-to-k-and-v kernel instead (launched with
+	 * x17h_attn_kernel_launch_d_kv; structure of attn_d_kv.cuh:1-431, likewise the reference's bf16 generation).  At most
+	 * one of backward_q and backward_kv may be set. */
+	int backward_kv;
 } X17hAttnConfig;
 /* AttnKernel::new, attn.rs:170-232 */
 int x17h_attn_kernel_new(X17hDevice *dev, char const *kernel_name, X17hAttnConfig const *config, X17hAttnKernel **out);
@@ -160,6 +164,14 @@ int x17h_attn_kernel_launch_row_scaled(X17hAttnKernel *k, X17hTensor *q, X17hTen
 int x17h_attn_kernel_launch_d_q(X17hAttnKernel *k, X17hTensor *q, X17hTensor *kv, X17hTensor *sink_k, X17hTensor *sink_v,
                                 X17hTensor *attn_temperature, X17hTensor *out, X17hTensor *d_out, X17hTensor *d_q,
                                 X17hTensor *l, X17hTensor *d, size_t window_size, size_t batch);
+/* Launch of a kernel built with backward_kv (structure of attn_d_kv.cuh:200-400: a block of keys walks the queries that
+ * see it; P from L, dV += P^T dO, dS = P (dP - D), dK += dS^T Q; like attn_d_kv.cuh it forms no gradient for the sink or
+ * the temperatures).  d_out: bf16 [rows, o_stride]; l: f32 [n_heads, rows] of the forward; d: f32 [n_heads, rows] as
+ * written by x17h_attn_kernel_launch_d_q; d_kv: bf16 [rows, kv_stride] (written), in the layout of kv: per head dK then
+ * dV, gradients with respect to the real k and v. */
+int x17h_attn_kernel_launch_d_kv(X17hAttnKernel *k, X17hTensor *q, X17hTensor *kv, X17hTensor *attn_temperature,
+                                 X17hTensor *d_out, X17hTensor *l, X17hTensor *d, X17hTensor *d_kv,
+                                 size_t window_size, size_t batch);
 /* AttnKernelConfig::n_ops, attn.rs:72-84 */
 double x17h_attn_kernel_n_ops(X17hAttnKernel *k, size_t seq_len, size_t window_size);
 int x17h_attn_kernel_metadata(X17hAttnKernel *k, size_t out[3]);

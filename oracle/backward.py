@@ -1,4 +1,4 @@
-"""Dense float64 definition of the attention backward with respect to q, for the int8 generation of the path.
+"""Dense float64 definition of the attention backward (dQ, dK, dV), for the int8 generation of the path.
 
 TEST INFRASTRUCTURE ONLY (same rules as oracle/strict.py and oracle/dense.py).
 
@@ -20,7 +20,12 @@ cuda/attn_fwd_i8.cuh:368-619:
   dq_i            = t_i * sum_j dS_ij * k_j          (gradient with respect to the REAL q; the quantisation of q is
                   treated as the identity as well)
 
-With the exact o and L of the dense forward this is the derivative of sum(dO * o) with respect to q
+  dk_j            = sum_i t_i * dS_ij * q_i          (structure of attn_d_kv.cuh:200-400: one block of keys walks the
+  dv_j            = sum_i P_ij * dO_i                 queries that see it; D comes from the dQ pass; gradients with
+                                                      respect to the REAL k and v of the sequence's own keys -- like
+                                                      attn_d_kv.cuh, no gradient is formed for the sink or the temperature)
+
+With the exact o and L of the dense forward this is the derivative of sum(dO * o) with respect to q, k and v
 (tests/test_oracle_backward.py holds it against torch autograd in float64).  With the stored int8 output in D the
 rows of dS no longer sum to exactly zero; the deviation is bounded by |dO_i| * |o_i - o_hat_i| and is part of the
 definition (the same happens with a bf16 O in the reference, at a smaller scale).
@@ -98,3 +103,36 @@ def attn_d_q(q_codes, kv_codes, sink_k_codes, sink_v_codes, head_temp, n_heads: 
 			sink_v_codes[h].astype(np.float64) / 8.0, float(head_temp[h]), w,
 			out_codes[:, sl].astype(np.float64) / 8.0, np.asarray(d_out, dtype=np.float64)[:, sl], l[h])
 	return dq, d
+
+
+def attn_d_kv_one_head(q, k, v, sink_k, sink_v, head_temp: float, window: int, d_o, l, d):
+	"""(dk [T, hd], dv [T, hd], d_sink_k [hd], d_sink_v [hd]) for one head.  `d` is the D of the dQ pass (whatever
+	output it was formed with); the sink's two gradients are returned for the tests' invariants only."""
+	t, hd = q.shape
+	ka = np.concatenate((sink_k[None, :], k), axis=0)
+	va = np.concatenate((sink_v[None, :], v), axis=0)
+	ti = temperature(t, hd, window, head_temp)
+	s = (q @ ka.T) * ti
+	prob = np.where(visible(t, window), np.exp2(s - (np.asarray(l, dtype=np.float64)[:, None] - LOG2_255)), 0.0)
+	ds = math.log(2.0) * prob * (d_o @ va.T - np.asarray(d, dtype=np.float64)[:, None])
+	dka = (ds * ti).T @ q
+	dva = prob.T @ d_o
+	return dka[1:], dva[1:], dka[0], dva[0]
+
+
+def attn_d_kv(q_codes, kv_codes, sink_k_codes, sink_v_codes, head_temp, n_heads: int, head_dim: int, window: int,
+              d_out, l, d):
+	"""The kernel's interface in float64: operands as in attn_d_q, d [H, T] from the dQ pass.  Returns d_kv float64
+	[T, H*2*hd] in the layout of kv (per head dK then dV)."""
+	t = q_codes.shape[0]
+	w = 0 if window == 0 else ((window - 1) // 16 + 1) * 16
+	d_kv = np.empty((t, 2 * n_heads * head_dim), dtype=np.float64)
+	for h in range(n_heads):
+		sl = slice(h * head_dim, (h + 1) * head_dim)
+		ks, vs = slice(2 * h * head_dim, (2 * h + 1) * head_dim), slice((2 * h + 1) * head_dim, (2 * h + 2) * head_dim)
+		d_kv[:, ks], d_kv[:, vs], _, _ = attn_d_kv_one_head(
+			q_codes[:, sl].astype(np.float64) / 8.0, kv_codes[:, ks].astype(np.float64) / 8.0,
+			kv_codes[:, vs].astype(np.float64) / 8.0, sink_k_codes[h].astype(np.float64) / 8.0,
+			sink_v_codes[h].astype(np.float64) / 8.0, float(head_temp[h]), w,
+			np.asarray(d_out, dtype=np.float64)[:, sl], l[h], d[h])
+	return d_kv

@@ -129,3 +129,67 @@ def test_multi_head_wrapper_slices_heads_and_rounds_the_window():
 	want, want_d = B.attn_d_q_one_head(qc[:, sl] / 8.0, kvc[:, 2 * hd:3 * hd] / 8.0, kvc[:, 3 * hd:4 * hd] / 8.0, skc[1] / 8.0, svc[1] / 8.0,
 	                                   1.0, 32, out[:, sl] / 8.0, d_o[:, sl], l[1])
 	assert np.array_equal(dq[:, sl], want) and np.array_equal(d[1], want_d)
+
+
+
+@pytest.mark.parametrize("window,temp", [(0, 1.0), (32, 0.7), (16, 1.4), (48, -0.8)])
+def test_d_kv_equals_torch_autograd(window, temp):
+	q, k, v, sk, sv, d_o = _case(103 + window)
+	o, l = B.attn_fwd_one_head(q, k, v, sk, sv, temp, window)
+	d = (d_o * o).sum(1)
+	dk, dv, dsk, dsv = B.attn_d_kv_one_head(q, k, v, sk, sv, temp, window, d_o, l, d)
+	tk, tv, tsk, tsv = (torch.tensor(a, requires_grad=True) for a in (k, v, sk, sv))
+	(_torch_forward(torch.tensor(q), tk, tv, tsk, tsv, temp, window) * torch.tensor(d_o)).sum().backward()
+	for got, want in ((dk, tk.grad), (dv, tv.grad), (dsk, tsk.grad), (dsv, tsv.grad)):
+		want = want.numpy()
+		assert np.abs(want).max() > 1e-3
+		assert np.abs(got - want).max() < 1e-12 * max(1.0, np.abs(want).max())
+
+
+def test_d_kv_against_finite_differences_and_its_invariants():
+	q, k, v, sk, sv, d_o = _case(111, t=48, hd=32)
+	temp, window = 0.9, 16
+	o, l = B.attn_fwd_one_head(q, k, v, sk, sv, temp, window)
+	d = (d_o * o).sum(1)
+	dk, dv, dsk, dsv = B.attn_d_kv_one_head(q, k, v, sk, sv, temp, window, d_o, l, d)
+	loss_k = lambda kk: float((B.attn_fwd_one_head(q, kk, v, sk, sv, temp, window)[0] * d_o).sum())
+	loss_v = lambda vv: float((B.attn_fwd_one_head(q, k, vv, sk, sv, temp, window)[0] * d_o).sum())
+	rng = np.random.default_rng(6)
+	for _ in range(6):
+		j, c = int(rng.integers(0, 47)), int(rng.integers(0, 32))
+		e = np.zeros_like(k)
+		e[j, c] = 1e-5
+		for loss, grad in ((loss_k, dk), (loss_v, dv)):
+			fd = (loss(k + e if grad is dk else v + e) - loss(k - e if grad is dk else v - e)) / 2e-5
+			assert abs(fd - grad[j, c]) < 1e-7 * max(1.0, abs(fd)), (j, c, fd, grad[j, c])
+	# the last key is seen by no query; key j is seen by at most `window` queries
+	assert np.abs(dk[-1]).max() == 0.0 and np.abs(dv[-1]).max() == 0.0
+	# probabilities of a row sum to one over the sink and the keys: the dv rows and the sink's sum to the dO rows' sum
+	assert np.abs(dv.sum(0) + dsv - d_o.sum(0)).max() < 1e-12
+	# rows of dS sum to zero with the exact D, so a shift of every key (sink included) by one vector changes nothing:
+	# sum_j dk_j + d_sink_k = sum_i t_i (sum_j dS_ij) q_i = 0
+	assert np.abs(dk.sum(0) + dsk).max() < 1e-12
+	# linear in (dO, D) together; zero temperature: scores do not depend on k
+	dk2, dv2, _, _ = B.attn_d_kv_one_head(q, k, v, sk, sv, temp, window, 3.0 * d_o, l, 3.0 * d)
+	assert np.abs(dk2 - 3.0 * dk).max() < 1e-12 and np.abs(dv2 - 3.0 * dv).max() < 1e-12
+	o0, l0 = B.attn_fwd_one_head(q, k, v, sk, sv, 0.0, window)
+	assert np.abs(B.attn_d_kv_one_head(q, k, v, sk, sv, 0.0, window, d_o, l0, (d_o * o0).sum(1))[0]).max() == 0.0
+
+
+def test_d_kv_multi_head_wrapper_uses_the_layout_of_kv():
+	rng = np.random.default_rng(4)
+	t, h, hd = 64, 2, 32
+	qc = np.clip(np.rint(rng.standard_normal((t, h * hd)) * 8), -127, 127).astype(np.int8)
+	kvc = np.clip(np.rint(rng.standard_normal((t, 2 * h * hd)) * 8), -127, 127).astype(np.int8)
+	skc = np.clip(np.rint(rng.standard_normal((h, hd)) * 8), -127, 127).astype(np.int8)
+	svc = np.clip(np.rint(rng.standard_normal((h, hd)) * 8), -127, 127).astype(np.int8)
+	temp = np.array([0.6, 1.2])
+	d_o = rng.standard_normal((t, h * hd)) * 0.1
+	l, d = np.empty((h, t)), rng.standard_normal((h, t)) * 0.05
+	for hh in range(h):
+		_, l[hh] = B.attn_fwd_one_head(qc[:, hh * hd:(hh + 1) * hd] / 8.0, kvc[:, 2 * hh * hd:(2 * hh + 1) * hd] / 8.0,
+		                               kvc[:, (2 * hh + 1) * hd:(2 * hh + 2) * hd] / 8.0, skc[hh] / 8.0, svc[hh] / 8.0, temp[hh], 32)
+	got = B.attn_d_kv(qc, kvc, skc, svc, temp, h, hd, 24, d_o, l, d)            # window 24 rounds up to 32
+	dk, dv, _, _ = B.attn_d_kv_one_head(qc[:, hd:] / 8.0, kvc[:, 2 * hd:3 * hd] / 8.0, kvc[:, 3 * hd:] / 8.0, skc[1] / 8.0, svc[1] / 8.0,
+	                                    1.2, 32, d_o[:, hd:], l[1], d[1])
+	assert np.array_equal(got[:, 2 * hd:3 * hd], dk) and np.array_equal(got[:, 3 * hd:], dv)

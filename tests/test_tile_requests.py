@@ -80,3 +80,27 @@ def test_attention_tile_requests_stay_inside_their_sequence(tmp_path, label, mak
 	assert rc != 0 and not rep["ok"] and "past the end" in rep["error"], rep
 	rep, rc = _audit(tmp_path, kern, "attn_requests_audit.cpp", 96, 1, 0)
 	assert rc != 0 and not rep["ok"]
+
+
+D_KVS = [
+	("config 4", lambda: recipes.attn_d_kv_kernel(None, 16, 128, False), ((2048, 16, 512), (128, 1, 0), (192, 3, 16), (320, 2, 4096))),
+	("head_dim 64 (two staging wavefronts)", lambda: recipes.attn_d_kv_kernel(None, 8, 64, True), ((1024, 1, 256), (192, 2, 0), (128, 1, 16))),
+	("head_dim 32 (one staging wavefront)", lambda: recipes.attn_d_kv_kernel(None, 4, 32, True), ((768, 1, 64), (256, 3, 16))),
+]
+
+
+@pytest.mark.parametrize("label,make,shapes", D_KVS, ids=[a[0] for a in D_KVS])
+def test_attention_backward_kv_requests_and_lds_layouts(tmp_path, label, make, shapes):
+	"""attn_bwd_kv_tile.h: the three LDS layouts' request maps are the inverses of the readers' offset functions, every
+	16-byte position of a tile is requested once, operand reads stay inside their tiles, and every workgroup's walk
+	over query tiles covers exactly the queries that see its keys, inside its own sequence and inside q, d_out, L and D."""
+	kern = make()
+	for seq_len, batch, window in shapes:
+		rep, rc = _audit(tmp_path, kern, "attn_bwd_kv_requests_audit.cpp", seq_len, batch, window)
+		assert rc == 0 and rep["ok"], (label, seq_len, batch, window, rep)
+		assert rep["q_extent"] == rep["q_bytes"] and rep["d_out_extent"] == rep["d_out_bytes"] and rep["ld_extent_rows"] == rep["rows"], rep
+	seq_len, batch, window = shapes[0]
+	rep, rc = _audit(tmp_path, kern, "attn_bwd_kv_requests_audit.cpp", seq_len, batch, window, seq_len * batch - 1)
+	assert rc != 0 and not rep["ok"] and "past the end" in rep["error"], rep
+	rep, rc = _audit(tmp_path, kern, "attn_bwd_kv_requests_audit.cpp", 64, 1, 0)
+	assert rc != 0 and not rep["ok"]

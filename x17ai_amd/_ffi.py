@@ -48,7 +48,7 @@ class AttnConfigC(ctypes.Structure):
 		("dtype", ctypes.c_int), ("n_heads", ctypes.c_size_t), ("head_dim", ctypes.c_size_t),
 		("q_stride", ctypes.c_size_t), ("kv_stride", ctypes.c_size_t), ("o_stride", ctypes.c_size_t),
 		("strict_math", ctypes.c_int), ("row_scales", ctypes.c_int), ("out_dtype", ctypes.c_int),
-		("backward_q", ctypes.c_int),
+		("backward_q", ctypes.c_int), ("backward_kv", ctypes.c_int),
 	]
 
 
@@ -113,6 +113,7 @@ def host() -> ctypes.CDLL:
 	h.x17h_attn_kernel_launch.argtypes = [P, P, P, P, P, P, P, P, SZ, SZ]
 	h.x17h_attn_kernel_launch_row_scaled.argtypes = [P, P, P, P, P, P, P, P, SZ, SZ, P, P, P, P, P]
 	h.x17h_attn_kernel_launch_d_q.argtypes = [P, P, P, P, P, P, P, P, P, P, P, SZ, SZ]
+	h.x17h_attn_kernel_launch_d_kv.argtypes = [P, P, P, P, P, P, P, P, SZ, SZ]
 	h.x17h_attn_kernel_n_ops.argtypes = [P, SZ, SZ]
 	h.x17h_attn_kernel_n_ops.restype = ctypes.c_double
 	h.x17h_attn_kernel_metadata.argtypes = [P, ctypes.POINTER(SZ)]

@@ -353,6 +353,8 @@ class AttnKernelConfig:         # attn.rs:45-84
 	out_dtype: int = INT8
 	# builds the backward-with-respect-to-q kernel (attn_d_q_i8.hip) instead of the forward: AttnKernel.launch_d_q
 	backward_q: bool = False
+	# builds the backward-with-respect-to-k-and-v kernel (attn_d_kv_i8.hip) instead: AttnKernel.launch_d_kv
+	backward_kv: bool = False
 
 	def heads_per_kernel(self) -> int:
 		return 1 if self.head_dim == 0 else max(128 // self.head_dim, 1)
@@ -366,7 +368,7 @@ class AttnKernel:
 
 	def __init__(self, device: Optional[Device], kernel_name: str, config: AttnKernelConfig, strict_math: bool = True):
 		c = _ffi.AttnConfigC(config.dtype, config.n_heads, config.head_dim, config.q_stride, config.kv_stride,
-		                     config.o_stride, int(strict_math), int(config.row_scales), config.out_dtype, int(config.backward_q))
+		                     config.o_stride, int(strict_math), int(config.row_scales), config.out_dtype, int(config.backward_q), int(config.backward_kv))
 		self.device = device
 		self.name = kernel_name
 		self.config = config
@@ -396,6 +398,14 @@ class AttnKernel:
 		check(_ffi.host().x17h_attn_kernel_launch_d_q(
 			self._h, q._h, kv._h, sink_k._h, sink_v._h, attn_temperature._h, out._h, d_out._h, d_q._h, l._h,
 			d._h if d is not None else None, window_size, batch))
+
+	def launch_d_kv(self, q: Tensor, kv: Tensor, attn_temperature: Tensor, d_out: Tensor, l: Tensor, d: Tensor,
+	                d_kv: Tensor, window_size: int, batch: int = 1) -> None:
+		"""Launch of a kernel built with config.backward_kv: q, kv, the temperatures, dO `d_out` (bf16), the forward's
+		log-sum-exp `l` and the dQ pass's `d` (f32 [H, rows]) -> `d_kv` (bf16 [rows, kv_stride], per head dK then dV,
+		with respect to the real k and v)."""
+		check(_ffi.host().x17h_attn_kernel_launch_d_kv(
+			self._h, q._h, kv._h, attn_temperature._h, d_out._h, l._h, d._h, d_kv._h, window_size, batch))
 
 	def n_ops(self, seq_len: int, window_size: int) -> float:
 		return float(_ffi.host().x17h_attn_kernel_n_ops(self._h, seq_len, window_size))

@@ -580,7 +580,7 @@ namespace kernel_build {
 		uint64_t h = 0xCBF29CE484222325ull;
 		h = fnv1a(h, common_text);
 		h = fnv1a(h, device_flags());
-		char const *deps[] = {"x17_device.h", "gemm_tile.h", "attn_tile.h", "rms_norm_tile.h", "decode_tile.h", "attn_bwd_tile.h"};
+		char const *deps[] = {"x17_device.h", "gemm_tile.h", "attn_tile.h", "rms_norm_tile.h", "decode_tile.h", "attn_bwd_tile.h", "attn_bwd_kv_tile.h"};
 		std::string text;
 		for (char const *d : deps) {
 			if (read_file(kdir + "/" + d, text)) h = fnv1a(h, text);
@@ -1095,12 +1095,17 @@ std::unique_ptr<AttnKernel> AttnKernel::create(std::shared_ptr<HipDevice> device
 	if (config.row_scales) {
 		common << "#define X17_ATTN_ROW_SCALES 1\n#define X17_ATTN_OUT_BF16 " << (config.out_dtype == DType::Bf16 ? 1 : 0) << "\n";
 	}
-	if (config.backward_q && (config.row_scales || config.out_dtype != DType::Int8)) {
-		diag.add_error("the attention backward kernel takes FixedI8 operands at the fixed scale (no row scales, i8 forward output)");
+	if ((config.backward_q || config.backward_kv) && (config.row_scales || config.out_dtype != DType::Int8)) {
+		diag.add_error("the attention backward kernels take FixedI8 operands at the fixed scale (no row scales, i8 forward output)");
 		return nullptr;
 	}
-	auto built = config.backward_q ? kernel_build::build(kernel_name, common.str(), "attn_d_q_i8.hip", "attn_bwd_meta.cpp", diag)
-	                               : kernel_build::build(kernel_name, common.str(), "attn_fwd_i8.hip", "attn_meta.cpp", diag);
+	if (config.backward_q && config.backward_kv) {
+		diag.add_error("an attention kernel is the forward, the backward with respect to q, or the backward with respect to k and v: backward_q and backward_kv are both set");
+		return nullptr;
+	}
+	auto built = config.backward_q  ? kernel_build::build(kernel_name, common.str(), "attn_d_q_i8.hip", "attn_bwd_meta.cpp", diag)
+	           : config.backward_kv ? kernel_build::build(kernel_name, common.str(), "attn_d_kv_i8.hip", "attn_bwd_kv_meta.cpp", diag)
+	                                : kernel_build::build(kernel_name, common.str(), "attn_fwd_i8.hip", "attn_meta.cpp", diag);
 	if (!built) return nullptr;
 	auto meta = kernel_build::read_metadata_json(built->meta_json_path, diag);
 	if (!meta) return nullptr;
@@ -1126,7 +1131,9 @@ std::unique_ptr<AttnKernel> AttnKernel::create(std::shared_ptr<HipDevice> device
 // attn.rs:353-447
 Status AttnKernel::launch(AttnKernelArgs const &a) {
 	if (!device || !kernel) return Status::err(TensorOpError::Other, "attention kernel " + name + " was built without a device");
-	if (config.backward_q) return Status::err(TensorOpError::Other, "attention kernel " + name + " is a backward kernel: use launch_d_q");
+	if (config.backward_q || config.backward_kv) {
+		return Status::err(TensorOpError::Other, "attention kernel " + name + " is a backward kernel: use launch_d_q / launch_d_kv");
+	}
 	size_t shp[2], tmp[2];
 	Status s = tensor_check::matrix_shape("attention", "q", *a.q, std::nullopt, config.q_stride, *device, config.dtype, shp);
 	if (!s.is_ok()) return s;
@@ -1205,7 +1212,7 @@ Status AttnKernel::launch(AttnKernelArgs const &a) {
 // The backward with respect to q: the forward's inputs, its output and log-sum-exp, and dO (bf16) -> dQ (bf16), D.
 Status AttnKernel::launch_d_q(AttnKernelArgs const &a) {
 	if (!device || !kernel) return Status::err(TensorOpError::Other, "attention kernel " + name + " was built without a device");
-	if (!config.backward_q) return Status::err(TensorOpError::Other, "attention kernel " + name + " is a forward kernel");
+	if (!config.backward_q) return Status::err(TensorOpError::Other, "attention kernel " + name + " is not a backward-with-respect-to-q kernel");
 	if (a.l == nullptr || a.d_out == nullptr || a.d_q == nullptr) {
 		return Status::err(TensorOpError::Other, "attention backward needs l, d_out and d_q");
 	}
@@ -1254,6 +1261,55 @@ Status AttnKernel::launch_d_q(AttnKernelArgs const &a) {
 	void *out_ptr = a.out->ptr, *do_ptr = a.d_out->ptr, *dq_ptr = a.d_q->ptr, *l_ptr = a.l->ptr;
 	void *d_ptr = a.d != nullptr ? a.d->ptr : nullptr;
 	void *raw_args[12] = {&seq_len_arg, &q_ptr, &kv_ptr, &sk, &sv, &tp, &out_ptr, &do_ptr, &dq_ptr, &l_ptr, &d_ptr, &window_arg};
+	size_t grid[3] = {(seq_len + metadata.Q_PER_BLOCK - 1) / metadata.Q_PER_BLOCK, config.head_group_cnt(), a.batch};
+	size_t block[3] = {metadata.THREADS_PER_BLOCK, 1, 1};
+	return kernel->launch(*device->stream, grid, block, metadata.SMEM_BYTES, raw_args);
+}
+
+// The backward with respect to k and v: q, kv, the temperatures, dO (bf16), the forward's L and the dQ pass's D
+// -> d_kv (bf16, the layout of kv).
+Status AttnKernel::launch_d_kv(AttnKernelArgs const &a) {
+	if (!device || !kernel) return Status::err(TensorOpError::Other, "attention kernel " + name + " was built without a device");
+	if (!config.backward_kv) return Status::err(TensorOpError::Other, "attention kernel " + name + " is not a backward-with-respect-to-k-and-v kernel");
+	if (a.l == nullptr || a.d == nullptr || a.d_out == nullptr || a.d_kv == nullptr) {
+		return Status::err(TensorOpError::Other, "attention backward (k, v) needs l, d, d_out and d_kv");
+	}
+	char const *op = "attention backward (k, v)";
+	size_t shp[2], tmp[2];
+	Status s = tensor_check::matrix_shape(op, "q", *a.q, std::nullopt, config.q_stride, *device, config.dtype, shp);
+	if (!s.is_ok()) return s;
+	size_t const rows = shp[0];
+	s = tensor_check::matrix_shape(op, "kv", *a.kv, rows, config.kv_stride, *device, config.dtype, tmp);
+	if (!s.is_ok()) return s;
+	s = tensor_check::vector_shape(op, "attn_temperature", *a.attn_temperature, config.n_heads, *device, DType::F32);
+	if (!s.is_ok()) return s;
+	s = tensor_check::matrix_shape(op, "d_out", *a.d_out, rows, config.o_stride, *device, DType::Bf16, tmp);
+	if (!s.is_ok()) return s;
+	s = tensor_check::matrix_shape(op, "l", *a.l, config.n_heads, rows, *device, DType::F32, tmp);
+	if (!s.is_ok()) return s;
+	s = tensor_check::matrix_shape(op, "d", *a.d, config.n_heads, rows, *device, DType::F32, tmp);
+	if (!s.is_ok()) return s;
+	s = tensor_check::matrix_shape(op, "d_kv", *a.d_kv, rows, config.kv_stride, *device, DType::Bf16, tmp);
+	if (!s.is_ok()) return s;
+	for (Tensor const *in : {a.q, a.kv, a.d_out, a.l, a.d}) {
+		if (overlaps(*a.d_kv, *in)) return Status::err(TensorOpError::Other, "attention backward output d_kv must not share memory with an input");
+	}
+	if (a.batch == 0 || rows % a.batch != 0) {
+		return Status::err(TensorOpError::Other, "attention rows (" + std::to_string(rows) + ") must be divisible by batch (" + std::to_string(a.batch) + ")");
+	}
+	size_t const seq_len = rows / a.batch;
+	if (seq_len % 64 != 0 || seq_len < metadata.Q_PER_BLOCK) {
+		return Status::err(TensorOpError::Other, "attention seq_len must be divisible by 64 (as in the reference) and hold at least one key block of "
+			+ std::to_string(metadata.Q_PER_BLOCK) + ", got " + std::to_string(seq_len));
+	}
+	if (a.window_size > 0 && a.window_size % 16 != 0) {
+		return Status::err(TensorOpError::Other, "attention window_size must be zero or divisible by 16, got " + std::to_string(a.window_size));
+	}
+	if (rows > 0xFFFFFFFFull || a.window_size > 0xFFFFFFFFull) return Status::err(TensorOpError::Other, "attention sizes exceed 32 bits");
+	size_t seq_len_arg = seq_len, window_arg = a.window_size;
+	void *q_ptr = a.q->ptr, *kv_ptr = a.kv->ptr, *tp = a.attn_temperature->ptr, *do_ptr = a.d_out->ptr, *l_ptr = a.l->ptr, *d_ptr = a.d->ptr;
+	void *dkv_ptr = a.d_kv->ptr;
+	void *raw_args[9] = {&seq_len_arg, &q_ptr, &kv_ptr, &tp, &do_ptr, &l_ptr, &d_ptr, &dkv_ptr, &window_arg};
 	size_t grid[3] = {(seq_len + metadata.Q_PER_BLOCK - 1) / metadata.Q_PER_BLOCK, config.head_group_cnt(), a.batch};
 	size_t block[3] = {metadata.THREADS_PER_BLOCK, 1, 1};
 	return kernel->launch(*device->stream, grid, block, metadata.SMEM_BYTES, raw_args);
@@ -1639,7 +1695,7 @@ int x17h_attn_kernel_new(X17hDevice *dev, char const *kernel_name, X17hAttnConfi
 		if (!valid_dtype(c->dtype)) return fail("unknown dtype");
 		if (!valid_dtype(c->out_dtype)) return fail("unknown out_dtype");
 		AttnKernelConfig cfg{DType(c->dtype), c->n_heads, c->head_dim, c->q_stride, c->kv_stride, c->o_stride,
-		                     c->row_scales != 0, DType(c->out_dtype), c->backward_q != 0};
+		                     c->row_scales != 0, DType(c->out_dtype), c->backward_q != 0, c->backward_kv != 0};
 		Diagnostics diag;
 		auto k = AttnKernel::create(dev != nullptr ? dev->dev : nullptr, kernel_name, cfg, c->strict_math != 0, diag);
 		if (!k) return fail_diag("attention", diag);
@@ -1679,6 +1735,17 @@ int x17h_attn_kernel_launch_d_q(X17hAttnKernel *k, X17hTensor *q, X17hTensor *kv
 	args.d_q = d_q->t.get();
 	args.d = d != nullptr ? d->t.get() : nullptr;
 	return from_status(k->k->launch_d_q(args));
+}
+int x17h_attn_kernel_launch_d_kv(X17hAttnKernel *k, X17hTensor *q, X17hTensor *kv, X17hTensor *temp, X17hTensor *d_out,
+                                 X17hTensor *l, X17hTensor *d, X17hTensor *d_kv, size_t window_size, size_t batch) {
+	if (q == nullptr || kv == nullptr || temp == nullptr || d_out == nullptr || l == nullptr || d == nullptr || d_kv == nullptr) {
+		return fail("attention backward (k, v) launch needs q, kv, the temperatures, d_out, l, d and d_kv");
+	}
+	AttnKernelArgs args{q->t.get(), kv->t.get(), nullptr, nullptr, temp->t.get(), nullptr, l->t.get(), window_size, batch};
+	args.d_out = d_out->t.get();
+	args.d = d->t.get();
+	args.d_kv = d_kv->t.get();
+	return from_status(k->k->launch_d_kv(args));
 }
 double x17h_attn_kernel_n_ops(X17hAttnKernel *k, size_t seq_len, size_t window_size) { return k->k->config.n_ops(seq_len, window_size); }
 int x17h_attn_kernel_metadata(X17hAttnKernel *k, size_t out[3]) {

@@ -257,6 +257,9 @@ struct AttnKernelConfig {
 	// Builds the backward-with-respect-to-q kernel (attn_d_q_i8.hip; the reference's attn_d_q.cuh is its bf16
 	// generation) instead of the forward: launched through AttnKernel::launch_d_q.
 	bool backward_q = false;
+	// Builds the backward-with-respect-to-k-and-v kernel (attn_d_kv_i8.hip; structure of attn_d_kv.cuh): launched
+	// through AttnKernel::launch_d_kv.
+	bool backward_kv = false;
 	size_t heads_per_kernel() const;
 	size_t head_group_cnt() const;
 	size_t head_group_dim() const;
@@ -274,6 +277,9 @@ struct AttnKernelArgs {
 	// backward_q kernels only: `out` is the forward's output (an input here), `l` its log-sum-exp (required);
 	// d_out bf16 [rows, o_stride] in, d_q bf16 [rows, q_stride] out, d f32 [n_heads, rows] out (may be null)
 	Tensor const *d_out = nullptr, *d_q = nullptr, *d = nullptr;
+	// backward_kv kernels only: q, kv, attn_temperature, d_out, l and d (the dQ pass's D, required) in;
+	// d_kv bf16 [rows, kv_stride] out, in the layout of kv (per head dK then dV)
+	Tensor const *d_kv = nullptr;
 };
 
 struct AttnLauncherMetadata { size_t THREADS_PER_BLOCK, SMEM_BYTES, Q_PER_BLOCK; };
@@ -289,6 +295,7 @@ struct AttnKernel {
 	                                           AttnKernelConfig const &config, bool strict_math, Diagnostics &diag);
 	Status launch(AttnKernelArgs const &args);
 	Status launch_d_q(AttnKernelArgs const &args);
+	Status launch_d_kv(AttnKernelArgs const &args);
 };
 
 // ---------------------------------------------------------------- rms_norm, decode
@@ -322,6 +329,9 @@ struct AttnDecodeArgs {
 	// backward_q kernels only: `out` is the forward's output (an input here), `l` its log-sum-exp (required);
 	// d_out bf16 [rows, o_stride] in, d_q bf16 [rows, q_stride] out, d f32 [n_heads, rows] out (may be null)
 	Tensor const *d_out = nullptr, *d_q = nullptr, *d = nullptr;
+	// backward_kv kernels only: q, kv, attn_temperature, d_out, l and d (the dQ pass's D, required) in;
+	// d_kv bf16 [rows, kv_stride] out, in the layout of kv (per head dK then dV)
+	Tensor const *d_kv = nullptr;
 };
 
 struct AttnDecodeKernel {

@@ -73,6 +73,10 @@ def _specs():
 		add(("attn_d_q", h, hd, True))
 	add(("attn_d_q", 8, 64, False))
 	add(("attn_d_q", 16, 128, False))                    # bench.py
+	for h, hd in ((8, 64), (2, 128), (4, 32), (2, 64)):
+		add(("attn_d_kv", h, hd, True))
+	add(("attn_d_kv", 8, 64, False))
+	add(("attn_d_kv", 16, 128, False))                   # bench.py
 	for h, hd, cap in ((4, 32, 256), (4, 64, 256), (2, 128, 512), (2, 32, 4096), (2, 64, 4096)):
 		add(("decode", h, hd, cap, True))
 	for h, hd, cap, out in ((4, 64, 256, BF16), (2, 128, 512, BF16), (4, 32, 256, INT8)):
@@ -161,6 +165,8 @@ def _build_one(spec) -> str:
 		return recipes.attn_kernel(None, spec[1], spec[2], spec[3]).name
 	if kind == "attn_d_q":
 		return recipes.attn_d_q_kernel(None, spec[1], spec[2], spec[3]).name
+	if kind == "attn_d_kv":
+		return recipes.attn_d_kv_kernel(None, spec[1], spec[2], spec[3]).name
 	if kind == "attn_rows":
 		return recipes.attn_row_scaled_kernel(None, spec[1], spec[2], spec[3], spec[4]).name
 	if kind == "decode":

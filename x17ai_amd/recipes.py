@@ -90,6 +90,14 @@ def attn_d_q_kernel(device: Optional[Device], n_heads: int, head_dim: int, stric
 	return AttnKernel(device, f"attn_d_q_i8-h{n_heads}-hd{head_dim}-{_mode(strict)}", cfg, strict)
 
 
+def attn_d_kv_kernel(device: Optional[Device], n_heads: int, head_dim: int, strict: bool = True) -> AttnKernel:
+	"""The backward of attn_kernel with respect to k and v (structure of the reference's attn_d_kv.cuh:200-400 on the
+	int8 generation's forward): launch_d_kv(q, kv, temperatures, d_out, l, d, d_kv, window)."""
+	w = n_heads * head_dim
+	cfg = AttnKernelConfig(INT8, n_heads, head_dim, w, 2 * w, w, False, INT8, False, True)
+	return AttnKernel(device, f"attn_d_kv_i8-h{n_heads}-hd{head_dim}-{_mode(strict)}", cfg, strict)
+
+
 def attn_row_scaled_kernel(device: Optional[Device], n_heads: int, head_dim: int, out_dtype: int = BF16,
                            strict: bool = True) -> AttnKernel:
 	"""The attention kernel over int8 codes with one scale per (row, head) -- symmetric absmax / 127
