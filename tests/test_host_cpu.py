@@ -148,6 +148,34 @@ def test_kernel_build_metadata_and_cache(tmp_path, monkeypatch):
 	assert a.n_ops(X.Tensor(None, (512, 256), X.INT8), X.Tensor(None, (256, 256), X.INT8)) == 2.0 * 512 * 256 * 256
 
 
+def test_build_key_follows_the_headers_a_kernel_includes(tmp_path, monkeypatch):
+	"""The key of a code object covers its generated common.h, the flags, its two sources and, transitively, the headers
+	of the kernels directory they include -- not the other kernels' headers: a comment added to the attention tile
+	header leaves an rms_norm build alone, one added to rms_norm_tile.h or x17_device.h rebuilds it."""
+	import shutil
+	from x17ai_amd import _ffi
+	src = os.path.join(os.path.dirname(os.path.abspath(_ffi.__file__)), "csrc", "kernels")
+	kernels = tmp_path / "kernels"
+	shutil.copytree(src, kernels)
+	monkeypatch.setenv("X17AI_KERNELS_DIR", str(kernels))
+	monkeypatch.setenv("X17AI_KERNEL_CACHE", str(tmp_path / "cache"))
+	build = lambda: X.RmsNormKernel(None, "key-probe", X.BF16, 512, 1e-6)
+	key_file = tmp_path / "cache" / "key-probe" / "build.key"
+	build()
+	first = key_file.read_text()
+	stamp = (tmp_path / "cache" / "key-probe" / "kernel.hsaco").stat().st_mtime_ns
+	with open(kernels / "attn_tile.h", "a") as f:
+		f.write("// a change to another kernel's header\n")
+	build()
+	assert key_file.read_text() == first and (tmp_path / "cache" / "key-probe" / "kernel.hsaco").stat().st_mtime_ns == stamp
+	for header in ("rms_norm_tile.h", "x17_device.h"):
+		before = key_file.read_text()
+		with open(kernels / header, "a") as f:
+			f.write("// a change to a header this kernel includes\n")
+		build()
+		assert key_file.read_text() != before, header
+
+
 def test_cpu_tensors_round_trip():
 	import numpy as np
 	t = X.Tensor.from_numpy(None, np.arange(24, dtype=np.int8).reshape(4, 6), X.INT8)

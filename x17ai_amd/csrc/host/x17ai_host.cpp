@@ -12,7 +12,9 @@
 #include <unistd.h>
 
 #include <cmath>
+#include <algorithm>
 #include <cstdio>
+#include <functional>
 #include <cstdlib>
 #include <cstring>
 #include <fstream>
@@ -580,21 +582,36 @@ namespace kernel_build {
 		uint64_t h = 0xCBF29CE484222325ull;
 		h = fnv1a(h, common_text);
 		h = fnv1a(h, device_flags());
-		char const *deps[] = {"x17_device.h", "gemm_tile.h", "attn_tile.h", "rms_norm_tile.h", "decode_tile.h", "attn_bwd_tile.h", "attn_bwd_kv_tile.h"};
+		// ... the two sources and, transitively, the headers of the kernels directory they include with #include "..."
+		// (common.h is the generated text above), in the order a depth-first walk meets them: a change to another
+		// kernel's tile header leaves this key alone.
 		std::string text;
-		for (char const *d : deps) {
-			if (read_file(kdir + "/" + d, text)) h = fnv1a(h, text);
-		}
 		if (!read_file(kdir + "/" + source_file, text)) {
 			diag.add_error("kernel source not found: " + kdir + "/" + source_file);
 			return std::nullopt;
 		}
-		h = fnv1a(h, text);
 		if (!read_file(kdir + "/" + meta_source_file, text)) {
 			diag.add_error("kernel metadata source not found: " + kdir + "/" + meta_source_file);
 			return std::nullopt;
 		}
-		h = fnv1a(h, text);
+		std::vector<std::string> seen;
+		std::function<void(std::string const &)> hash_with_includes = [&](std::string const &file) {
+			if (std::find(seen.begin(), seen.end(), file) != seen.end()) return;
+			seen.push_back(file);
+			std::string body;
+			if (!read_file(kdir + "/" + file, body)) return;           // not a file of this directory (common.h, system headers)
+			h = fnv1a(h, file);
+			h = fnv1a(h, body);
+			size_t pos = 0;
+			while ((pos = body.find("#include \"", pos)) != std::string::npos) {
+				size_t const from = pos + 10, to = body.find('"', from);
+				if (to == std::string::npos) break;
+				hash_with_includes(body.substr(from, to - from));
+				pos = to;
+			}
+		};
+		hash_with_includes(source_file);
+		hash_with_includes(meta_source_file);
 		char keybuf[32];
 		std::snprintf(keybuf, sizeof keybuf, "%016llx", (unsigned long long)h);
 
