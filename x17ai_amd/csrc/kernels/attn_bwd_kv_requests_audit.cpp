@@ -70,53 +70,74 @@ int main(int argc, char **argv) {
 		for (unsigned v : seen_rows) if (v != 1) return fail("row layout is not a bijection", v, 1);
 		for (unsigned v : seen_tr) if (v != 1) return fail("granule layout is not a bijection", v, 1);
 	}
-	// ---- the staging threads: whole wavefronts; their requests fill every position once and stay in the head's columns
-	if (kt::STAGERS % at::WAVE != 0 || kt::STAGERS > kt::THREADS_PER_BLOCK) return fail("staging threads are not whole wavefronts", kt::STAGERS, kt::THREADS_PER_BLOCK);
+	// ---- the requesting threads: whole wavefronts; their requests fill every position once and stay in the head's columns
+	if (kt::Q_STAGERS % at::WAVE != 0 || kt::WIDE_STAGERS % at::WAVE != 0 || kt::WIDE_STAGERS > kt::THREADS_PER_BLOCK) {
+		return fail("requesting threads are not whole wavefronts of the workgroup", kt::WIDE_STAGERS, kt::THREADS_PER_BLOCK);
+	}
 	{
-		std::vector<unsigned> q_pos(ROWS * CPR, 0), wide_pos(ROWS * WIDE_CPR, 0);
-		unsigned stagers = 0;
+		std::vector<unsigned> q_pos(ROWS * CPR, 0), wide_pos(ROWS * WIDE_CPR, 0), widened(ROWS * CPR * 2, 0);
 		for (unsigned tid = 0; tid < kt::THREADS_PER_BLOCK; ++tid) {
-			if (!kt::is_stager(tid)) continue;
-			++stagers;
 			unsigned const wave = tid / at::WAVE, lane = tid % at::WAVE;
-			// LDS destination of the request: (region offset) + wave * 1024 + lane * 16 must be position `tid`
+			// LDS destination of a request: (region offset) + wave * 1024 + lane * 16 must be position `tid`
 			if (wave * 1024 + lane * 16 != tid * 16) return fail("a request's LDS destination is not its position", wave * 1024 + lane * 16, tid * 16);
-			++q_pos[tid];
-			unsigned const qs = kt::q_raw_source(tid, Q_STRIDE);
-			if (qs / Q_STRIDE >= ROWS || qs % Q_STRIDE + 16 > HD) return fail("a Q request leaves the tile's rows or the head's columns", qs, ROWS * Q_STRIDE);
-			for (unsigned j = 0; j < kt::WIDE_REQUESTS; ++j) {
-				unsigned const p = kt::wide_position(tid, j);
-				if (p >= ROWS * WIDE_CPR) return fail("a dO request's position is behind the tile", p, ROWS * WIDE_CPR);
-				if (j * kt::STAGERS * 16 + wave * 1024 + lane * 16 != p * 16) return fail("a dO request's LDS destination is not its position", j, p);
-				++wide_pos[p];
-				for (unsigned src : {kt::rows_source(p, O_STRIDE * 2), kt::granule_source(p, O_STRIDE * 2)}) {
+			if (kt::is_q_stager(tid)) {
+				if (tid >= ROWS * CPR) return fail("a Q request's position is behind the tile", tid, ROWS * CPR);
+				++q_pos[tid];
+				unsigned const qs = kt::q_raw_source(tid, Q_STRIDE);
+				if (qs / Q_STRIDE >= ROWS || qs % Q_STRIDE + 16 > HD) return fail("a Q request leaves the tile's rows or the head's columns", qs, ROWS * Q_STRIDE);
+			}
+			if (kt::is_wide_stager(tid)) {
+				if (tid >= ROWS * WIDE_CPR) return fail("a dO request's position is behind the tile", tid, ROWS * WIDE_CPR);
+				++wide_pos[tid];
+				for (unsigned src : {kt::rows_source(tid, O_STRIDE * 2), kt::granule_source(tid, O_STRIDE * 2)}) {
 					if (src / (O_STRIDE * 2) >= ROWS || src % (O_STRIDE * 2) + 16 > HD * 2) return fail("a dO request leaves the tile's rows or the head's columns", src, ROWS * O_STRIDE * 2);
 				}
 			}
+			if (kt::is_widener(tid)) {
+				// reads the 8 bytes at tid * 8 of the raw tile (position tid / 2, requested by a thread of another wavefront:
+				// the kernel widens only behind a barrier) and writes 16 bytes of the widened tile
+				if (tid * 8 + 8 > kt::Q_RAW_BYTES) return fail("a widening read leaves the raw tile", tid * 8 + 8, kt::Q_RAW_BYTES);
+				if (!kt::is_q_stager(tid / 2)) return fail("a widening thread reads a position nobody requested", tid / 2, kt::Q_STAGERS);
+				unsigned const n = kt::q_raw_logical_chunk(tid / 2);
+				unsigned const dst = kt::granule_offset(n / CPR, n % CPR) + 16 * (tid % 2);
+				if (dst + 16 > kt::WIDE_BYTES) return fail("a widening write leaves the bf16 tile", dst + 16, kt::WIDE_BYTES);
+				++widened[dst / 16];
+			}
 		}
-		if (stagers != kt::STAGERS) return fail("number of staging threads", stagers, kt::STAGERS);
 		for (unsigned v : q_pos) if (v != 1) return fail("a raw Q position is not requested exactly once", v, 1);
 		for (unsigned v : wide_pos) if (v != 1) return fail("a dO position is not requested exactly once", v, 1);
+		for (unsigned v : widened) if (v != 1) return fail("a 16-byte piece of the widened Q tile is not written exactly once", v, 1);
 	}
 	// ---- operand reads of a wavefront inside the tile (the lane formulas of attn_d_kv_i8.hip)
 	for (unsigned lane = 0; lane < at::WAVE; ++lane) {
-		unsigned const half = lane / 32, t = lane % 16, dh = (lane / 16) % 2;
-		for (unsigned db = 0; db < HD / 32; ++db) {
-			unsigned const lo0 = kt::granule_offset(4 * half + (t >> 2), 2 * db + dh) + 8 * (t & 3);
-			unsigned const lo8 = kt::granule_offset(8 + 4 * half + (t >> 2), 2 * db + dh) + 8 * (t & 3);
-			for (unsigned tt = 0; tt < 2; ++tt) {
-				unsigned const lo = lo0 + tt * (16 * CPR * 32);
-				unsigned const hi = CPR >= 4 ? lo + 8 * CPR * 32 : lo8 + tt * (16 * CPR * 32);
-				if (lo + 8 > kt::WIDE_BYTES || hi + 8 > kt::WIDE_BYTES) return fail("a transposed read leaves its tile", (lo > hi ? lo : hi) + 8, kt::WIDE_BYTES);
-				// the shortcuts the kernel takes must name the rows the layout function names
-				unsigned const row_lo = 16 * tt + 4 * half + (t >> 2);
-				if (lo != kt::granule_offset(row_lo, 2 * db + dh) + 8 * (t & 3)) return fail("transposed read: 16 rows further is not a constant stride", lo, row_lo);
-				if (hi != kt::granule_offset(row_lo + 8, 2 * db + dh) + 8 * (t & 3)) return fail("transposed read: 8 rows further is not the stride the kernel assumes", hi, row_lo + 8);
+		unsigned const group = lane / 16, klane = lane % 16;
+		for (unsigned qt = 0; qt < ROWS / 16; ++qt) {
+			for (unsigned s = 0; s < (HD + 63) / 64; ++s) {
+				unsigned const off = kt::q_raw_offset(16 * qt + klane, 16 * group < HD ? 4 * s + group : 0);
+				if (off + 16 > kt::Q_RAW_BYTES) return fail("an S operand read leaves the raw Q tile", off + 16, kt::Q_RAW_BYTES);
+			}
+			for (unsigned sl = 0; sl < HD / 32; ++sl) {
+				unsigned const off = kt::rows_offset(16 * qt + klane, 4 * sl + group);
+				if (off + 16 > kt::WIDE_BYTES) return fail("a dP operand read leaves the dO tile", off + 16, kt::WIDE_BYTES);
 			}
 		}
-		if (3 * ROWS * 4 > kt::CONST_BYTES_PER_WAVE || (2 * ROWS + 8 * 3 + 4 * half) * 4 + 16 > kt::CONST_BYTES_PER_WAVE) {
-			return fail("a constant read leaves the wavefront's block", (2 * ROWS + 8 * 3 + 4 * half) * 4 + 16, kt::CONST_BYTES_PER_WAVE);
+		for (unsigned dt = 0; dt < HD / 16; ++dt) {
+			unsigned const lo = kt::granule_offset(4 * group + (klane >> 2), dt) + 8 * (klane & 3);
+			unsigned const hi = lo + 16 * CPR * 32;
+			if (lo + 8 > kt::WIDE_BYTES || hi + 8 > kt::WIDE_BYTES) return fail("a transposed read leaves its tile", hi + 8, kt::WIDE_BYTES);
+			// the shortcut the kernel takes must name the row the layout function names
+			if (hi != kt::granule_offset(16 + 4 * group + (klane >> 2), dt) + 8 * (klane & 3)) return fail("transposed read: 16 rows further is not a constant stride", hi, lo);
 		}
+		if ((2 * ROWS + 16 + 4 * group) * 4 + 16 > kt::CONST_BYTES_PER_WAVE) {
+			return fail("a constant read leaves the wavefront's block", (2 * ROWS + 16 + 4 * group) * 4 + 16, kt::CONST_BYTES_PER_WAVE);
+		}
+	}
+	// the 32 lanes a transposed read serves at a time (eight consecutive rows, one granule column) lie in eight different
+	// 32-byte columns of the 256-byte bank window
+	for (unsigned dt = 0; dt < HD / 16; ++dt) for (unsigned row0 = 0; row0 < ROWS; row0 += 8) {
+		unsigned mask = 0;
+		for (unsigned r = 0; r < 8; ++r) mask |= 1u << ((kt::granule_offset(row0 + r, dt) >> 5) & 7);
+		if (mask != 0xFF) return fail("transposed reads of eight consecutive rows share a bank column", mask, 0xFF);
 	}
 	if (at::WAVE * 4 > kt::LD_BYTES_PER_WAVE) return fail("the L / D request is larger than its block", at::WAVE * 4, kt::LD_BYTES_PER_WAVE);
 	if (kt::SMEM_BYTES > 160 * 1024) return fail("LDS map larger than a CU's LDS", kt::SMEM_BYTES, 160 * 1024);
@@ -152,7 +173,7 @@ int main(int argc, char **argv) {
 				q_extent = q_end > q_extent ? q_end : q_extent;
 				do_extent = do_end > do_extent ? do_end : do_extent;
 				ld_extent = first_row + ROWS > ld_extent ? first_row + ROWS : ld_extent;
-				requests += (1ull + 2 * kt::WIDE_REQUESTS) * kt::STAGERS + kt::THREADS_PER_BLOCK;
+				requests += kt::Q_STAGERS + 2ull * kt::WIDE_STAGERS + kt::THREADS_PER_BLOCK;
 				++steps;
 			}
 		}

@@ -11,22 +11,25 @@ namespace x17 { namespace attn_bwd_kv_tile {
 namespace at = x17::attn_tile;
 
 constexpr unsigned HEAD_DIM = at::HEAD_DIM;
-constexpr unsigned KEY_WAVES = 4;
-constexpr unsigned KEYS_PER_WAVE = 32;
+constexpr unsigned KEY_WAVES = 8;
+constexpr unsigned KEYS_PER_WAVE = 16;
 constexpr unsigned KEYS_PER_BLOCK = KEY_WAVES * KEYS_PER_WAVE;        // 128 keys of one head per workgroup
 constexpr unsigned Q_PER_STEP = 32;                                    // queries staged per pipeline step
 constexpr unsigned THREADS_PER_BLOCK = at::WAVE * KEY_WAVES;
 static_assert(KEYS_PER_BLOCK == at::Q_PER_BLOCK, "the launcher's grid and its smallest sequence are the forward's");
 // tiles are requested PREFETCH steps ahead into rings of PREFETCH + 1 slots; one step before its use the int8 Q tile
-// is widened to bf16 by the threads that requested it
+// is widened to bf16
 constexpr unsigned PREFETCH = 2;
 constexpr unsigned RING = PREFETCH + 1;
-// 128 accumulators (dK^T and dV^T of 32 keys x head_dim 128) plus the key block's own K and V fragments: one wavefront per SIMD
-constexpr unsigned WAVES_PER_SIMD = 1;
+// 16 keys per wavefront on the 16 x 16 matrix instructions: 64 accumulators (dK^T and dV^T of 16 keys x head_dim 128)
+// and the keys' own K and V fragments leave room for two wavefronts per SIMD, which a lone wavefront's issue rate needs
+constexpr unsigned WAVES_PER_SIMD = 2;
 
 constexpr unsigned CPR = at::CHUNKS_PER_ROW;                // 16-byte chunks of an int8 row of the head
 constexpr unsigned WIDE_CPR = 2 * CPR;                      // ... of a bf16 row
-constexpr unsigned STAGERS = Q_PER_STEP * CPR;              // threads that request tiles: 16-byte chunk t of the Q tile each
+constexpr unsigned Q_STAGERS = Q_PER_STEP * CPR;            // threads that request the raw Q tile: 16-byte chunk t each
+constexpr unsigned WIDE_STAGERS = Q_PER_STEP * WIDE_CPR;    // threads that request the dO tile: chunk t of each of its two layouts
+static_assert(WIDE_STAGERS <= THREADS_PER_BLOCK && Q_STAGERS % at::WAVE == 0, "whole wavefronts request, one chunk per lane");
 constexpr unsigned Q_RAW_BYTES = Q_PER_STEP * HEAD_DIM;     // int8 queries as they arrive
 constexpr unsigned WIDE_BYTES = Q_PER_STEP * HEAD_DIM * 2;  // a bf16 tile (dO as it arrives, Q widened)
 constexpr unsigned LD_BYTES_PER_WAVE = 2 * Q_PER_STEP * 4;  // the tile's L and D values (f32), one copy per wavefront
@@ -57,7 +60,8 @@ constexpr unsigned end_query_tile(unsigned last_key, unsigned wr, unsigned seq_l
 // ---- LDS layouts (byte offsets inside a tile) and the requests that fill them.  A request moves 16 bytes per lane to
 // consecutive LDS addresses, so a layout is made by choosing which chunk of the source a lane asks for: position p
 // (in 16-byte units) of a tile receives the source chunk the *_source function names.
-constexpr bool is_stager(unsigned tid) { return tid < STAGERS; }
+constexpr bool is_q_stager(unsigned tid) { return tid < Q_STAGERS; }
+constexpr bool is_wide_stager(unsigned tid) { return tid < WIDE_STAGERS; }
 // raw int8 Q tile: the forward's K tile layout (linear chunk n = row * CPR + c in 128-byte line n / 8 at position
 // (n % 8) ^ ((line >> 1) & 7)): one request per staging thread
 constexpr unsigned q_raw_offset(unsigned row, unsigned c) {
@@ -85,18 +89,18 @@ constexpr unsigned rows_source(unsigned p, unsigned row_stride_bytes) {
 	return (line * RPL + slot / WIDE_CPR) * row_stride_bytes + ((slot % WIDE_CPR) ^ (line & (WIDE_CPR - 1))) * 16;
 }
 // bf16 tile read transposed (eight queries of one dim per lane): 32-byte granule n = row * CPR + g (16 dims) in
-// 256-byte line n / 8 at position (n % 8) ^ ((line & 3) << 1)
+// 256-byte line n / 8 at position (n % 8) ^ (line % CPR): the 32 lanes a ds_read_b64_tr_b16 serves at a time ask for
+// granule g of eight consecutive rows, which then lie in eight different 32-byte columns
 constexpr unsigned granule_offset(unsigned row, unsigned g) {
 	unsigned const n = row * CPR + g, line = n >> 3;
-	return (line << 8) | (((n & 7) ^ ((line & 3) << 1)) << 5);
+	return (line << 8) | (((n & 7) ^ (line & (CPR - 1))) << 5);
 }
 constexpr unsigned granule_source(unsigned p, unsigned row_stride_bytes) {
 	unsigned const gp = p / 2, line = gp / 8;
-	unsigned const n = line * 8 + ((gp % 8) ^ ((line & 3) << 1));
+	unsigned const n = line * 8 + ((gp % 8) ^ (line & (CPR - 1)));
 	return (n / CPR) * row_stride_bytes + (2 * (n % CPR) + p % 2) * 16;
 }
-// a bf16 tile has 2 * STAGERS chunks: a staging thread issues two requests per layout, for positions t and STAGERS + t
-constexpr unsigned WIDE_REQUESTS = 2;
-constexpr unsigned wide_position(unsigned tid, unsigned request) { return request * STAGERS + tid; }
+// Q tile int8 -> bf16: thread t < 2 * Q_STAGERS widens half a chunk (eight codes) of raw position t / 2
+constexpr bool is_widener(unsigned tid) { return tid < 2 * Q_STAGERS; }
 
 }} // namespace x17::attn_bwd_kv_tile

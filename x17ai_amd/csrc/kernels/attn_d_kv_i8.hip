@@ -14,19 +14,20 @@
 // Like attn_d_kv.cuh, no gradient is formed for the sink or the temperatures; the sink enters through L and D only.
 //
 // Design, MI355X-first:
-//   * One workgroup = 4 wavefronts = 128 keys of one head; a wavefront owns 32 keys: its int8 K fragments and its V
-//     fragments widened to bf16 stay in registers, with the 2 x 64 accumulators of dK^T and dV^T (dims x keys) --
-//     one wavefront per SIMD.
-//   * Orientation: S and dP are (queries x keys), so a lane owns ONE key and 16 queries of the tile.  Their MFMA
-//     results are then, packed to bf16, directly the "B" operands (contraction over queries) of
+//   * One workgroup = 8 wavefronts = 128 keys of one head; a wavefront owns 16 keys and works on the 16 x 16 matrix
+//     instructions: its int8 K fragments, its V fragments widened to bf16 and the 2 x 32 accumulators of dK^T and dV^T
+//     (dims x keys) stay in registers and leave room for two wavefronts per SIMD -- with a lone wavefront per SIMD
+//     (32 keys, 32 x 32 instructions, 380 registers) no unit was busy more than a third of the time.
+//   * Orientation: S and dP are (queries x keys), so a lane owns ONE key and 8 queries of the 32-query tile.  Their
+//     MFMA results are then, packed to bf16, directly the "B" operand (contraction over the tile's 32 queries) of
 //     dV^T += dO^T . P and dK^T += Q^T . dS; no lane exchange, no LDS round trip.
-//   * S runs on v_mfma_i32_32x32x32_i8 from the raw int8 Q tile; dP, dV^T, dK^T on v_mfma_f32_32x32x16_bf16 (dO is bf16
-//     in memory and is used as it is; int8 codes are exact in bf16).
+//   * S runs on v_mfma_i32_16x16x64_i8 from the raw int8 Q tile; dP, dV^T, dK^T on v_mfma_f32_16x16x32_bf16 (dO is bf16
+//     in memory and is used as it is; int8 codes are exact in bf16): 28 matrix instructions per step for head_dim 128.
 //   * Tiles of 32 queries arrive global -> LDS directly, two steps ahead: the raw Q rows, the dO rows twice -- once
 //     laid out for row reads ("A" of dP: eight dims of one query) and once for ds_read_b64_tr_b16 ("A" of dV^T: eight
 //     queries of one dim); a layout is chosen by which source chunk a lane requests, so neither copy costs an
-//     LDS -> LDS pass -- and the tile's L and D values.  One step ahead the requesting threads widen the Q tile to
-//     bf16 into the transposed-read layout ("A" of dK^T) and every wavefront writes the tile's per-query constants
+//     LDS -> LDS pass -- and the tile's L and D values.  One step ahead the workgroup widens the Q tile to bf16 into
+//     the transposed-read layout ("A" of dK^T) and every wavefront writes the tile's per-query constants
 //     (temperature, L - lg2 255, D) for itself.
 //
 // common.h (generated per kernel) provides X17_N_HEADS, X17_HEAD_DIM, X17_Q_STRIDE, X17_KV_STRIDE, X17_O_STRIDE,
@@ -48,9 +49,10 @@ constexpr u32 Q_STRIDE = X17_Q_STRIDE;
 constexpr u32 KV_STRIDE = X17_KV_STRIDE;
 constexpr u32 O_STRIDE = X17_O_STRIDE;
 constexpr u32 HPK = at::HEADS_PER_KERNEL;
-constexpr u32 K_SLICES = HD / 32;      // 32 bytes of head_dim per QK MFMA
-constexpr u32 D_SLICES = HD / 16;      // 16 dims per dP MFMA
-constexpr u32 D_BLOCKS = HD / 32;      // 32 output dims per dK^T / dV^T MFMA
+constexpr u32 K_SLICES = (HD + 63) / 64;   // 64 bytes of head_dim per QK MFMA (head_dim 32: the upper half is zero)
+constexpr u32 D_SLICES = HD / 32;          // 32 dims per dP MFMA
+constexpr u32 D_TILES = HD / 16;           // 16 output dims per dK^T / dV^T MFMA
+constexpr u32 Q_TILES = kt::Q_PER_STEP / 16;   // S and dP: two 16-query tiles per step
 constexpr u32 CPR = kt::CPR;
 
 static_assert(HD == 32 || HD == 64 || HD == 128, "head_dim must be 32, 64 or 128");
@@ -101,8 +103,8 @@ void kernel(
 	u32 const tid = threadIdx.x;
 	u32 const lane = tid % 64;
 	u32 const wave = __builtin_amdgcn_readfirstlane(tid / 64);
-	u32 const half = lane / 32;
-	u32 const rlane = lane % 32;
+	u32 const group = lane / 16;          // the lane's k-group in the operands, its row group in the results
+	u32 const klane = lane % 16;          // its key in S, dP and the accumulators; its row or dim in the "A" operands
 
 	u32 const pairs = gridDim.y * gridDim.z;
 	u32 const lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
@@ -114,7 +116,7 @@ void kernel(
 	size_t const all_rows = (size_t)gridDim.z * seq_len;
 	u32 const key_block0 = kt::block_first_key(key_block_index, seq_len);
 	u32 const key_wave0 = key_block0 + wave * kt::KEYS_PER_WAVE;
-	u32 const key = key_wave0 + rlane;
+	u32 const key = key_wave0 + klane;
 	u32 const wr = at::rounded_window(window_size);
 	u32 const vis_bound = wr - 1 < 0x7FFFFFFFu ? wr - 1 : 0x7FFFFFFFu;
 	u32 const tile_begin = kt::first_query_tile(key_block0);
@@ -124,26 +126,30 @@ void kernel(
 	u32 const n_steps = tile_end - tile_begin;
 
 	// ---- lane constants of the requests and of the operand reads
-	bool const stager = kt::is_stager(tid);
+	bool const q_stager = kt::is_q_stager(tid), wide_stager = kt::is_wide_stager(tid), widener = kt::is_widener(tid);
 	u32 const q_src = kt::q_raw_source(tid, Q_STRIDE);
-	u32 rows_src[kt::WIDE_REQUESTS], tr_src[kt::WIDE_REQUESTS];
-	X17_UNROLL for (u32 j = 0; j < kt::WIDE_REQUESTS; ++j) {
-		rows_src[j] = kt::rows_source(kt::wide_position(tid, j), O_STRIDE * 2);
-		tr_src[j] = kt::granule_source(kt::wide_position(tid, j), O_STRIDE * 2);
+	u32 const rows_src = kt::rows_source(tid, O_STRIDE * 2);
+	u32 const tr_src = kt::granule_source(tid, O_STRIDE * 2);
+	// stored chunk tid / 2 of the raw Q tile holds logical chunk n: query n / CPR, dims 16 * (n % CPR) .. + 15; this
+	// thread widens its half tid % 2
+	u32 const q_logical = kt::q_raw_logical_chunk(tid / 2);
+	u32 const q_wide_dst = kt::granule_offset(q_logical / CPR, q_logical % CPR) + 16 * (tid % 2);
+	// "A" of S: query 16 qt + klane, the 16 bytes 64 s + 16 group of its row (none for head_dim 32's upper half)
+	bool const k_group_in_row = 16 * group < HD;
+	u32 q_read_off[Q_TILES][K_SLICES];
+	// "A" of dP: query 16 qt + klane, dims 32 sl + 8 group + 0..7
+	u32 do_read_off[Q_TILES][D_SLICES];
+	X17_UNROLL for (u32 qt = 0; qt < Q_TILES; ++qt) {
+		X17_UNROLL for (u32 s = 0; s < K_SLICES; ++s) q_read_off[qt][s] = kt::q_raw_offset(16 * qt + klane, k_group_in_row ? 4 * s + group : 0);
+		X17_UNROLL for (u32 sl = 0; sl < D_SLICES; ++sl) do_read_off[qt][sl] = kt::rows_offset(16 * qt + klane, 4 * sl + group);
 	}
-	// stored chunk `tid` of the raw Q tile holds logical chunk n: query n / CPR, dims 16 * (n % CPR) .. + 15
-	u32 const q_logical = kt::q_raw_logical_chunk(tid);
-	u32 const q_wide_dst = kt::granule_offset(q_logical / CPR, q_logical % CPR);
-	// transposed reads: lane t of sixteen asks for eight bytes of query 4 half + t / 4 (lo) and 8 more (hi)
-	u32 tr_lane_off[D_BLOCKS];
-	[[maybe_unused]] u32 tr_lane_off8[D_BLOCKS];
-	{
-		u32 const t = lane % 16, dh = (lane / 16) % 2;
-		X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
-			tr_lane_off[db] = kt::granule_offset(4 * half + (t >> 2), 2 * db + dh) + 8 * (t & 3);
-			tr_lane_off8[db] = kt::granule_offset(8 + 4 * half + (t >> 2), 2 * db + dh) + 8 * (t & 3);
-		}
+	// transposed reads ("A" of dV^T and dK^T: dim 16 dt + klane, the 8 queries 4 group + 0..3 and 16 + 4 group + 0..3):
+	// lane t of sixteen asks for eight bytes of query 4 group + t / 4; sixteen queries further is a constant stride
+	u32 tr_lane_off[D_TILES];
+	X17_UNROLL for (u32 dt = 0; dt < D_TILES; ++dt) {
+		tr_lane_off[dt] = kt::granule_offset(4 * group + (klane >> 2), dt) + 8 * (klane & 3);
 	}
+	constexpr u32 TR_SIXTEEN_ROWS = 16 * CPR * 32;
 
 	for (u32 hh = 0; hh < HPK; ++hh) {
 		u32 const head = head_group * HPK + hh;
@@ -156,62 +162,56 @@ void kernel(
 
 		auto issue_loads = [&](u32 tile, u32 slot) {
 			u8 *base = smem + slot * kt::SLOT_BYTES;
-			if (stager) {
+			if (q_stager) {
 				i8 const *q_tile = q_head + (size_t)(tile * kt::Q_PER_STEP) * Q_STRIDE;
-				u8 const *do_tile = do_head + (size_t)(tile * kt::Q_PER_STEP) * (O_STRIDE * 2);
 				__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(q_tile + q_src), X17_LDS_PTR(base + kt::Q_RAW_OFFSET + wave * 1024), 16, 0, 0);
-				X17_UNROLL for (u32 j = 0; j < kt::WIDE_REQUESTS; ++j) {
-					__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(do_tile + rows_src[j]),
-						X17_LDS_PTR(base + kt::DO_ROWS_OFFSET + j * kt::STAGERS * 16 + wave * 1024), 16, 0, 0);
-					__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(do_tile + tr_src[j]),
-						X17_LDS_PTR(base + kt::DO_TR_OFFSET + j * kt::STAGERS * 16 + wave * 1024), 16, 0, 0);
-				}
+			}
+			if (wide_stager) {
+				u8 const *do_tile = do_head + (size_t)(tile * kt::Q_PER_STEP) * (O_STRIDE * 2);
+				__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(do_tile + rows_src), X17_LDS_PTR(base + kt::DO_ROWS_OFFSET + wave * 1024), 16, 0, 0);
+				__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(do_tile + tr_src), X17_LDS_PTR(base + kt::DO_TR_OFFSET + wave * 1024), 16, 0, 0);
 			}
 			// every wavefront for itself: lanes 0..31 the tile's L, lanes 32..63 its D
-			f32 const *ld_src = (half == 0 ? l_head : d_head) + tile * kt::Q_PER_STEP + rlane;
+			f32 const *ld_src = (lane < 32 ? l_head : d_head) + tile * kt::Q_PER_STEP + lane % 32;
 			__builtin_amdgcn_global_load_lds(X17_GLOBAL_PTR(ld_src), X17_LDS_PTR(base + kt::LD_OFFSET + wave * kt::LD_BYTES_PER_WAVE), 4, 0, 0);
 		};
-		// Q tile int8 -> bf16 by the thread that requested the chunk, and this wavefront's per-query constants
+		// Q tile int8 -> bf16, half a chunk per thread -- a chunk some other wavefront requested: only called behind a
+		// barrier that every thread passed after waiting for its own requests -- and this wavefront's per-query constants
 		auto prepare = [&](u32 tile, u32 slot) {
-			u32 const buf = slot;
 			u8 const *base = smem + slot * kt::SLOT_BYTES;
-			if (stager) {
-				v4u const raw = *reinterpret_cast<v4u const *>(base + kt::Q_RAW_OFFSET + tid * 16);
-				u32 w[8];
-				X17_UNROLL for (int i = 0; i < 4; ++i) {
-					u32 const biased = raw[i] ^ 0x80808080u;
-					w[2 * i] = bf16_pair(biased, 0);
-					w[2 * i + 1] = bf16_pair(biased, 2);
-				}
-				u8 *dst = smem + kt::Q_WIDE_OFFSET + buf * kt::WIDE_BYTES + q_wide_dst;
-				*reinterpret_cast<v4u *>(dst) = v4u{w[0], w[1], w[2], w[3]};
-				*reinterpret_cast<v4u *>(dst + 16) = v4u{w[4], w[5], w[6], w[7]};
+			if (widener) {
+				v2u const raw = *reinterpret_cast<v2u const *>(base + kt::Q_RAW_OFFSET + tid * 8);
+				u32 const b0 = raw[0] ^ 0x80808080u, b1 = raw[1] ^ 0x80808080u;
+				*reinterpret_cast<v4u *>(smem + kt::Q_WIDE_OFFSET + slot * kt::WIDE_BYTES + q_wide_dst) =
+					v4u{bf16_pair(b0, 0), bf16_pair(b0, 2), bf16_pair(b1, 0), bf16_pair(b1, 2)};
 			}
 			f32 const landed = *reinterpret_cast<f32 const *>(base + kt::LD_OFFSET + wave * kt::LD_BYTES_PER_WAVE + lane * 4);
-			f32 *cst = reinterpret_cast<f32 *>(smem + kt::CONST_OFFSET + (buf * kt::KEY_WAVES + wave) * kt::CONST_BYTES_PER_WAVE);
-			cst[kt::Q_PER_STEP + lane] = half == 0 ? landed - LOG2_PROB_SCALE : landed;       // L - lg2 255 | D
-			if (half == 0) {
-				u32 const qi = tile * kt::Q_PER_STEP + rlane;
+			f32 *cst = reinterpret_cast<f32 *>(smem + kt::CONST_OFFSET + (slot * kt::KEY_WAVES + wave) * kt::CONST_BYTES_PER_WAVE);
+			cst[kt::Q_PER_STEP + lane] = lane < 32 ? landed - LOG2_PROB_SCALE : landed;       // L - lg2 255 | D
+			if (lane < 32) {
+				u32 const qi = tile * kt::Q_PER_STEP + lane;
 				u32 const visible = qi < wr ? qi : wr;
 				cst[lane] = (BASE_TEMPERATURE * sfu::lg2(f32(visible + 4u))) * head_temperature;
 			}
 		};
 
-		// ---- the key block's own operands
-		v4i kf[K_SLICES];                    // "B" of S: lane = key, 16 bytes of every 32-dim slice
+		// ---- the wavefront's own operands
+		v4i kf[K_SLICES];                    // "B" of S: lane = key, the 16 bytes 64 s + 16 group of its row
 		X17_UNROLL for (u32 s = 0; s < K_SLICES; ++s) {
-			kf[s] = *reinterpret_cast<v4i const *>(kv_head + (size_t)key * KV_STRIDE + 32 * s + 16 * half);
+			kf[s] = v4i{0, 0, 0, 0};
+			if (k_group_in_row) kf[s] = *reinterpret_cast<v4i const *>(kv_head + (size_t)key * KV_STRIDE + 64 * s + 16 * group);
 		}
-		v8bf vfrag[D_SLICES];                // "B" of dP: lane = key, dims 16 sl + 8 half + 0..7 as bf16
+		v8bf vfrag[D_SLICES];                // "B" of dP: lane = key, dims 32 sl + 8 group + 0..7 as bf16
 		X17_UNROLL for (u32 sl = 0; sl < D_SLICES; ++sl) {
-			v2u const raw = *reinterpret_cast<v2u const *>(kv_head + (size_t)key * KV_STRIDE + HD + 16 * sl + 8 * half);
+			v2u const raw = *reinterpret_cast<v2u const *>(kv_head + (size_t)key * KV_STRIDE + HD + 32 * sl + 8 * group);
 			u32 const b0 = raw[0] ^ 0x80808080u, b1 = raw[1] ^ 0x80808080u;
 			v4u const words = {bf16_pair(b0, 0), bf16_pair(b0, 2), bf16_pair(b1, 0), bf16_pair(b1, 2)};
 			vfrag[sl] = __builtin_bit_cast(v8bf, words);
 		}
-		v16f dk_acc[D_BLOCKS], dv_acc[D_BLOCKS];    // (dims x keys): lane = key, register r = dim 32 db + 8 (r / 4) + 4 half + r % 4
-		X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
-			X17_UNROLL for (int r = 0; r < 16; ++r) { dk_acc[db][r] = 0.0f; dv_acc[db][r] = 0.0f; }
+		v4f dk_acc[D_TILES], dv_acc[D_TILES];    // (dims x keys): lane = key, register r = dim 16 dt + 4 group + r
+		X17_UNROLL for (u32 dt = 0; dt < D_TILES; ++dt) {
+			dk_acc[dt] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+			dv_acc[dt] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 		}
 
 		// ---- pipeline prologue
@@ -220,6 +220,7 @@ void kernel(
 			if (j < n_steps) issue_loads(tile_begin + j, j);
 		}
 		__builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+		__builtin_amdgcn_s_barrier();         // everybody's requests for tile 0 have landed
 		prepare(tile_begin, 0);
 
 		// one pipeline step, common to all wavefronts of the workgroup
@@ -237,107 +238,91 @@ void kernel(
 				prepare(tile + 1, (slot + 1) % kt::RING);
 			}
 		};
-		// the step's arithmetic for this wavefront's 32 keys
+		// the step's arithmetic for this wavefront's 16 keys
 		auto compute = [&](u32 i, u32 slot) {
 			u32 const tile = tile_begin + i;
 			u8 const *base = smem + slot * kt::SLOT_BYTES;
 			u8 const *q_wide = smem + kt::Q_WIDE_OFFSET + slot * kt::WIDE_BYTES;
 			f32 const *cst = reinterpret_cast<f32 const *>(smem + kt::CONST_OFFSET + (slot * kt::KEY_WAVES + wave) * kt::CONST_BYTES_PER_WAVE);
-
-			// S block: rows = the tile's 32 queries, columns = this wave's 32 keys
-			v16i s_acc = {0};
-			X17_UNROLL for (u32 s = 0; s < K_SLICES; ++s) {
-				v4i const qa = *reinterpret_cast<v4i const *>(base + kt::Q_RAW_OFFSET + kt::q_raw_offset(rlane, 2 * s + half));
-				s_acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa, kf[s], s_acc, 0, 0, 0);
-			}
-			// dP block (times 8: v codes)
-			v16f dp_acc = {0};
-			X17_UNROLL for (u32 sl = 0; sl < D_SLICES; ++sl) {
-				v8bf const da = *reinterpret_cast<v8bf const *>(base + kt::DO_ROWS_OFFSET + kt::rows_offset(rlane, 2 * sl + half));
-				dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vfrag[sl], dp_acc, 0, 0, 0);
-			}
-
 			u32 const q0 = tile * kt::Q_PER_STEP;
-			bool const need_mask = !(key_wave0 + 31 < q0 && (q0 + 31 - key_wave0) <= wr);
-			// register r of a block belongs to query q0 + 8 (r / 4) + 4 half + r % 4; key j is visible to query i iff
-			// the distance i - 1 - j, as an unsigned number, is at most W' - 1
-			u32 const first = q0 + 4 * half - 1 - key;
-			u32 pw[8], ww[8];                 // P and the dK weights as bf16 pairs: "B" operands, slots = this lane's queries
-			X17_UNROLL for (u32 g = 0; g < 4; ++g) {
-				v4f const ct = *reinterpret_cast<v4f const *>(cst + 8 * g + 4 * half);
-				v4f const cl = *reinterpret_cast<v4f const *>(cst + kt::Q_PER_STEP + 8 * g + 4 * half);
-				v4f const cd = *reinterpret_cast<v4f const *>(cst + 2 * kt::Q_PER_STEP + 8 * g + 4 * half);
+			bool const need_mask = !(key_wave0 + kt::KEYS_PER_WAVE - 1 < q0 && (q0 + kt::Q_PER_STEP - 1 - key_wave0) <= wr);
+			u32 pw[2 * Q_TILES], ww[2 * Q_TILES];     // P and the dK weights as bf16 pairs: "B" operands, slots = this lane's 8 queries
+			X17_UNROLL for (u32 qt = 0; qt < Q_TILES; ++qt) {
+				// S and dP (times 8: v codes) blocks: rows = 16 queries of the tile, columns = this wave's 16 keys
+				v4i s_acc = {0, 0, 0, 0};
+				X17_UNROLL for (u32 s = 0; s < K_SLICES; ++s) {
+					v4i qa = *reinterpret_cast<v4i const *>(base + kt::Q_RAW_OFFSET + q_read_off[qt][s]);
+					if (!k_group_in_row) qa = v4i{0, 0, 0, 0};
+					s_acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(qa, kf[s], s_acc, 0, 0, 0);
+				}
+				v4f dp_acc = {0.0f, 0.0f, 0.0f, 0.0f};
+				X17_UNROLL for (u32 sl = 0; sl < D_SLICES; ++sl) {
+					v8bf const da = *reinterpret_cast<v8bf const *>(base + kt::DO_ROWS_OFFSET + do_read_off[qt][sl]);
+					dp_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(da, vfrag[sl], dp_acc, 0, 0, 0);
+				}
+				// register r belongs to query q0 + 16 qt + 4 group + r; key j is visible to query i iff the distance
+				// i - 1 - j, as an unsigned number, is at most W' - 1
+				u32 const first = q0 + 16 * qt + 4 * group - 1 - key;
+				v4f const ct = *reinterpret_cast<v4f const *>(cst + 16 * qt + 4 * group);
+				v4f const cl = *reinterpret_cast<v4f const *>(cst + kt::Q_PER_STEP + 16 * qt + 4 * group);
+				v4f const cd = *reinterpret_cast<v4f const *>(cst + 2 * kt::Q_PER_STEP + 16 * qt + 4 * group);
 				f32 p[4], w[4];
-				X17_UNROLL for (u32 e = 0; e < 4; ++e) {
-					u32 const r = 4 * g + e;
-					f32 pe = sfu::ex2(fmaf32(f32(s_acc[r]), ct[e], -cl[e]));
+				X17_UNROLL for (u32 r = 0; r < 4; ++r) {
+					f32 pe = sfu::ex2(fmaf32(f32(s_acc[r]), ct[r], -cl[r]));
 					if (need_mask) {
-						pe = first + (8 * g + e) <= vis_bound ? pe : 0.0f;
+						pe = first + r <= vis_bound ? pe : 0.0f;
 					}
-					p[e] = pe;
-					w[e] = (pe * fmaf32(dp_acc[r], 0.125f, -cd[e])) * ct[e];
+					p[r] = pe;
+					w[r] = (pe * fmaf32(dp_acc[r], 0.125f, -cd[r])) * ct[r];
 				}
-				pw[2 * g] = pack2_bf16_rne(p[0], p[1]);
-				pw[2 * g + 1] = pack2_bf16_rne(p[2], p[3]);
-				ww[2 * g] = pack2_bf16_rne(w[0], w[1]);
-				ww[2 * g + 1] = pack2_bf16_rne(w[2], w[3]);
+				pw[2 * qt] = pack2_bf16_rne(p[0], p[1]);
+				pw[2 * qt + 1] = pack2_bf16_rne(p[2], p[3]);
+				ww[2 * qt] = pack2_bf16_rne(w[0], w[1]);
+				ww[2 * qt + 1] = pack2_bf16_rne(w[2], w[3]);
 			}
-			X17_UNROLL for (u32 t = 0; t < 2; ++t) {
-				v8bf const pfrag = __builtin_bit_cast(v8bf, (v4u{pw[4 * t], pw[4 * t + 1], pw[4 * t + 2], pw[4 * t + 3]}));
-				v8bf const wfrag = __builtin_bit_cast(v8bf, (v4u{ww[4 * t], ww[4 * t + 1], ww[4 * t + 2], ww[4 * t + 3]}));
-				X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
-					u32 const lo = tr_lane_off[db] + t * (16 * CPR * 32);
-					u32 const hi = CPR >= 4 ? lo + 8 * CPR * 32 : tr_lane_off8[db] + t * (16 * CPR * 32);
-					dv_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-						transposed_fragment(base + kt::DO_TR_OFFSET + lo, base + kt::DO_TR_OFFSET + hi), pfrag, dv_acc[db], 0, 0, 0);
-					dk_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-						transposed_fragment(q_wide + lo, q_wide + hi), wfrag, dk_acc[db], 0, 0, 0);
-				}
+			static_assert(Q_TILES == 2, "one 16 x 16 x 32 instruction contracts over the step's 32 queries");
+			v8bf const pfrag = __builtin_bit_cast(v8bf, (v4u{pw[0], pw[1], pw[2], pw[3]}));
+			v8bf const wfrag = __builtin_bit_cast(v8bf, (v4u{ww[0], ww[1], ww[2], ww[3]}));
+			X17_UNROLL for (u32 dt = 0; dt < D_TILES; ++dt) {
+				u32 const lo = tr_lane_off[dt], hi = lo + TR_SIXTEEN_ROWS;
+				dv_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+					transposed_fragment(base + kt::DO_TR_OFFSET + lo, base + kt::DO_TR_OFFSET + hi), pfrag, dv_acc[dt], 0, 0, 0);
+				dk_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+					transposed_fragment(q_wide + lo, q_wide + hi), wfrag, dk_acc[dt], 0, 0, 0);
 			}
 		};
 		// A wavefront's keys are seen by the tiles [wave_tile_first, wave_tile_last] of the workgroup's walk.  Plain loops
-		// instead of one loop with a skip, so that the 128 accumulators (in the second half of the register file: one
-		// wavefront per SIMD owns all 512 registers; pinned there by the empty asm) are carried round the loops where the
-		// matrix instructions use them in place -- around a skip they were copied to the first half and back once per
-		// step.  The middle stretch runs three steps per trip, so that the ring slot of every LDS address is an
-		// immediate; the steps before it reaches a multiple of three, and the last ones, take the slot from i.
+		// instead of one loop with a skip (around a skip the compiler moves the accumulators about once per step), and
+		// the middle stretch runs three steps per trip so that the ring slot of every LDS address is an immediate; the
+		// steps before it reaches a multiple of three, and the last ones, take the slot from i.
 		u32 const lead = wave_tile_first - tile_begin;
 		u32 const active_end = wave_tile_last + 1 - tile_begin < n_steps ? wave_tile_last + 1 - tile_begin : n_steps;
-		auto pin_accumulators = [&]() {
-			X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) asm volatile("" : "+a"(dk_acc[db]), "+a"(dv_acc[db]));
-		};
 		u32 i = 0;
 		for (; i < lead; ++i) advance(i, i % kt::RING);
 		for (; i < active_end && i % kt::RING != 0; ++i) {
 			advance(i, i % kt::RING);
-			pin_accumulators();
 			compute(i, i % kt::RING);
 		}
 		for (; i + kt::RING <= active_end; i += kt::RING) {
 			X17_UNROLL for (u32 slot = 0; slot < kt::RING; ++slot) {
 				advance(i + slot, slot);
-				pin_accumulators();
 				compute(i + slot, slot);
 			}
 		}
 		for (; i < active_end; ++i) {
 			advance(i, i % kt::RING);
-			pin_accumulators();
 			compute(i, i % kt::RING);
 		}
 		for (; i < n_steps; ++i) advance(i, i % kt::RING);
 
 		// ---- output: dk = 8 ln 2 * dk_acc, dv = dv_acc
 		u16 *dkv_row = d_kv + (row_base + key) * KV_STRIDE + (size_t)head * 2 * HD;
-		X17_UNROLL for (u32 db = 0; db < D_BLOCKS; ++db) {
-			X17_UNROLL for (int g = 0; g < 4; ++g) {
-				v2u const k_pair = {pack2_bf16_rne(dk_acc[db][4 * g] * EIGHT_LN2, dk_acc[db][4 * g + 1] * EIGHT_LN2),
-				                    pack2_bf16_rne(dk_acc[db][4 * g + 2] * EIGHT_LN2, dk_acc[db][4 * g + 3] * EIGHT_LN2)};
-				v2u const v_pair = {pack2_bf16_rne(dv_acc[db][4 * g], dv_acc[db][4 * g + 1]),
-				                    pack2_bf16_rne(dv_acc[db][4 * g + 2], dv_acc[db][4 * g + 3])};
-				*reinterpret_cast<v2u *>(dkv_row + 32 * db + 8 * g + 4 * half) = k_pair;
-				*reinterpret_cast<v2u *>(dkv_row + HD + 32 * db + 8 * g + 4 * half) = v_pair;
-			}
+		X17_UNROLL for (u32 dt = 0; dt < D_TILES; ++dt) {
+			v2u const k_pair = {pack2_bf16_rne(dk_acc[dt][0] * EIGHT_LN2, dk_acc[dt][1] * EIGHT_LN2),
+			                    pack2_bf16_rne(dk_acc[dt][2] * EIGHT_LN2, dk_acc[dt][3] * EIGHT_LN2)};
+			v2u const v_pair = {pack2_bf16_rne(dv_acc[dt][0], dv_acc[dt][1]), pack2_bf16_rne(dv_acc[dt][2], dv_acc[dt][3])};
+			*reinterpret_cast<v2u *>(dkv_row + 16 * dt + 4 * group) = k_pair;
+			*reinterpret_cast<v2u *>(dkv_row + HD + 16 * dt + 4 * group) = v_pair;
 		}
 	}
 }
