@@ -5,7 +5,9 @@ such a write in front of a request -- their addresses are scalar arithmetic -- a
 to that: it disassembles this repository's own kernels (never a shipped library) and scans every memory instruction.
 A second rule of the same family: a scalar write of M0 needs one wait state before a direct-to-LDS load reads it (the
 compiler inserts an s_nop for its own loads; the hand-written requests carry their own), so no instruction that writes
-M0 may sit directly in front of a *_load_lds_* instruction."""
+M0 may sit directly in front of a *_load_lds_* instruction.
+A third rule is this pool's: packed single-precision arithmetic (v_pk_add_f32, v_pk_mul_f32, v_pk_fma_f32) is compiled out
+(-target-feature -packed-fp32-ops) and never written by hand; the scan holds every built code object to it."""
 import glob
 import os
 import re
@@ -23,6 +25,7 @@ SCALAR_WRITE = re.compile(r"(v_readfirstlane_b32|v_readlane_b32)\s+s(\d+)")
 SCALAR_PAIR = re.compile(r"s\[(\d+):(\d+)\]")
 M0_WRITE = re.compile(r"s_\w+\s+m0\s*,")
 LDS_DMA = re.compile(r"(global|buffer)_load_lds_\w+|buffer_load_\w+.*\blds\b")
+PACKED_F32 = re.compile(r"v_pk_(add|mul|fma)_f32")
 
 
 def _instructions(code_object, tmp_path):
@@ -73,6 +76,7 @@ def test_no_memory_instruction_reads_a_scalar_register_the_vector_unit_has_just_
 		ins = _instructions(code_object, str(tmp_path))
 		assert _hazards(ins) == [], code_object
 		assert _m0_hazards(ins) == [], code_object
+		assert [line for line in ins if PACKED_F32.match(line)] == [], code_object
 		scanned += 1
 	assert scanned >= len(kernels)
 
