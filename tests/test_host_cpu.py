@@ -45,6 +45,24 @@ def test_the_product_headers_and_libraries_hold_no_measurement_aids():
 	assert not [s for s in _exported(_ffi.lib_paths()["host"]) if "probe" in s and s.startswith("x17h_")]
 
 
+def test_the_headers_are_plain_c_and_a_c_program_links_against_both_libraries(tmp_path):
+	"""The boundary is a C ABI: both headers compile as strict C99 and as C++17, and a C program that takes the address of
+	every declared entry point links against the two libraries (no GPU is touched: nothing is called)."""
+	inc = os.path.join(ROOT, "include")
+	for header in ("x17ai_hip_shim.h", "x17ai_host.h"):
+		subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-x", "c", os.path.join(inc, header)], check=True)
+		subprocess.run(["g++", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-x", "c++", os.path.join(inc, header)], check=True)
+	names = _declared("x17ai_hip_shim.h") + _declared("x17ai_host.h")
+	prog = '#include "x17ai_hip_shim.h"\n#include "x17ai_host.h"\n#include <stdio.h>\nint main(void) {\n\tvoid (*table[])(void) = {\n'
+	prog += "".join(f"\t\t(void (*)(void)){n},\n" for n in names)
+	prog += '\t};\n\tprintf("%u\\n", (unsigned)(sizeof table / sizeof table[0]));\n\treturn 0;\n}\n'
+	exe = str(tmp_path / "links")
+	libdir = os.path.dirname(_ffi.lib_paths()["host"])
+	subprocess.run(["gcc", "-std=c99", "-x", "c", "-", "-I", inc, "-L", libdir, "-lx17ai_host", "-lx17ai_hip_shim",
+	                "-Wl,-rpath," + libdir, "-o", exe], input=prog, text=True, check=True)
+	assert int(subprocess.run([exe], capture_output=True, text=True, check=True).stdout) == len(names) > 60
+
+
 def test_struct_layouts_match_the_reference_ffi(tmp_path):
 	# CudaKernelAttrs: nine int32 (cuda_shim.rs:51-63); PtrResult: two pointers (cuda_shim.rs:70-74)
 	src = open(os.path.join(ROOT, "include", "x17ai_hip_shim.h")).read()
