@@ -290,3 +290,33 @@ def test_backward_speed_builds_at_the_size_of_benchmark_config_4(dev):
 		terms = _term_magnitudes(q[r][:, qc], kv[r][:, kc], sk[head:head + 1], sv[head:head + 1], temp[head:head + 1], 1, hd, w,
 		                         d_o[r][:, qc], l_h[head:head + 1, r], d1[head:head + 1, r])
 		_check_kv(_bf16_bits(dkv1[r][:, kc]), want_kv, terms, 1, hd)
+
+
+def test_backward_launches_are_repeatable_and_long_walks_are_homogeneous(dev):
+	"""One 16384-token sequence with a 4096-key window (the window of benchmark config 5: 133 query tiles per key block,
+	129 key tiles per query block), 4 heads x 128, speed builds.  Launching twice gives the same bytes (overhanging
+	blocks store the same values, no accumulation order depends on timing), and dO and D times 4 give exactly 4 times
+	every output."""
+	t, h, hd, w = 16384, 4, 128, 4096
+	rng = rng_for("attn-bwd-long")
+	q, kv, sk, sv, temp = _inputs(rng, t, h, hd)
+	d_o = _bf16_value(_bf16_bits(rng.standard_normal((t, h * hd)) * 0.05))
+	up = lambda a, dt: X.Tensor.from_numpy(dev, a, dt)
+	tq, tkv, tsk, tsv, tt = up(q, X.INT8), up(kv, X.INT8), up(sk, X.INT8), up(sv, X.INT8), up(temp, X.F32)
+	out, l = X.Tensor(dev, (t, h * hd), X.INT8), X.Tensor(dev, (h, t), X.F32)
+	recipes.attn_kernel(dev, h, hd, False).launch(tq, tkv, tsk, tsv, tt, out, l, w, 1)
+	k_q, k_kv = recipes.attn_d_q_kernel(dev, h, hd, False), recipes.attn_d_kv_kernel(dev, h, hd, False)
+	runs = []
+	for factor in (1.0, 1.0, 4.0):
+		t_do = up(_bf16_bits(d_o * factor), X.BF16)
+		dq, d, dkv = X.Tensor(dev, (t, h * hd), X.BF16), X.Tensor(dev, (h, t), X.F32), X.Tensor(dev, (t, 2 * h * hd), X.BF16)
+		k_q.launch_d_q(tq, tkv, tsk, tsv, tt, out, t_do, dq, l, d, w, 1)
+		k_kv.launch_d_kv(tq, tkv, tt, t_do, l, d, dkv, w, 1)
+		runs.append((dq.download(), d.download(), dkv.download()))
+	for a, b in zip(runs[0], runs[1]):
+		assert np.array_equal(a, b)
+	dq1, d1, dkv1 = _bf16_value(runs[0][0]), runs[0][1].astype(np.float64), _bf16_value(runs[0][2])
+	dq4, d4, dkv4 = _bf16_value(runs[2][0]), runs[2][1].astype(np.float64), _bf16_value(runs[2][2])
+	assert np.array_equal(dq4, 4.0 * dq1) and np.array_equal(d4, 4.0 * d1) and np.array_equal(dkv4, 4.0 * dkv1)
+	assert np.isfinite(dkv1).all() and np.abs(dkv1).max() > 1e-4 and np.abs(dq1).max() > 1e-4
+	assert not dq1[0].any() and not dkv1[t - 1].any()

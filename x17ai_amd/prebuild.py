@@ -77,6 +77,9 @@ def _specs():
 		add(("attn_d_kv", h, hd, True))
 	add(("attn_d_kv", 8, 64, False))
 	add(("attn_d_kv", 16, 128, False))                   # bench.py
+	add(("attn_d_q", 4, 128, False))
+	add(("attn_d_kv", 4, 128, False))
+	add(("attn", 4, 128, False))
 	for h, hd, cap in ((4, 32, 256), (4, 64, 256), (2, 128, 512), (2, 32, 4096), (2, 64, 4096)):
 		add(("decode", h, hd, cap, True))
 	for h, hd, cap, out in ((4, 64, 256, BF16), (2, 128, 512, BF16), (4, 32, 256, INT8)):
